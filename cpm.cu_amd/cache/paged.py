@@ -1,0 +1,251 @@
+"""The sequence cache: a slot per live sequence, pages of tokens per slot.
+
+What the model's mixers need is declared as ``CacheNeeds`` (per-token streams
+such as keys and values, fixed-size per-slot state, all tokens or a trailing
+window).  Cache entries with equal needs form a *group*; each group has page
+pool storage of its own and a page table of its own, so a group that keeps a
+window gives old pages back while a group that keeps everything does not.
+
+A slot is acquired when a sequence starts and released when it ends; its pages
+return to the pools and its fixed-size state is zeroed at the next acquire.
+Tokens are addressed as (slot, position); a stream's row for a token lies at
+``page_table[slot, position // page_size] * rows_per_page + (position % page_size) // every``.
+
+The reference engine holds one sequence in one contiguous buffer per layer
+(src/model/kvcache.cuh:7-65) plus compressed-key buffers beside it
+(src/model/minicpm4/minicpm4_kvcache.cuh:204-255); slots, pages and groups are
+this engine's own.  All bookkeeping is host-side Python over plain lists; the
+device sees the page tables and the pools.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+
+class CacheError(RuntimeError):
+    pass
+
+
+@dataclass(frozen=True)
+class StreamSpec:
+    """One row of ``width`` elements for every ``every`` tokens."""
+    width: int
+    every: int = 1
+    dtype: Optional[torch.dtype] = None       # None: the engine's element type
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """Fixed-size state per slot, zeroed when a slot is acquired."""
+    shape: Tuple[int, ...]
+    dtype: Optional[torch.dtype] = None
+
+
+@dataclass(frozen=True)
+class CacheNeeds:
+    """What one cache entry (a mixer's storage) asks for."""
+    streams: Tuple[Tuple[str, StreamSpec], ...] = ()
+    state: Tuple[Tuple[str, StateSpec], ...] = ()
+    window: Optional[int] = None              # None: keep every token; w: only the last w tokens are read
+
+    def group_key(self):
+        return (self.streams, self.state, self.window)
+
+
+@dataclass
+class CacheView:
+    """What a mixer sees of its cache entry."""
+    streams: Dict[str, torch.Tensor]          # name -> [n_pages, page_size // every, width]
+    state: Dict[str, torch.Tensor]            # name -> [max_slots, *shape]
+    page_table: Optional[torch.Tensor]        # int32 [max_slots, table_width] of the entry's group
+    page_size: int
+    window: Optional[int]
+
+
+class _Group:
+    def __init__(self, needs: CacheNeeds, entries: List[int], n_pages: int, max_slots: int, table_width: int,
+                 page_size: int, device, dtype):
+        self.needs = needs
+        self.entries = entries
+        self.n_pages = n_pages
+        self.page_size = page_size
+        self.free_pages: List[int] = list(range(n_pages - 1, -1, -1))   # pop() gives the lowest page first
+        # host page table: slot -> list of physical pages by page number (-1: given back / never held)
+        self.pages: List[List[int]] = [[] for _ in range(max_slots)]
+        self.table = torch.zeros((max_slots, table_width), dtype=torch.int32, device=device)
+        self.table_host = torch.zeros((max_slots, table_width), dtype=torch.int32)
+        self.dirty: set = set()
+        self.storage: Dict[int, Dict[str, torch.Tensor]] = {}
+        self.state: Dict[int, Dict[str, torch.Tensor]] = {}
+        for e in entries:
+            self.storage[e] = {}
+            for name, s in needs.streams:
+                if page_size % s.every:
+                    raise CacheError(f"cache stream '{name}' keeps a row every {s.every} tokens, which does not "
+                                     f"divide the page of {page_size} tokens")
+                self.storage[e][name] = torch.zeros((n_pages, page_size // s.every, s.width),
+                                                    dtype=s.dtype or dtype, device=device)
+            self.state[e] = {name: torch.zeros((max_slots,) + tuple(s.shape), dtype=s.dtype or dtype, device=device)
+                             for name, s in needs.state}
+
+    def held(self, slot: int) -> int:
+        return sum(1 for p in self.pages[slot] if p >= 0)
+
+
+class SequenceCache:
+    """Slots, pages and per-slot state for all cache entries of a model."""
+
+    def __init__(self, needs: List[CacheNeeds], max_tokens: int, max_slots: int, max_seq_len: int,
+                 page_size: int = 64, device="cpu", dtype=torch.float32):
+        if page_size <= 0 or max_tokens <= 0 or max_slots <= 0 or max_seq_len <= 0:
+            raise CacheError("cache sizes must be positive")
+        self.page_size = page_size
+        self.max_slots = max_slots
+        self.max_seq_len = max_seq_len
+        self.device = torch.device(device)
+        self.dtype = dtype
+        self.n_pages = -(-max_tokens // page_size)
+        self.table_width = min(-(-max_seq_len // page_size), self.n_pages)
+        self.groups: List[_Group] = []
+        self.entry_group: List[int] = []
+        by_key: Dict[object, List[int]] = {}
+        for e, n in enumerate(needs):
+            by_key.setdefault(n.group_key(), []).append(e)
+        self.entry_group = [0] * len(needs)
+        for key, entries in by_key.items():
+            g = _Group(needs[entries[0]], entries, self.n_pages, max_slots, self.table_width, page_size,
+                       self.device, dtype)
+            for e in entries:
+                self.entry_group[e] = len(self.groups)
+            self.groups.append(g)
+        self.free_slots: List[int] = list(range(max_slots - 1, -1, -1))
+        self.live: Dict[int, int] = {}        # slot -> tokens held
+        self._views: Dict[int, CacheView] = {}
+
+    # ---- slots ----
+    def acquire(self) -> int:
+        if not self.free_slots:
+            raise CacheError(f"no free slot: all {self.max_slots} are held by live sequences")
+        slot = self.free_slots.pop()
+        self.live[slot] = 0
+        for g in self.groups:
+            for e in g.entries:
+                for t in g.state[e].values():
+                    t[slot].zero_()
+        return slot
+
+    def release(self, slot: int):
+        if slot not in self.live:
+            raise CacheError(f"slot {slot} is not held (released twice, or never acquired)")
+        for g in self.groups:
+            for p in g.pages[slot]:
+                if p >= 0:
+                    g.free_pages.append(p)
+            g.pages[slot] = []
+        del self.live[slot]
+        self.free_slots.append(slot)
+
+    def length(self, slot: int) -> int:
+        try:
+            return self.live[slot]
+        except KeyError:
+            raise CacheError(f"slot {slot} is not held by a live sequence") from None
+
+    # ---- tokens ----
+    def pages_needed(self, slot: int, new_len: int) -> int:
+        """Pages a full-history group must still take for the slot to hold new_len tokens."""
+        have = -(-self.length(slot) // self.page_size)
+        return max(-(-new_len // self.page_size) - have, 0)
+
+    def free_page_count(self) -> int:
+        return min(len(g.free_pages) for g in self.groups) if self.groups else self.n_pages
+
+    def extend(self, slot: int, n_new: int) -> int:
+        """Make room for n_new more tokens of the slot; returns the position of the first of them."""
+        old = self.length(slot)
+        new = old + n_new
+        if n_new <= 0:
+            raise CacheError(f"slot {slot}: a step must bring at least one token")
+        if new > self.max_seq_len:
+            raise CacheError(f"slot {slot}: {new} tokens exceed the longest sequence this engine holds "
+                             f"({self.max_seq_len})")
+        n_pg = -(-new // self.page_size)
+        # check every group before touching any, so a refused step changes nothing
+        for g in self.groups:
+            first_kept = 0 if g.needs.window is None else max(old - g.needs.window + 1, 0) // self.page_size
+            need = sum(1 for pn in range(first_kept, n_pg) if pn >= len(g.pages[slot]) or g.pages[slot][pn] < 0)
+            freed = 0 if g.needs.window is None else sum(1 for p in g.pages[slot][:first_kept] if p >= 0)
+            if need > len(g.free_pages) + freed:
+                raise CacheError(f"the cache is full: slot {slot} needs {need} more pages of {self.page_size} tokens, "
+                                 f"{len(g.free_pages) + freed} are free of {g.n_pages}")
+        for g in self.groups:
+            pages = g.pages[slot]
+            if g.needs.window is not None:
+                # the step's first query (position `old`) still reads back to old - window + 1
+                first_kept = max(old - g.needs.window + 1, 0) // self.page_size
+                for pn in range(min(first_kept, len(pages))):
+                    if pages[pn] >= 0:
+                        g.free_pages.append(pages[pn])
+                        pages[pn] = -1
+            else:
+                first_kept = 0
+            changed = False
+            while len(pages) < n_pg:
+                pn = len(pages)
+                pages.append(g.free_pages.pop() if pn >= first_kept else -1)
+                changed = True
+            if changed or g.needs.window is not None:
+                row = g.table_host[slot]
+                for pn, p in enumerate(pages):
+                    row[pn] = max(p, 0)
+                g.dirty.add(slot)
+        self.live[slot] = new
+        return old
+
+    def sync(self):
+        """Copy the page-table rows that changed to the device (before kernels read them)."""
+        for g in self.groups:
+            if not g.dirty:
+                continue
+            if self.device.type == "cpu":
+                g.table.copy_(g.table_host)
+            else:
+                rows = sorted(g.dirty)
+                idx = torch.tensor(rows, dtype=torch.long)
+                g.table.index_copy_(0, idx.to(self.device), g.table_host[idx].to(self.device))
+            g.dirty.clear()
+
+    # ---- views ----
+    def view(self, entry: int) -> CacheView:
+        v = self._views.get(entry)
+        if v is None:
+            g = self.groups[self.entry_group[entry]]
+            v = CacheView(g.storage[entry], g.state[entry], g.table, self.page_size, g.needs.window)
+            self._views[entry] = v
+        return v
+
+    # ---- accounting (tests and reports) ----
+    def check(self):
+        """Every page is free or held exactly once; every slot is free or live exactly once."""
+        for gi, g in enumerate(self.groups):
+            held = [p for pages in g.pages for p in pages if p >= 0]
+            allp = held + g.free_pages
+            if len(allp) != g.n_pages or len(set(allp)) != g.n_pages:
+                raise CacheError(f"group {gi}: pages lost or held twice ({len(held)} held, {len(g.free_pages)} free, "
+                                 f"{g.n_pages} in all)")
+        slots = list(self.live) + self.free_slots
+        if len(slots) != self.max_slots or len(set(slots)) != self.max_slots:
+            raise CacheError("slots lost or held twice")
+        for s in range(self.max_slots):
+            if s not in self.live and any(g.pages[s] for g in self.groups):
+                raise CacheError(f"free slot {s} still holds pages")
+
+    def bytes(self) -> int:
+        n = 0
+        for g in self.groups:
+            for d in list(g.storage.values()) + list(g.state.values()):
+                n += sum(t.numel() * t.element_size() for t in d.values())
+        return n

@@ -1,0 +1,206 @@
+// Row-wise kernels around the matrix products: token embedding, residual add
+// fused with RMSNorm, SiLU gating, rotary position encoding fused with the
+// write of keys and values into the paged cache.
+//
+// The residual stream is always float; `T` is the activation/weight element
+// type of the engine (float in the 32-bit engine, bf16 in the serving one).
+// All statistics (sum of squares, rsqrt, angles, sin/cos, sigmoid) are float.
+#include "common.h"
+
+// ---------------------------------------------------------------------------
+// embedding:  out[r,:] = float(table[ids[r],:]) * scale
+// (reference: src/model/embedding.cuh:7-20 gathers, elementwise.cuh:34-41 scales)
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids, float* __restrict__ out,
+                             int H, float scale) {
+    const long r = blockIdx.x;
+    const T* src = table + (long)ids[r] * H;
+    float* dst = out + r * H;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) dst[c] = to_f32(src[c]) * scale;
+}
+
+extern "C" const char* cpmcu_embed(const void* table, int dtype, const int* ids, float* out, int n, int H, int V,
+                                   float scale, hipStream_t stream) {
+    CPMCU_REQUIRE(n > 0 && H > 0 && V > 0, "embed: empty shape n=%d H=%d V=%d", n, H, V);
+    CPMCU_REQUIRE(dtype == CPMCU_F32 || dtype == CPMCU_BF16, "embed: unknown dtype %d", dtype);
+    const int block = H >= 1024 ? 256 : 64;
+    if (dtype == CPMCU_F32)
+        embed_kernel<float><<<n, block, 0, stream>>>((const float*)table, ids, out, H, scale);
+    else
+        embed_kernel<bf16_t><<<n, block, 0, stream>>>((const bf16_t*)table, ids, out, H, scale);
+    CPMCU_LAUNCH_CHECK("embed");
+    return nullptr;
+}
+
+// ---------------------------------------------------------------------------
+// x += bscale * sum_p branch[p]   (written back unless `rows` selects rows)
+// out = x * rsqrt(mean(x^2) + eps) * w
+// (reference: src/model/norm.cuh:53-99; eps inside the root, weight after)
+// `branch` may be null (plain norm), and may come as `nparts` partial sums of
+// a split matrix product, `part_stride` elements apart.
+// ---------------------------------------------------------------------------
+template <typename BT, typename OT>
+__global__ void add_rms_norm_kernel(float* __restrict__ x, const BT* __restrict__ branch, int nparts,
+                                    long part_stride, float bscale, const float* __restrict__ w, float eps,
+                                    OT* __restrict__ out, const int* __restrict__ rows, int H) {
+    __shared__ float red[17];
+    const long r_out = blockIdx.x;
+    const long r = rows ? rows[r_out] : r_out;
+    float* xr = x + r * H;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        float v = xr[c];
+        if (branch) {
+            float b = 0.f;
+            for (int p = 0; p < nparts; ++p) b += to_f32(branch[p * part_stride + r * H + c]);
+            v += bscale * b;
+            if (!rows) xr[c] = v;
+        }
+        ss += v * v;
+    }
+    ss = block_sum(ss, red);
+    const float rs = 1.0f / sqrtf(ss / (float)H + eps);
+    OT* o = out + r_out * H;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        float v = xr[c];
+        if (branch && rows) {
+            float b = 0.f;
+            for (int p = 0; p < nparts; ++p) b += to_f32(branch[p * part_stride + r * H + c]);
+            v += bscale * b;
+        }
+        o[c] = from_f32<OT>(v * rs * w[c]);
+    }
+}
+
+extern "C" const char* cpmcu_add_rms_norm(float* x, const void* branch, int branch_dtype, int nparts,
+                                          long part_stride, float bscale, const float* w, float eps, void* out,
+                                          int out_dtype, const int* rows, int n_out, int H, hipStream_t stream) {
+    CPMCU_REQUIRE(n_out > 0 && H > 0, "add_rms_norm: empty shape rows=%d H=%d", n_out, H);
+    CPMCU_REQUIRE(!branch || nparts >= 1, "add_rms_norm: nparts=%d", nparts);
+    const int block = H >= 2048 ? 512 : (H >= 512 ? 256 : 64);
+#define LAUNCH(BT, OT)                                                                                         \
+    add_rms_norm_kernel<BT, OT><<<n_out, block, 0, stream>>>(x, (const BT*)branch, nparts, part_stride, bscale, \
+                                                             w, eps, (OT*)out, rows, H)
+    if (branch_dtype == CPMCU_F32 && out_dtype == CPMCU_F32) LAUNCH(float, float);
+    else if (branch_dtype == CPMCU_F32 && out_dtype == CPMCU_BF16) LAUNCH(float, bf16_t);
+    else if (branch_dtype == CPMCU_BF16 && out_dtype == CPMCU_F32) LAUNCH(bf16_t, float);
+    else if (branch_dtype == CPMCU_BF16 && out_dtype == CPMCU_BF16) LAUNCH(bf16_t, bf16_t);
+    else CPMCU_FAIL("add_rms_norm: unknown dtypes %d %d", branch_dtype, out_dtype);
+#undef LAUNCH
+    CPMCU_LAUNCH_CHECK("add_rms_norm");
+    return nullptr;
+}
+
+// ---------------------------------------------------------------------------
+// out[r,c] = silu(gu[r,c]) * gu[r,c+I],  silu(g) = g / (1 + exp(-g))
+// (reference: src/model/activation.cuh:6-18, gate columns first, then up)
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, long n, int I) {
+    const long total = n * I;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+        const long r = i / I;
+        const int c = (int)(i - r * I);
+        const float g = to_f32(gu[r * 2 * I + c]);
+        const float u = to_f32(gu[r * 2 * I + I + c]);
+        out[i] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+    }
+}
+
+extern "C" const char* cpmcu_silu_mul(const void* gu, void* out, int dtype, int n, int I, hipStream_t stream) {
+    CPMCU_REQUIRE(n > 0 && I > 0, "silu_mul: empty shape n=%d I=%d", n, I);
+    const long total = (long)n * I;
+    const int block = 256;
+    const int grid = (int)((total + block - 1) / block < 65535 * 16 ? (total + block - 1) / block : 65535 * 16);
+    if (dtype == CPMCU_F32)
+        silu_mul_kernel<float><<<grid, block, 0, stream>>>((const float*)gu, (float*)out, n, I);
+    else if (dtype == CPMCU_BF16)
+        silu_mul_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, n, I);
+    else
+        CPMCU_FAIL("silu_mul: unknown dtype %d", dtype);
+    CPMCU_LAUNCH_CHECK("silu_mul");
+    return nullptr;
+}
+
+// ---------------------------------------------------------------------------
+// Rotary position encoding (rotate-half) on q and k, then k and v into the
+// paged cache.  A row of `qkv` (`row_width` elements) is [q: nh*hd | k: nkv*hd | v: nkv*hd]; it may
+// come as `nparts` float partial sums of a split matrix product.  q is written
+// to `q_out` (row stride nh*hd).  theta = pos * inv_freq[c];
+// (a, b) = (x[c], x[c+hd/2]) -> (a cos - b sin, a sin + b cos), cos and sin
+// times `mscale` (reference: src/model/rotary.cuh:7-34; cache rows
+// src/model/attn.cuh:14-21).  inv_freq null: no rotation.
+// ---------------------------------------------------------------------------
+template <typename IT, typename T>
+__global__ void rope_store_kernel(const IT* __restrict__ qkv, long width, int nparts, long part_stride,
+                                  T* __restrict__ q_out, int nh, int nkv, int hd, const int* __restrict__ positions,
+                                  const int* __restrict__ tok_slot, const float* __restrict__ inv_freq, float mscale,
+                                  T* __restrict__ kpool, T* __restrict__ vpool, PagedView pv, int write_kv) {
+    const long t = blockIdx.x;
+    const int half = hd / 2;
+    const int pos = positions[t];
+    const IT* row = qkv + t * width;
+    auto load = [&](long i) {
+        float s = 0.f;
+        for (int p = 0; p < nparts; ++p) s += to_f32(row[p * part_stride + i]);
+        return s;
+    };
+    long kv_row = 0;
+    if (write_kv) kv_row = paged_row(pv, tok_slot[t], pos);
+    const int n_rot = (nh + (write_kv ? nkv : 0)) * half;
+    for (int i = threadIdx.x; i < n_rot; i += blockDim.x) {
+        const int head = i / half, c = i - head * half;
+        float cs = 1.f, sn = 0.f;
+        if (inv_freq) {
+            const float ang = (float)pos * inv_freq[c];
+            cs = cosf(ang) * mscale;
+            sn = sinf(ang) * mscale;
+        }
+        const long off = (long)head * hd + c;
+        const float a = load(off), b = load(off + half);
+        const float ra = a * cs - b * sn, rb = a * sn + b * cs;
+        if (head < nh) {
+            T* dst = q_out + t * (long)nh * hd + off;
+            dst[0] = from_f32<T>(ra);
+            dst[half] = from_f32<T>(rb);
+        } else {
+            T* dst = kpool + kv_row * (long)nkv * hd + (off - (long)nh * hd);
+            dst[0] = from_f32<T>(ra);
+            dst[half] = from_f32<T>(rb);
+        }
+    }
+    if (write_kv) {
+        const long voff = (long)(nh + nkv) * hd;
+        T* dst = vpool + kv_row * (long)nkv * hd;
+        for (int i = threadIdx.x; i < nkv * hd; i += blockDim.x) dst[i] = from_f32<T>(load(voff + i));
+    }
+}
+
+extern "C" const char* cpmcu_rope_store(const void* qkv, long row_width, int in_dtype, int nparts, long part_stride, void* q_out,
+                                        int dtype, int n, int nh, int nkv, int hd, const int* positions,
+                                        const int* tok_slot, const float* inv_freq, float mscale, void* kpool,
+                                        void* vpool, const int* page_table, int table_width, int page_size,
+                                        int write_kv, hipStream_t stream) {
+    CPMCU_REQUIRE(n > 0 && nh > 0 && nkv >= 0 && hd > 0 && hd % 2 == 0,
+                  "rope_store: bad shape n=%d heads=%d kv_heads=%d head_dim=%d (head_dim must be even)", n, nh, nkv, hd);
+    CPMCU_REQUIRE(!write_kv || (kpool && vpool && page_table && table_width > 0 && page_size > 0),
+                  "rope_store: cache pointers missing");
+    CPMCU_REQUIRE(nparts >= 1, "rope_store: nparts=%d", nparts);
+    CPMCU_REQUIRE(row_width >= (long)(nh + (write_kv ? 2 * nkv : 0)) * hd,
+                  "rope_store: a row of %ld elements cannot hold %d query%s heads of %d", row_width, nh,
+                  write_kv ? " and key/value" : "", hd);
+    PagedView pv{page_table, table_width, page_size};
+    const int block = 256;
+#define LAUNCH(IT, T)                                                                                          \
+    rope_store_kernel<IT, T><<<n, block, 0, stream>>>((const IT*)qkv, row_width, nparts, part_stride, (T*)q_out, nh, nkv, \
+                                                      hd, positions, tok_slot, inv_freq, mscale, (T*)kpool,   \
+                                                      (T*)vpool, pv, write_kv)
+    if (in_dtype == CPMCU_F32 && dtype == CPMCU_F32) LAUNCH(float, float);
+    else if (in_dtype == CPMCU_F32 && dtype == CPMCU_BF16) LAUNCH(float, bf16_t);
+    else if (in_dtype == CPMCU_BF16 && dtype == CPMCU_BF16) LAUNCH(bf16_t, bf16_t);
+    else CPMCU_FAIL("rope_store: unsupported dtypes in=%d out=%d", in_dtype, dtype);
+#undef LAUNCH
+    CPMCU_LAUNCH_CHECK("rope_store");
+    return nullptr;
+}

@@ -1,0 +1,122 @@
+// Next-token choice from float logits: argmax, and a draw from
+// softmax(logits / temperature).
+//
+// The reference samples with library calls on one row: argmax, or
+// multinomial(softmax(logits/temperature)) (cpmcu/llm.py:282-285).  Here a
+// row's random number comes from a counter-based generator keyed by
+// (seed, request id, step), so what a request draws does not depend on which
+// other requests share its batch.
+#include "common.h"
+
+// ties go to the lowest index
+__global__ void argmax_kernel(const float* __restrict__ logits, long ld, int V, int* __restrict__ out) {
+    __shared__ float bv[16];
+    __shared__ int bi[16];
+    const float* row = logits + (long)blockIdx.x * ld;
+    float best = -INFINITY;
+    int idx = 0x7fffffff;
+    for (int i = threadIdx.x; i < V; i += blockDim.x) {
+        const float v = row[i];
+        if (v > best || (v == best && i < idx)) { best = v; idx = i; }
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o, 64);
+        const int oi = __shfl_xor(idx, o, 64);
+        if (ov > best || (ov == best && oi < idx)) { best = ov; idx = oi; }
+    }
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    if (lane == 0) { bv[w] = best; bi[w] = idx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int i = 1; i < nw; ++i)
+            if (bv[i] > best || (bv[i] == best && bi[i] < idx)) { best = bv[i]; idx = bi[i]; }
+        out[blockIdx.x] = idx == 0x7fffffff ? 0 : idx;
+    }
+}
+
+extern "C" const char* cpmcu_argmax(const float* logits, long ld, int rows, int V, int* out, hipStream_t stream) {
+    CPMCU_REQUIRE(rows > 0 && V > 0 && ld >= V, "argmax: bad shape rows=%d V=%d ld=%ld", rows, V, ld);
+    argmax_kernel<<<rows, V >= 4096 ? 1024 : 256, 0, stream>>>(logits, ld, V, out);
+    CPMCU_LAUNCH_CHECK("argmax");
+    return nullptr;
+}
+
+// Philox-4x32-10: counter (c0..c3), key (k0,k1) -> 4 random words
+__device__ inline void philox4x32(uint32_t c[4], uint32_t k0, uint32_t k1) {
+#pragma unroll
+    for (int r = 0; r < 10; ++r) {
+        const uint64_t p0 = (uint64_t)0xD2511F53u * c[0];
+        const uint64_t p1 = (uint64_t)0xCD9E8D57u * c[2];
+        const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c[1] ^ k0;
+        const uint32_t n1 = (uint32_t)p1;
+        const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c[3] ^ k1;
+        const uint32_t n3 = (uint32_t)p0;
+        c[0] = n0; c[1] = n1; c[2] = n2; c[3] = n3;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+}
+
+// One block per row.  Thread i owns the contiguous vocabulary segment
+// [i*seg, (i+1)*seg); the thread whose range of the cumulative sum holds
+// u * total walks its segment.
+__global__ __launch_bounds__(256) void sample_kernel(const float* __restrict__ logits, long ld, int V,
+                                                    float inv_temperature, uint32_t seed_lo, uint32_t seed_hi,
+                                                    const int* __restrict__ request_ids, const int* __restrict__ steps,
+                                                    int* __restrict__ out, float* __restrict__ u_out) {
+    __shared__ float red[17];
+    __shared__ float seg_sum[256];
+    __shared__ float seg_pre[257];
+    __shared__ int owner;
+    const int r = blockIdx.x, tid = threadIdx.x;
+    const float* row = logits + (long)r * ld;
+    float mx = -INFINITY;
+    for (int i = tid; i < V; i += blockDim.x) mx = fmaxf(mx, row[i]);
+    mx = block_max(mx, red);
+    const int seg = (V + blockDim.x - 1) / blockDim.x;
+    const int i0 = min(tid * seg, V), i1 = min(i0 + seg, V);
+    float s = 0.f;
+    for (int i = i0; i < i1; ++i) s += expf((row[i] - mx) * inv_temperature);
+    seg_sum[tid] = s;
+    __syncthreads();
+    uint32_t ctr[4] = {(uint32_t)request_ids[r], (uint32_t)steps[r], 0u, 0u};
+    philox4x32(ctr, seed_lo, seed_hi);
+    const float u = (float)(ctr[0] >> 8) * (1.0f / 16777216.0f);   // [0, 1)
+    if (tid == 0) {
+        float c = 0.f;
+        for (int i = 0; i < (int)blockDim.x; ++i) { seg_pre[i] = c; c += seg_sum[i]; }
+        seg_pre[blockDim.x] = c;
+        // the owner: the last thread with a non-empty segment that starts at or before the target
+        const float tg = u * c;
+        int o = 0;
+        for (int i = 0; i < (int)blockDim.x; ++i)
+            if (seg_sum[i] > 0.f && seg_pre[i] <= tg) o = i;
+        owner = o;
+        if (u_out) u_out[r] = u;
+    }
+    __syncthreads();
+    const float target = u * seg_pre[blockDim.x];
+    const bool mine = tid == owner;
+    if (mine) {
+        float c = seg_pre[tid];
+        int pick = -1, last = i0;
+        for (int i = i0; i < i1; ++i) {
+            const float e = expf((row[i] - mx) * inv_temperature);
+            if (e > 0.f) last = i;
+            c += e;
+            if (c > target) { pick = i; break; }
+        }
+        out[r] = pick >= 0 ? pick : last;
+    }
+}
+
+extern "C" const char* cpmcu_sample(const float* logits, long ld, int rows, int V, float temperature,
+                                    unsigned long long seed, const int* request_ids, const int* steps, int* out,
+                                    float* u_out, hipStream_t stream) {
+    CPMCU_REQUIRE(rows > 0 && V > 0 && ld >= V, "sample: bad shape rows=%d V=%d ld=%ld", rows, V, ld);
+    CPMCU_REQUIRE(temperature > 0.f, "sample: temperature %g must be positive (0 is greedy: use argmax)", temperature);
+    sample_kernel<<<rows, 256, 0, stream>>>(logits, ld, V, 1.0f / temperature, (uint32_t)seed,
+                                            (uint32_t)(seed >> 32), request_ids, steps, out, u_out);
+    CPMCU_LAUNCH_CHECK("sample");
+    return nullptr;
+}

@@ -1,0 +1,204 @@
+// InfLLM-v2 block selection: compressed keys, their scores, block pooling and
+// top-k, as a function of a query's prefix only (so that the chosen blocks do
+// not depend on how tokens were cut into steps).
+//
+// Stages (reference: src/model/minicpm4/minicpm4_attn.cuh:107-202 runs them per
+// call; kernels src/model/minicpm4/minicpm4_kvcache.cuh:6-142, src/model/topk.cuh):
+//   ck[j]    = mean(K[st*j : st*j+ks])                      (compress_keys)
+//   score[j] = sum_{h in group} softmax_j(q_h.ck[j]*scale)  over ck with st*j+ks <= p
+//   pool[b]  = max score[j] over ck overlapping block b; +inf for b < init_blocks
+//   chosen   = the min(topk, #candidates) candidates b <= p/bs - lb of largest
+//              pool, ties to the lower index
+//   list     = chosen U window (p/bs - lb < b <= p/bs), ascending
+// The attention kernels then visit exactly the listed blocks.
+#include "common.h"
+
+// ---------------------------------------------------------------------------
+// One block per token of the step.  The token at position p completes the
+// compressed key j = (p+1-ks)/st when (p+1-ks) is a non-negative multiple of
+// st.  The compressed keys live in a paged stream with page_size/st rows a page.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void compress_keys_kernel(const T* __restrict__ kpool, T* __restrict__ ckpool, PagedView pv,
+                                     const int* __restrict__ positions, const int* __restrict__ tok_slot, int width,
+                                     int ks, int st) {
+    const int t = blockIdx.x;
+    const int p = positions[t];
+    if (p + 1 < ks || (p + 1 - ks) % st != 0) return;
+    const int j = (p + 1 - ks) / st;
+    const int slot = tok_slot[t];
+    const int first = st * j;
+    const int page = pv.page_table[(long)slot * pv.table_width + first / pv.page_size];
+    const long ck_row = (long)page * (pv.page_size / st) + (first % pv.page_size) / st;
+    for (int e = threadIdx.x; e < width; e += blockDim.x) {
+        float s = 0.f;
+        for (int r = 0; r < ks; ++r) s += to_f32(kpool[paged_row(pv, slot, first + r) * width + e]);
+        ckpool[ck_row * width + e] = from_f32<T>(s / (float)ks);
+    }
+}
+
+extern "C" const char* cpmcu_compress_keys(const void* kpool, void* ckpool, int dtype, int n, int width,
+                                           const int* page_table, int table_width, int page_size,
+                                           const int* positions, const int* tok_slot, int ks, int st,
+                                           hipStream_t stream) {
+    CPMCU_REQUIRE(n > 0 && width > 0, "compress_keys: empty shape");
+    CPMCU_REQUIRE(st > 0 && ks >= st && page_size % st == 0,
+                  "compress_keys: kernel_stride %d must divide the cache page of %d tokens (kernel_size %d)", st,
+                  page_size, ks);
+    PagedView pv{page_table, table_width, page_size};
+    if (dtype == CPMCU_F32)
+        compress_keys_kernel<float><<<n, 128, 0, stream>>>((const float*)kpool, (float*)ckpool, pv, positions,
+                                                           tok_slot, width, ks, st);
+    else if (dtype == CPMCU_BF16)
+        compress_keys_kernel<bf16_t><<<n, 128, 0, stream>>>((const bf16_t*)kpool, (bf16_t*)ckpool, pv, positions,
+                                                            tok_slot, width, ks, st);
+    else
+        CPMCU_FAIL("compress_keys: unknown dtype %d", dtype);
+    CPMCU_LAUNCH_CHECK("compress_keys");
+    return nullptr;
+}
+
+// ---------------------------------------------------------------------------
+// One block per (token, kv head).  LDS: tmp[max_ck] score[max_ck] pool[max_blocks]
+// flag[max_blocks] q[hd].
+// ---------------------------------------------------------------------------
+struct SelectParams {
+    int nh, nkv, hd;
+    float scale;
+    int ks, st, bs, init_blocks, topk, window_blocks, dense_len;
+    int max_ck, max_blocks, max_sel;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void sparse_select_kernel(const T* __restrict__ q, const T* __restrict__ ckpool,
+                                                           PagedView pv, const int* __restrict__ positions,
+                                                           const int* __restrict__ tok_slot, SelectParams sp,
+                                                           int* __restrict__ sel_blocks, int* __restrict__ sel_count) {
+    extern __shared__ float lds[];
+    __shared__ float red[17];
+    float* tmp = lds;
+    float* score = tmp + sp.max_ck;
+    float* pool = score + sp.max_ck;
+    int* flag = (int*)(pool + sp.max_blocks);
+    float* qs = (float*)(flag + sp.max_blocks);
+
+    const int t = blockIdx.x, g = blockIdx.y, tid = threadIdx.x;
+    const int p = positions[t];
+    const long out_idx = (long)t * sp.nkv + g;
+    if (p + 1 <= sp.dense_len) {
+        if (tid == 0) sel_count[out_idx] = -1;
+        return;
+    }
+    const int slot = tok_slot[t];
+    const int G = sp.nh / sp.nkv;
+    const int n_vis = p < sp.ks ? 0 : (p - sp.ks) / sp.st + 1;
+    const int q_block = p / sp.bs;
+    const int n_cand = max(q_block - sp.window_blocks + 1, 0);
+    const int rows_per_page = pv.page_size / sp.st;
+    const long width = (long)sp.nkv * sp.hd;
+
+    for (int j = tid; j < n_vis; j += blockDim.x) score[j] = 0.f;
+    for (int hh = 0; hh < G; ++hh) {
+        __syncthreads();
+        const T* qrow = q + ((long)t * sp.nh + (long)g * G + hh) * sp.hd;
+        for (int d = tid; d < sp.hd; d += blockDim.x) qs[d] = to_f32(qrow[d]);
+        __syncthreads();
+        float mx = -INFINITY;
+        for (int j = tid; j < n_vis; j += blockDim.x) {
+            const int first = sp.st * j;
+            const int page = pv.page_table[(long)slot * pv.table_width + first / pv.page_size];
+            const T* ck = ckpool + ((long)page * rows_per_page + (first % pv.page_size) / sp.st) * width + (long)g * sp.hd;
+            float dot = 0.f;
+            for (int d = 0; d < sp.hd; ++d) dot += qs[d] * to_f32(ck[d]);
+            const float s = dot * sp.scale;
+            tmp[j] = s;
+            mx = fmaxf(mx, s);
+        }
+        mx = block_max(mx, red);
+        float sum = 0.f;
+        for (int j = tid; j < n_vis; j += blockDim.x) {
+            const float e = expf(tmp[j] - mx);
+            tmp[j] = e;
+            sum += e;
+        }
+        sum = block_sum(sum, red);
+        for (int j = tid; j < n_vis; j += blockDim.x) score[j] += tmp[j] / sum;
+    }
+    __syncthreads();
+    // pool the scores of the compressed keys that overlap each candidate block
+    for (int b = tid; b < n_cand; b += blockDim.x) {
+        float v = -INFINITY;
+        if (b < sp.init_blocks) {
+            v = INFINITY;
+        } else {
+            const int lo_tok = sp.bs * b - sp.ks + 1;                 // st*j >= lo_tok
+            const int j_lo = lo_tok <= 0 ? 0 : (lo_tok + sp.st - 1) / sp.st;
+            const int j_hi = min((sp.bs * (b + 1) - 1) / sp.st, n_vis - 1);
+            for (int j = j_lo; j <= j_hi; ++j) v = fmaxf(v, score[j]);
+        }
+        pool[b] = v;
+    }
+    __syncthreads();
+    // rank by (larger pool, lower index); the first `topk` ranks are chosen
+    for (int b = tid; b <= q_block; b += blockDim.x) {
+        int f = 0;
+        if (b < n_cand) {
+            const float v = pool[b];
+            int rank = 0;
+            for (int o = 0; o < n_cand; ++o) {
+                const float w = pool[o];
+                rank += (w > v || (w == v && o < b)) ? 1 : 0;
+            }
+            f = rank < sp.topk;
+        } else {
+            f = 1;   // sliding window, the query's own block included
+        }
+        flag[b] = f;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int* dst = sel_blocks + out_idx * sp.max_sel;
+        int c = 0;
+        for (int b = 0; b <= q_block; ++b)
+            if (flag[b] && c < sp.max_sel) dst[c++] = b;
+        sel_count[out_idx] = c;
+    }
+}
+
+extern "C" const char* cpmcu_sparse_select(const void* q, const void* ckpool, int dtype, int n, int nh, int nkv,
+                                           int hd, float scale, const int* page_table, int table_width,
+                                           int page_size, const int* positions, const int* tok_slot, int ks, int st,
+                                           int bs, int init_blocks, int topk, int window_blocks, int dense_len,
+                                           int max_pos, int* sel_blocks, int* sel_count, int max_sel,
+                                           hipStream_t stream) {
+    CPMCU_REQUIRE(n > 0 && nh > 0 && nkv > 0 && hd > 0 && nh % nkv == 0, "sparse_select: bad shape");
+    CPMCU_REQUIRE(st > 0 && ks >= st && bs % st == 0 && page_size % st == 0,
+                  "sparse_select: kernel_stride %d must divide block_size %d and the cache page of %d tokens", st, bs,
+                  page_size);
+    CPMCU_REQUIRE(window_blocks >= 1 && max_sel >= topk + window_blocks,
+                  "sparse_select: block list of %d entries cannot hold topk %d + window %d", max_sel, topk,
+                  window_blocks);
+    SelectParams sp;
+    sp.nh = nh; sp.nkv = nkv; sp.hd = hd; sp.scale = scale;
+    sp.ks = ks; sp.st = st; sp.bs = bs; sp.init_blocks = init_blocks; sp.topk = topk;
+    sp.window_blocks = window_blocks; sp.dense_len = dense_len;
+    sp.max_ck = max_pos < ks ? 1 : (max_pos - ks) / st + 1;
+    sp.max_blocks = max_pos / bs + 1;
+    sp.max_sel = max_sel;
+    const size_t lds = sizeof(float) * ((size_t)2 * sp.max_ck + 2 * sp.max_blocks + hd);
+    CPMCU_REQUIRE(lds <= 60 * 1024,
+                  "sparse_select: a context of %d tokens needs %zu bytes of LDS for its block scores (limit 61440)",
+                  max_pos + 1, lds);
+    dim3 grid(n, nkv);
+    PagedView pv{page_table, table_width, page_size};
+    if (dtype == CPMCU_F32)
+        sparse_select_kernel<float><<<grid, 256, lds, stream>>>((const float*)q, (const float*)ckpool, pv, positions,
+                                                                tok_slot, sp, sel_blocks, sel_count);
+    else if (dtype == CPMCU_BF16)
+        sparse_select_kernel<bf16_t><<<grid, 256, lds, stream>>>((const bf16_t*)q, (const bf16_t*)ckpool, pv,
+                                                                 positions, tok_slot, sp, sel_blocks, sel_count);
+    else
+        CPMCU_FAIL("sparse_select: unknown dtype %d", dtype);
+    CPMCU_LAUNCH_CHECK("sparse_select");
+    return nullptr;
+}

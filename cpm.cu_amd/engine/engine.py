@@ -1,0 +1,244 @@
+"""The engine: a model bound to a GPU, its cache, and the one step function.
+
+``step`` takes a batch of sequences, each with the next tokens it brings
+(a whole prompt, a chunk of one, or a single token) and the places among them
+whose logits are wanted.  It runs only those tokens, as one packed batch without
+padding, against what earlier steps left in the cache, and returns float32
+logits.  The reference has two entry points for one sequence, ``prefill(n,
+history, ...)`` and ``decode(...)`` (src/entry.cu:558-584,
+src/model/minicpm4/minicpm4_model.cuh:125-153); batches, slots and the single
+step function are this engine's own.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from ..cache.paged import CacheError, SequenceCache
+from ..config.base import ModelConfig, architecture_name, read_config_json
+from ..parts.base import Runtime, StepContext, Workspace
+from ..registry import get_architecture
+from ..weights.loader import checkpoint_names, load_tensors
+
+_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "fp32": torch.float32, "bf16": torch.bfloat16}
+
+
+class StepError(ValueError):
+    """A step was refused; nothing was run and the cache is unchanged."""
+
+
+@dataclass
+class EngineOptions:
+    dtype: str = "bfloat16"                 # 'bfloat16' (serving kernels) or 'float32' (everything in true 32-bit)
+    max_tokens: int = 8192                  # tokens all live sequences hold together (each rounded up to a page)
+    max_seq_len: Optional[int] = None       # longest sequence; default: the model's max_position_embeddings
+    max_slots: Optional[int] = None         # live sequences; default: one per page, at most 1024
+    max_step_tokens: int = 2048             # tokens one forward pass carries (the reference's chunk_length)
+    page_size: int = 64
+    device: str = "cuda:0"
+    hip_graph: bool = False                 # replay single-token steps from a captured graph
+    sparse: bool = True                     # honour sparse_config (False: dense attention everywhere)
+
+
+@dataclass
+class StepEntry:
+    slot: int
+    tokens: Sequence[int]
+    want: Sequence[int] = ()                # indices into ``tokens`` whose logits are returned
+
+
+class Engine:
+    def __init__(self, config: ModelConfig, model, tensors: Dict[str, torch.Tensor], options: EngineOptions):
+        if options.dtype not in _DTYPES:
+            raise ValueError(f"dtype '{options.dtype}' is not supported (float32, bfloat16)")
+        self.options = options
+        self.config = config
+        self.model = model
+        self.device = torch.device(options.device)
+        if self.device.type != "cuda":
+            raise RuntimeError("the engine runs on a GPU only (device 'cuda:N'); there is no CPU path")
+        if not torch.cuda.is_available():
+            raise RuntimeError("no GPU is visible: the engine's kernels cannot run")
+        self.dtype = _DTYPES[options.dtype]
+        max_seq_len = options.max_seq_len or getattr(config, "max_position_embeddings", None) or options.max_tokens
+        self.max_seq_len = int(max_seq_len)
+        self.workspace = Workspace(self.device)
+        self.runtime = Runtime(self.device, self.dtype, self.workspace, self.max_seq_len)
+        with torch.cuda.device(self.device):
+            model.bind_all(tensors, self.runtime)
+        n_pages = -(-options.max_tokens // options.page_size)
+        max_slots = options.max_slots or min(n_pages, 1024)
+        self.cache = SequenceCache(model.cache_needs(), options.max_tokens, max_slots, self.max_seq_len,
+                                   options.page_size, self.device, self.dtype)
+        self.max_step_tokens = max(int(options.max_step_tokens), 1)
+        cap = 3 * self.max_step_tokens + 3 * max_slots + 1 + self.max_step_tokens
+        self._meta = torch.zeros(cap, dtype=torch.int32, device=self.device)
+        self.vocab_size = model.vocab_size
+        self.steps_run = 0
+
+    # ------------------------------------------------------------------
+    @classmethod
+    def from_dir(cls, model_dir: str, options: Optional[EngineOptions] = None) -> "Engine":
+        """Build the model that config.json names and load its weights from the folder."""
+        options = options or EngineOptions()
+        raw = read_config_json(model_dir)
+        arch = get_architecture(architecture_name(raw))
+        config = arch.config_class.from_dict(raw)
+        tied = None
+        if arch.tie_key is not None:
+            tied = arch.tie_key not in checkpoint_names(model_dir)
+        model = arch.build(config, tied=tied, sparse=options.sparse)
+        tensors = load_tensors(
+            model_dir, model.all_weight_specs(), device=options.device,
+            split_fused=(lambda n, t: arch.split_fused(config, n, t)) if arch.split_fused else None,
+            ignore=(lambda n: arch.ignore_tensor(config, n)) if arch.ignore_tensor else None)
+        return cls(config, model, tensors, options)
+
+    @classmethod
+    def from_tensors(cls, config: ModelConfig, tensors: Dict[str, torch.Tensor],
+                     options: Optional[EngineOptions] = None) -> "Engine":
+        options = options or EngineOptions()
+        arch = get_architecture(config.architecture)
+        tied = (arch.tie_key not in tensors) if arch.tie_key is not None else None
+        model = arch.build(config, tied=tied, sparse=options.sparse)
+        from ..weights.loader import _compare
+        _compare(model.all_weight_specs(), {k: tuple(v.shape) for k, v in tensors.items()}, "the given tensors")
+        dev = torch.device(options.device)
+        return cls(config, model, {k: v.to(dev) for k, v in tensors.items()}, options)
+
+    # ------------------------------------------------------------------
+    def acquire(self) -> int:
+        return self.cache.acquire()
+
+    def release(self, slot: int):
+        self.cache.release(slot)
+
+    def length(self, slot: int) -> int:
+        return self.cache.length(slot)
+
+    # ------------------------------------------------------------------
+    def _validate(self, entries: Sequence[StepEntry]):
+        if not entries:
+            raise StepError("a step needs at least one sequence")
+        seen = set()
+        V = self.vocab_size
+        pages = 0
+        for e in entries:
+            if e.slot in seen:
+                raise StepError(f"slot {e.slot} occurs twice in one step")
+            seen.add(e.slot)
+            try:
+                have = self.cache.length(e.slot)
+            except CacheError as err:
+                raise StepError(str(err)) from None
+            n = len(e.tokens)
+            if n == 0:
+                raise StepError(f"slot {e.slot}: a step must bring at least one token")
+            if have + n > self.max_seq_len:
+                raise StepError(f"slot {e.slot}: {have} cached + {n} new tokens exceed the longest sequence "
+                                f"this engine holds ({self.max_seq_len})")
+            bad = [t for t in e.tokens if not 0 <= int(t) < V]
+            if bad:
+                raise StepError(f"slot {e.slot}: token id {bad[0]} is outside the vocabulary [0, {V})")
+            for w in e.want:
+                if not 0 <= int(w) < n:
+                    raise StepError(f"slot {e.slot}: wanted place {w} is outside the {n} tokens of this step")
+            pages += self.cache.pages_needed(e.slot, have + n)
+        if pages > self.cache.free_page_count():
+            raise StepError(f"the cache is full: this step needs {pages} more pages of {self.cache.page_size} tokens, "
+                            f"{self.cache.free_page_count()} are free (max_tokens={self.options.max_tokens})")
+
+    def _chunks(self, entries: Sequence[StepEntry]):
+        """Cut a step into forward passes of at most max_step_tokens tokens.  Yields lists of
+        (entry index, first token, last token + 1)."""
+        cur: List[Tuple[int, int, int]] = []
+        room = self.max_step_tokens
+        for i, e in enumerate(entries):
+            a, n = 0, len(e.tokens)
+            while a < n:
+                take = min(n - a, room)
+                cur.append((i, a, a + take))
+                a += take
+                room -= take
+                if room == 0:
+                    yield cur
+                    cur, room = [], self.max_step_tokens
+        if cur:
+            yield cur
+
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """Run the entries' tokens; float32 logits [wanted, vocab] in the order of entries and of ``want``
+        (None if nothing is wanted)."""
+        entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
+        self._validate(entries)
+        row_of: Dict[Tuple[int, int], List[int]] = {}
+        n_rows = 0
+        for i, e in enumerate(entries):
+            for w in e.want:
+                row_of.setdefault((i, int(w)), []).append(n_rows)
+                n_rows += 1
+        result = torch.empty((n_rows, self.vocab_size), dtype=torch.float32, device=self.device) if n_rows else None
+        with torch.cuda.device(self.device):
+            for chunk in self._chunks(entries):
+                self._forward(entries, chunk, row_of, result)
+        self.steps_run += 1
+        return result
+
+    def _forward(self, entries, chunk, row_of, result):
+        cache = self.cache
+        B = len(chunk)
+        q_lens = [b - a for _, a, b in chunk]
+        n = sum(q_lens)
+        tok = np.empty(n, dtype=np.int32)
+        pos = np.empty(n, dtype=np.int32)
+        tslot = np.empty(n, dtype=np.int32)
+        cu = np.zeros(B + 1, dtype=np.int32)
+        sslot = np.empty(B, dtype=np.int32)
+        slen = np.empty(B, dtype=np.int32)
+        rows: List[int] = []
+        dest: List[int] = []
+        o = 0
+        for bi, (i, a, b) in enumerate(chunk):
+            e = entries[i]
+            first = cache.extend(e.slot, b - a)
+            q = b - a
+            tok[o:o + q] = np.asarray(e.tokens[a:b], dtype=np.int64)
+            pos[o:o + q] = np.arange(first, first + q, dtype=np.int32)
+            tslot[o:o + q] = e.slot
+            cu[bi + 1] = o + q
+            sslot[bi] = e.slot
+            slen[bi] = first + q
+            for w in e.want:
+                w = int(w)
+                if a <= w < b and (i, w) in row_of:
+                    for r in row_of.pop((i, w)):
+                        rows.append(o + (w - a))
+                        dest.append(r)
+            o += q
+        cache.sync()
+        R = len(rows)
+        host = np.concatenate([tok, pos, tslot, cu, sslot, slen, np.asarray(rows, dtype=np.int32)])
+        if host.size > self._meta.numel():
+            self._meta = torch.zeros(host.size * 2, dtype=torch.int32, device=self.device)
+        meta = self._meta
+        meta[:host.size].copy_(torch.from_numpy(host))
+        o1, o2, o3 = n, 2 * n, 3 * n
+        o4 = o3 + B + 1
+        o5 = o4 + B
+        o6 = o5 + B
+        ctx = StepContext(
+            n_tokens=n, n_seqs=B, token_ids=meta[0:o1], positions=meta[o1:o2], tok_slot=meta[o2:o3],
+            cu_q=meta[o3:o4], seq_slot=meta[o4:o5], seq_len=meta[o5:o6], q_lens=q_lens,
+            kv_lens=[int(x) for x in slen], max_pos=int(pos.max()), single_token=all(q == 1 for q in q_lens),
+            ws=self.workspace, cache=cache, logit_rows=meta[o6:o6 + R] if R else None)
+        logits = self.model.forward(ctx)
+        if R:
+            result.index_copy_(0, torch.tensor(dest, dtype=torch.long, device=self.device), logits)
+
+    # ------------------------------------------------------------------
+    def memory_report(self) -> Dict[str, int]:
+        return {"cache_bytes": self.cache.bytes(), "workspace_bytes": self.workspace.bytes(),
+                "pages": self.cache.n_pages, "slots": self.cache.max_slots}

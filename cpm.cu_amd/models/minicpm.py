@@ -1,0 +1,98 @@
+"""MiniCPM4 (``MiniCPMForCausalLM``): which parts, with which numbers.
+
+Pre-norm decoder with muP scaling (cpmcu/llm.py:67-69): embeddings times
+scale_emb, residual branches times scale_depth/sqrt(L), final hidden times
+dim_model_base/hidden before the head; GQA attention with LongRoPE, InfLLM-v2
+block-sparse attention when sparse_config is given; SiLU-gated feed-forward;
+RMSNorm.  Checkpoint names are the HF ones (src/model/model.cuh:122-143,
+src/model/minicpm4/minicpm4_attn.cuh:79-95, src/model/ffn.cuh:61-75); fused
+``qkv_proj`` / ``gate_up_proj`` tensors are split as cpmcu/llm.py:125-131 does.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from ..config.minicpm import MiniCPMConfig
+from ..parts import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, LMHead, PartSpec, TokenEmbedding)
+from ..registry import Architecture, register_architecture
+from .decoder import DecoderModel
+
+ARCHITECTURE = "MiniCPMForCausalLM"
+
+
+def layer_specs(cfg: MiniCPMConfig, sparse: bool = True) -> List[Dict[str, PartSpec]]:
+    """The parts of every layer, chosen layer by layer from the configuration."""
+    if cfg.rope_scaling is not None:
+        rs = cfg.rope_scaling
+        position = PartSpec.of("longrope", head_dim=cfg.head_dim, theta=cfg.rope_theta,
+                               short_factor=rs.short_factor, long_factor=rs.long_factor,
+                               original_max_position=rs.original_max_position_embeddings,
+                               max_position=cfg.max_position_embeddings,
+                               attention_scaling=cfg.rope_attention_scaling)
+    else:
+        position = PartSpec.of("rope", head_dim=cfg.head_dim, theta=cfg.rope_theta)
+    specs = []
+    for i in range(cfg.num_hidden_layers):
+        p = f"model.layers.{i}."
+        attn = dict(prefix=p + "self_attn.", hidden_size=cfg.hidden_size, num_heads=cfg.num_attention_heads,
+                    num_kv_heads=cfg.num_key_value_heads, head_dim=cfg.head_dim)
+        if cfg.sparse_config is not None and sparse:
+            mixer = PartSpec.of("infllm_v2_attention", **attn, **cfg.sparse_config.to_dict())
+        else:
+            mixer = PartSpec.of("gqa_attention", **attn)
+        specs.append({
+            "position": position,
+            "mixer_norm": PartSpec.of("rms_norm", name=p + "input_layernorm.weight", hidden_size=cfg.hidden_size,
+                                      eps=cfg.rms_norm_eps),
+            "mixer": mixer,
+            "ff_norm": PartSpec.of("rms_norm", name=p + "post_attention_layernorm.weight",
+                                   hidden_size=cfg.hidden_size, eps=cfg.rms_norm_eps),
+            "feed_forward": PartSpec.of("gated_silu", prefix=p + "mlp.", hidden_size=cfg.hidden_size,
+                                        intermediate_size=cfg.intermediate_size),
+            "block": PartSpec.of("pre_norm", residual_scale=cfg.residual_scale),
+        })
+    return specs
+
+
+def build(cfg: MiniCPMConfig, tied: Optional[bool] = None, sparse: bool = True) -> DecoderModel:
+    tie = cfg.tie_word_embeddings if cfg.tie_word_embeddings is not None else bool(tied)
+    layers = []
+    for s in layer_specs(cfg, sparse):
+        position = s["position"].build(POSITION_ENCODINGS)
+        layers.append(s["block"].build(
+            BLOCKS,
+            mixer_norm=s["mixer_norm"].build(NORMS),
+            mixer=s["mixer"].build(MIXERS, position=position),
+            ff_norm=s["ff_norm"].build(NORMS),
+            feed_forward=s["feed_forward"].build(FEED_FORWARDS)))
+    embedding = TokenEmbedding("model.embed_tokens.weight", cfg.vocab_size, cfg.hidden_size, cfg.scale_emb)
+    head = LMHead("lm_head.weight", cfg.vocab_size, cfg.hidden_size, cfg.head_scale, tied_to=embedding if tie else None)
+    final_norm = NORMS.build("rms_norm", name="model.norm.weight", hidden_size=cfg.hidden_size, eps=cfg.rms_norm_eps)
+    return DecoderModel(cfg, embedding, layers, final_norm, head)
+
+
+def split_fused(cfg: MiniCPMConfig, name: str, tensor: torch.Tensor) -> Optional[List[Tuple[str, torch.Tensor]]]:
+    """Checkpoints may hold q,k,v or gate,up as one tensor stacked on the output axis (cpmcu/llm.py:125-131)."""
+    if "gate_up_proj" in name:
+        half = tensor.shape[0] // 2
+        return [(name.replace("gate_up_proj", "gate_proj"), tensor[:half]),
+                (name.replace("gate_up_proj", "up_proj"), tensor[half:])]
+    if "qkv_proj" in name:
+        q = cfg.num_attention_heads * cfg.head_dim
+        kv = cfg.num_key_value_heads * cfg.head_dim
+        return [(name.replace("qkv_proj", "q_proj"), tensor[:q]),
+                (name.replace("qkv_proj", "k_proj"), tensor[q:q + kv]),
+                (name.replace("qkv_proj", "v_proj"), tensor[q + kv:])]
+    return None
+
+
+def ignore_tensor(cfg: MiniCPMConfig, name: str) -> bool:
+    """Tensors a checkpoint may carry that the engine computes itself."""
+    return "rotary_emb.inv_freq" in name
+
+
+register_architecture(Architecture(
+    name=ARCHITECTURE, config_class=MiniCPMConfig, build=build, split_fused=split_fused, ignore_tensor=ignore_tensor,
+    tie_key="lm_head.weight"))

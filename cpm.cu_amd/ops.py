@@ -1,0 +1,266 @@
+"""Python face of the HIP kernels: argument checks, then one launch each.
+
+Tensors are torch tensors on the GPU, used as typed memory only; every function
+launches on torch's current stream and allocates nothing.  Shapes are checked
+here, on the host, before a pointer reaches a kernel; a size a kernel does not
+take is refused with an error that names it.  There is no fallback: without a
+GPU or without the built libraries these functions raise.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_char_p, c_float, c_int, c_long, c_ulonglong, c_void_p
+from typing import Optional, Sequence
+
+import torch
+
+from .csrc import build as _build
+
+F32, BF16 = 0, 1
+_DT = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+class KernelError(RuntimeError):
+    """A kernel entry point refused its arguments or failed to launch."""
+
+
+def _code(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise KernelError(f"element type {t.dtype} is not supported (float32 or bfloat16)") from None
+
+
+def _need(t: torch.Tensor, name: str, dtype=None, shape: Optional[Sequence[Optional[int]]] = None):
+    if not isinstance(t, torch.Tensor) or t.device.type != "cuda":
+        raise KernelError(f"{name}: a GPU tensor is needed (no CPU path exists), got "
+                          f"{getattr(t, 'device', type(t).__name__)}")
+    if not t.is_contiguous():
+        raise KernelError(f"{name}: must be contiguous, strides {tuple(t.stride())} for shape {tuple(t.shape)}")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name}: dtype {t.dtype}, expected {dtype}")
+    if shape is not None:
+        if t.dim() != len(shape) or any(s is not None and s != d for s, d in zip(shape, t.shape)):
+            raise KernelError(f"{name}: shape {tuple(t.shape)}, expected {tuple('*' if s is None else s for s in shape)}")
+
+
+def _p(t: Optional[torch.Tensor]):
+    return c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream():
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+_fn_cache = {}
+
+
+def _fn(module: str, name: str):
+    key = (module, name)
+    f = _fn_cache.get(key)
+    if f is None:
+        lib = _build.load(module)
+        f = getattr(lib, name)
+        f.restype = c_char_p
+        _fn_cache[key] = f
+    return f
+
+
+def _check(msg):
+    if msg:
+        raise KernelError(msg.decode())
+
+
+# ---------------------------------------------------------------------------
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, scale: float):
+    """out[r] = float(table[ids[r]]) * scale;  table [V,H], ids int32 [n], out float32 [n,H]."""
+    _need(table, "embed table", shape=(None, None))
+    V, H = table.shape
+    _need(ids, "embed ids", torch.int32, (None,))
+    n = ids.shape[0]
+    _need(out, "embed out", torch.float32, (n, H))
+    _check(_fn("core", "cpmcu_embed")(_p(table), c_int(_code(table)), _p(ids), _p(out), c_int(n), c_int(H), c_int(V),
+                                      c_float(scale), _stream()))
+
+
+def add_rms_norm(x: torch.Tensor, branch: Optional[torch.Tensor], branch_scale: float, weight: torch.Tensor,
+                 eps: float, out: torch.Tensor, rows: Optional[torch.Tensor] = None):
+    """x += branch_scale * branch (in place; summed over the leading axis if branch is [P,n,H]);
+    out = rmsnorm(x) * weight.  With ``rows`` (int32 [R]) only those rows are normed, into out [R,H],
+    and x is left as it was."""
+    _need(x, "norm x", torch.float32, (None, None))
+    n, H = x.shape
+    _need(weight, "norm weight", torch.float32, (H,))
+    nparts, stride, bcode = 1, 0, F32
+    if branch is not None:
+        if branch.dim() == 3:
+            _need(branch, "norm branch", shape=(None, n, H))
+            nparts, stride = branch.shape[0], n * H
+        else:
+            _need(branch, "norm branch", shape=(n, H))
+        bcode = _code(branch)
+    if rows is not None:
+        _need(rows, "norm rows", torch.int32, (None,))
+        n_out = rows.shape[0]
+    else:
+        n_out = n
+    _need(out, "norm out", shape=(n_out, H))
+    _check(_fn("core", "cpmcu_add_rms_norm")(_p(x), _p(branch), c_int(bcode), c_int(nparts), c_long(stride),
+                                             c_float(branch_scale), _p(weight), c_float(eps), _p(out),
+                                             c_int(_code(out)), _p(rows), c_int(n_out), c_int(H), _stream()))
+
+
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor):
+    """out[r,c] = silu(gate_up[r,c]) * gate_up[r,c+I];  gate_up [n,2I], out [n,I]."""
+    _need(gate_up, "silu_mul input", shape=(None, None))
+    n, two_i = gate_up.shape
+    if two_i % 2:
+        raise KernelError(f"silu_mul: input width {two_i} is odd")
+    _need(out, "silu_mul out", gate_up.dtype, (n, two_i // 2))
+    _check(_fn("core", "cpmcu_silu_mul")(_p(gate_up), _p(out), c_int(_code(out)), c_int(n), c_int(two_i // 2), _stream()))
+
+
+def rope_store(qkv: torch.Tensor, q_out: torch.Tensor, nh: int, nkv: int, hd: int, positions: torch.Tensor,
+               tok_slot: torch.Tensor, inv_freq: Optional[torch.Tensor], mscale: float,
+               kpool: Optional[torch.Tensor], vpool: Optional[torch.Tensor], page_table: Optional[torch.Tensor],
+               page_size: int, write_kv: bool = True):
+    """Rotate q (and k), write q to q_out [n, nh*hd] and k, v into the paged cache.
+    qkv [n, W] or float32 partial sums [P, n, W] with W >= (nh + 2 nkv) hd (nh*hd if not write_kv)."""
+    if qkv.dim() == 3:
+        _need(qkv, "rope qkv", torch.float32, (None, None, None))
+        nparts, n, width = qkv.shape
+        stride = n * width
+    else:
+        _need(qkv, "rope qkv", shape=(None, None))
+        n, width = qkv.shape
+        nparts, stride = 1, 0
+    _need(q_out, "rope q_out", shape=(n, nh * hd))
+    _need(positions, "rope positions", torch.int32, (n,))
+    _need(tok_slot, "rope token slots", torch.int32, (n,))
+    if inv_freq is not None:
+        _need(inv_freq, "rope inv_freq", torch.float32, (hd // 2,))
+    tw = 0
+    if write_kv:
+        _need(page_table, "rope page table", torch.int32, (None, None))
+        tw = page_table.shape[1]
+        _need(kpool, "rope key pool", q_out.dtype, (None, page_size, nkv * hd))
+        _need(vpool, "rope value pool", q_out.dtype, tuple(kpool.shape))
+    _check(_fn("core", "cpmcu_rope_store")(_p(qkv), c_long(width), c_int(_code(qkv)), c_int(nparts), c_long(stride),
+                                           _p(q_out), c_int(_code(q_out)), c_int(n), c_int(nh), c_int(nkv), c_int(hd),
+                                           _p(positions), _p(tok_slot), _p(inv_freq), c_float(mscale), _p(kpool),
+                                           _p(vpool), _p(page_table), c_int(tw), c_int(page_size),
+                                           c_int(1 if write_kv else 0), _stream()))
+
+
+def gemm_nt_plain(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, alpha: float = 1.0):
+    """out[m,N] = alpha * x[m,K] . w[N,K]^T with scalar float FMAs (any size, both element types)."""
+    _need(x, "gemm x", shape=(None, None))
+    M, K = x.shape
+    _need(w, "gemm weight", x.dtype, (None, K))
+    N = w.shape[0]
+    _need(out, "gemm out", shape=(M, N))
+    _check(_fn("gemm", "cpmcu_gemm_nt_plain")(_p(x), c_long(K), _p(w), c_long(K), _p(out), c_long(N), c_int(_code(x)),
+                                              c_int(_code(out)), c_int(M), c_int(N), c_int(K), c_float(alpha),
+                                              _stream()))
+
+
+def attention_plain(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hd: int, scale: float,
+                    kpool: torch.Tensor, vpool: torch.Tensor, page_table: torch.Tensor, page_size: int,
+                    positions: torch.Tensor, tok_slot: torch.Tensor,
+                    sel_blocks: Optional[torch.Tensor] = None, sel_count: Optional[torch.Tensor] = None,
+                    block_size: int = 0):
+    """Causal GQA attention of n query tokens over their sequences' cached keys (plain kernel)."""
+    _need(q, "attention q", shape=(None, nh * hd))
+    n = q.shape[0]
+    _need(out, "attention out", q.dtype, (n, nh * hd))
+    _need(kpool, "attention key pool", q.dtype, (None, page_size, nkv * hd))
+    _need(vpool, "attention value pool", q.dtype, tuple(kpool.shape))
+    _need(page_table, "attention page table", torch.int32, (None, None))
+    _need(positions, "attention positions", torch.int32, (n,))
+    _need(tok_slot, "attention token slots", torch.int32, (n,))
+    max_sel = 0
+    if sel_count is not None:
+        _need(sel_count, "attention block counts", torch.int32, (n, nkv))
+        _need(sel_blocks, "attention block list", torch.int32, (n, nkv, None))
+        max_sel = sel_blocks.shape[2]
+    _check(_fn("attention", "cpmcu_attention_plain")(
+        _p(q), _p(out), c_int(_code(q)), c_int(n), c_int(nh), c_int(nkv), c_int(hd), c_float(scale), _p(kpool),
+        _p(vpool), _p(page_table), c_int(page_table.shape[1]), c_int(page_size), _p(positions), _p(tok_slot),
+        _p(sel_blocks), _p(sel_count), c_int(max_sel), c_int(block_size), _stream()))
+
+
+def compress_keys(kpool: torch.Tensor, ckpool: torch.Tensor, page_table: torch.Tensor, page_size: int,
+                  positions: torch.Tensor, tok_slot: torch.Tensor, kernel_size: int, kernel_stride: int):
+    """Write the compressed keys (means of kernel_size keys, every kernel_stride) that the step's tokens complete."""
+    _need(kpool, "compress key pool", shape=(None, page_size, None))
+    width = kpool.shape[2]
+    if kernel_stride <= 0 or page_size % kernel_stride:
+        raise KernelError(f"compress_keys: kernel_stride {kernel_stride} must divide the cache page of {page_size} tokens")
+    _need(ckpool, "compressed key pool", kpool.dtype, (kpool.shape[0], page_size // kernel_stride, width))
+    _need(page_table, "compress page table", torch.int32, (None, None))
+    _need(positions, "compress positions", torch.int32, (None,))
+    n = positions.shape[0]
+    _need(tok_slot, "compress token slots", torch.int32, (n,))
+    _check(_fn("sparse", "cpmcu_compress_keys")(_p(kpool), _p(ckpool), c_int(_code(kpool)), c_int(n), c_int(width),
+                                                _p(page_table), c_int(page_table.shape[1]), c_int(page_size),
+                                                _p(positions), _p(tok_slot), c_int(kernel_size), c_int(kernel_stride),
+                                                _stream()))
+
+
+def sparse_select(q: torch.Tensor, ckpool: torch.Tensor, nh: int, nkv: int, hd: int, scale: float,
+                  page_table: torch.Tensor, page_size: int, positions: torch.Tensor, tok_slot: torch.Tensor,
+                  kernel_size: int, kernel_stride: int, block_size: int, init_blocks: int, topk: int,
+                  window_blocks: int, dense_len: int, max_pos: int, sel_blocks: torch.Tensor, sel_count: torch.Tensor):
+    """Block list per (token, kv head): sel_count -1 = dense, else the ascending blocks to attend to."""
+    _need(q, "select q", shape=(None, nh * hd))
+    n = q.shape[0]
+    _need(ckpool, "select compressed keys", q.dtype, (None, page_size // max(kernel_stride, 1), nkv * hd))
+    _need(page_table, "select page table", torch.int32, (None, None))
+    _need(positions, "select positions", torch.int32, (n,))
+    _need(tok_slot, "select token slots", torch.int32, (n,))
+    _need(sel_count, "select counts", torch.int32, (n, nkv))
+    _need(sel_blocks, "select block list", torch.int32, (n, nkv, None))
+    _check(_fn("sparse", "cpmcu_sparse_select")(
+        _p(q), _p(ckpool), c_int(_code(q)), c_int(n), c_int(nh), c_int(nkv), c_int(hd), c_float(scale),
+        _p(page_table), c_int(page_table.shape[1]), c_int(page_size), _p(positions), _p(tok_slot),
+        c_int(kernel_size), c_int(kernel_stride), c_int(block_size), c_int(init_blocks), c_int(topk),
+        c_int(window_blocks), c_int(dense_len), c_int(max_pos), _p(sel_blocks), _p(sel_count),
+        c_int(sel_blocks.shape[2]), _stream()))
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor):
+    """out[r] = index of the largest logits[r] (ties: the lowest index)."""
+    _need(logits, "argmax logits", torch.float32, (None, None))
+    R, V = logits.shape
+    _need(out, "argmax out", torch.int32, (R,))
+    _check(_fn("core", "cpmcu_argmax")(_p(logits), c_long(V), c_int(R), c_int(V), _p(out), _stream()))
+
+
+def sample(logits: torch.Tensor, temperature: float, seed: int, request_ids: torch.Tensor, steps: torch.Tensor,
+           out: torch.Tensor, u_out: Optional[torch.Tensor] = None):
+    """out[r] ~ softmax(logits[r] / temperature), the uniform number keyed by (seed, request_ids[r], steps[r])."""
+    _need(logits, "sample logits", torch.float32, (None, None))
+    R, V = logits.shape
+    _need(request_ids, "sample request ids", torch.int32, (R,))
+    _need(steps, "sample steps", torch.int32, (R,))
+    _need(out, "sample out", torch.int32, (R,))
+    if u_out is not None:
+        _need(u_out, "sample u_out", torch.float32, (R,))
+    _check(_fn("core", "cpmcu_sample")(_p(logits), c_long(V), c_int(R), c_int(V), c_float(temperature),
+                                       c_ulonglong(seed & 0xFFFFFFFFFFFFFFFF), _p(request_ids), _p(steps), _p(out),
+                                       _p(u_out), _stream()))
+
+
+# ---------------------------------------------------------------------------
+# dispatchers: choose the kernel for a shape and element type
+# ---------------------------------------------------------------------------
+def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, alpha: float = 1.0):
+    """out = alpha * x . w^T with the kernel that suits the element type and the number of rows."""
+    gemm_nt_plain(x, w, out, alpha)
+
+
+def attention(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, ctx,
+              sel_blocks=None, sel_count=None, block_size=0):
+    """Attention of the step's queries over the cache, with the kernel that suits the step."""
+    attention_plain(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, ctx.positions, ctx.tok_slot,
+                    sel_blocks, sel_count, block_size)

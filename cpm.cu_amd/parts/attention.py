@@ -1,0 +1,120 @@
+"""Attention mixers: dense causal GQA attention, and InfLLM-v2 block-sparse
+attention on top of it.
+
+Dense (src/model/attn.cuh:58-284): q, k, v from one stacked product, position
+encoding on q and k, k and v into the cache (the cache holds encoded keys),
+attention of every query over its sequence's cached keys up to itself, output
+projection.  scores = (q.k) * head_dim^-1/2; query head h reads kv head
+h // (heads / kv_heads).
+
+InfLLM-v2 (src/model/minicpm4/minicpm4_attn.cuh:107-202): past ``dense_len``
+tokens a query attends only to chosen blocks of keys: blocks scored through
+compressed keys (means of kernel_size keys every kernel_stride), the top-k of
+them, plus initial blocks and a trailing window.  The reference selects per
+call; here the selection of the query at position p uses only what lies before
+p, so it does not depend on how the tokens were cut into steps:
+compressed key j is visible iff kernel_stride*j + kernel_size <= p.
+"""
+from __future__ import annotations
+
+from typing import List, Mapping, Optional
+
+import torch
+
+from .. import ops
+from ..cache.paged import CacheNeeds, CacheView, StreamSpec
+from .base import MIXERS, Mixer, Part, PositionEncoding, Runtime, StepContext
+from .linear import Linear
+
+
+@MIXERS.register("gqa_attention")
+class GQAAttention(Mixer):
+    def __init__(self, prefix: str, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 position: Optional[PositionEncoding], scale: Optional[float] = None):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"attention: {num_heads} heads are not a multiple of {num_kv_heads} kv heads")
+        self.hidden_size = hidden_size
+        self.nh, self.nkv, self.hd = num_heads, num_kv_heads, head_dim
+        self.position = position
+        self.scale = float(scale) if scale is not None else head_dim ** -0.5
+        self.qkv = Linear([(prefix + "q_proj.weight", num_heads * head_dim),
+                           (prefix + "k_proj.weight", num_kv_heads * head_dim),
+                           (prefix + "v_proj.weight", num_kv_heads * head_dim)], hidden_size)
+        self.o = Linear([(prefix + "o_proj.weight", hidden_size)], num_heads * head_dim)
+
+    def parts(self) -> List[Part]:
+        return [self.qkv, self.o] + ([self.position] if self.position is not None else [])
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime):
+        self.rt = rt
+
+    def cache_needs(self) -> CacheNeeds:
+        w = self.nkv * self.hd
+        return CacheNeeds(streams=(("k", StreamSpec(w)), ("v", StreamSpec(w))))
+
+    # -- steps of forward, so that a subclass can put its own between them --
+    def project_and_store(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool) -> torch.Tensor:
+        n = h.shape[0]
+        nh, nkv, hd = self.nh, self.nkv, self.hd
+        qkv = self.qkv.forward(h, ctx, "attn.qkv", rows=None if writes_cache else nh * hd)
+        rot = self.position.rotary_params() if self.position is not None else None
+        inv_freq, mag = (rot if rot is not None else (None, 1.0))
+        if self.position is not None and rot is None:
+            q3 = qkv[:, :nh * hd].unflatten(1, (nh, hd))
+            k3 = qkv[:, nh * hd:(nh + nkv) * hd].unflatten(1, (nkv, hd)) if writes_cache else None
+            self.position.apply(q3, k3, ctx)
+        q = ctx.ws.get("attn.q", (n, nh * hd), self.rt.dtype)
+        ops.rope_store(qkv, q, nh, nkv, hd, ctx.positions, ctx.tok_slot, inv_freq, mag,
+                       cache.streams["k"] if writes_cache else None, cache.streams["v"] if writes_cache else None,
+                       cache.page_table if writes_cache else None, cache.page_size, writes_cache)
+        return q
+
+    def attend(self, q, ctx: StepContext, cache: CacheView, sel=None) -> torch.Tensor:
+        out = ctx.ws.get("attn.out", tuple(q.shape), q.dtype)
+        sel_blocks, sel_count, bs = sel if sel is not None else (None, None, 0)
+        ops.attention(q, out, self.nh, self.nkv, self.hd, self.scale, cache.streams["k"], cache.streams["v"],
+                      cache.page_table, cache.page_size, ctx, sel_blocks, sel_count, bs)
+        return out
+
+    def forward(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool = True) -> torch.Tensor:
+        q = self.project_and_store(h, ctx, cache, writes_cache)
+        a = self.attend(q, ctx, cache)
+        return self.o.forward(a, ctx, "attn.o", out_dtype=torch.float32)
+
+
+@MIXERS.register("infllm_v2_attention")
+class InfLLMv2Attention(GQAAttention):
+    def __init__(self, prefix: str, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 position: Optional[PositionEncoding], kernel_size: int, kernel_stride: int, block_size: int,
+                 init_blocks: int, topk: int, window_size: int, dense_len: int, scale: Optional[float] = None):
+        super().__init__(prefix, hidden_size, num_heads, num_kv_heads, head_dim, position, scale)
+        if block_size % kernel_stride or kernel_size < kernel_stride:
+            raise ValueError("infllm_v2: block_size must be a multiple of kernel_stride <= kernel_size")
+        if window_size % block_size or window_size < block_size:
+            raise ValueError("infllm_v2: window_size must be a positive multiple of block_size")
+        self.ks, self.st, self.bs = kernel_size, kernel_stride, block_size
+        self.init_blocks, self.topk, self.dense_len = init_blocks, topk, dense_len
+        self.window_blocks = window_size // block_size
+
+    def cache_needs(self) -> CacheNeeds:
+        w = self.nkv * self.hd
+        return CacheNeeds(streams=(("k", StreamSpec(w)), ("v", StreamSpec(w)), ("ck", StreamSpec(w, every=self.st))))
+
+    def forward(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool = True) -> torch.Tensor:
+        q = self.project_and_store(h, ctx, cache, writes_cache)
+        if writes_cache:
+            ops.compress_keys(cache.streams["k"], cache.streams["ck"], cache.page_table, cache.page_size,
+                              ctx.positions, ctx.tok_slot, self.ks, self.st)
+        sel = None
+        if ctx.max_pos + 1 > self.dense_len:
+            n = q.shape[0]
+            max_sel = self.topk + self.window_blocks
+            sel_blocks = ctx.ws.get("attn.sel_blocks", (n, self.nkv, max_sel), torch.int32)
+            sel_count = ctx.ws.get("attn.sel_count", (n, self.nkv), torch.int32)
+            ops.sparse_select(q, cache.streams["ck"], self.nh, self.nkv, self.hd, self.scale, cache.page_table,
+                              cache.page_size, ctx.positions, ctx.tok_slot, self.ks, self.st, self.bs,
+                              self.init_blocks, self.topk, self.window_blocks, self.dense_len, ctx.max_pos,
+                              sel_blocks, sel_count)
+            sel = (sel_blocks, sel_count, self.bs)
+        a = self.attend(q, ctx, cache, sel)
+        return self.o.forward(a, ctx, "attn.o", out_dtype=torch.float32)

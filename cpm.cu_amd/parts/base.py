@@ -1,0 +1,227 @@
+"""Interfaces of the parts a layer is put together from, and their registries.
+
+A part owns its sizes and constants (given to its constructor), says which
+checkpoint tensors it needs (``weight_specs``), takes them (``bind``) and runs
+(``forward``).  No part knows which model it is in: a model file only chooses
+parts by name and hands them numbers from its configuration.
+
+Kinds of parts and what each must provide:
+
+* ``Norm``:      forward(x, branch, branch_scale, ctx, rows=None) -> normed [n or R, H]
+                 (adds ``branch_scale * branch`` into the float residual ``x`` first)
+* ``PositionEncoding``: rotary_params() -> (inv_freq, magnitude) or None, and
+                 apply(q, k, ctx) for encodings that are not a plain rotation
+* ``Mixer``:     cache_needs() and forward(h, ctx, cache, writes_cache) -> branch [n, H] or [P, n, H]
+* ``FeedForward``: forward(h, ctx) -> branch [n, H] or [P, n, H]
+* ``Block``:     forward(stream, ctx, cache, writes_cache): the arrangement of the above
+                 around the residual stream
+
+Branches may come back as float partial sums ``[P, n, H]`` of a split matrix
+product; whoever adds them to the residual sums them.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Callable, Dict, List, Mapping, Optional, Sequence, Tuple
+
+import torch
+
+from ..cache.paged import CacheNeeds, CacheView, SequenceCache
+
+
+# ---------------------------------------------------------------------------
+# weights
+# ---------------------------------------------------------------------------
+@dataclass(frozen=True)
+class WeightSpec:
+    """A checkpoint tensor a part needs.  ``init`` tells the random-weights
+    writer how to draw it: 'matrix' N(0, std), 'norm' 1 + N(0, norm_std),
+    'table' like 'matrix'.  ``storage`` is the dtype it is written in and kept
+    in by the loader ('bfloat16', 'float32' or 'int32')."""
+    name: str
+    shape: Tuple[int, ...]
+    init: str = "matrix"
+    storage: str = "bfloat16"
+
+
+# ---------------------------------------------------------------------------
+# run-time objects handed to parts
+# ---------------------------------------------------------------------------
+class Workspace:
+    """Named scratch buffers that live as long as the engine: a part asks for
+    ``get(name, shape, dtype)`` and receives the same memory at every step (it
+    grows when a larger shape is asked for), so steps allocate nothing and a
+    captured step replays on fixed addresses."""
+
+    def __init__(self, device):
+        self.device = torch.device(device)
+        self._buf: Dict[str, torch.Tensor] = {}
+
+    def get(self, name: str, shape: Sequence[int], dtype: torch.dtype) -> torch.Tensor:
+        n = 1
+        for s in shape:
+            n *= int(s)
+        nbytes = n * torch.empty((), dtype=dtype).element_size()
+        buf = self._buf.get(name)
+        if buf is None or buf.numel() < nbytes:
+            buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=self.device)
+            self._buf[name] = buf
+        return buf[:nbytes].view(dtype).view(*shape)
+
+    def bytes(self) -> int:
+        return sum(b.numel() for b in self._buf.values())
+
+
+@dataclass
+class Runtime:
+    """What an engine gives every part at bind time."""
+    device: torch.device
+    dtype: torch.dtype            # element type of activations, weights and cache: float32 or bfloat16
+    workspace: Workspace
+    max_seq_len: int              # longest sequence the engine holds
+
+
+@dataclass
+class StepContext:
+    """One step's batch as every part sees it: packed tokens of several sequences."""
+    n_tokens: int
+    n_seqs: int
+    token_ids: torch.Tensor       # int32 [n]
+    positions: torch.Tensor       # int32 [n] absolute position of each token in its sequence
+    tok_slot: torch.Tensor        # int32 [n] cache slot of each token
+    cu_q: torch.Tensor            # int32 [B+1] start of each sequence's tokens in the packed batch
+    seq_slot: torch.Tensor        # int32 [B]
+    seq_len: torch.Tensor         # int32 [B] tokens each sequence holds after this step
+    q_lens: List[int]             # host copies
+    kv_lens: List[int]
+    max_pos: int                  # largest position in the step
+    single_token: bool            # every sequence brings exactly one token
+    ws: Workspace
+    cache: Optional[SequenceCache]
+    logit_rows: Optional[torch.Tensor] = None     # int32 [R]: packed token rows whose logits are wanted
+
+
+@dataclass
+class ResidualStream:
+    """The float residual ``x`` [n, H] and a branch not yet added to it."""
+    x: torch.Tensor
+    pending: Optional[torch.Tensor] = None
+    pending_scale: float = 1.0
+
+
+# ---------------------------------------------------------------------------
+# the part interfaces
+# ---------------------------------------------------------------------------
+class Part:
+    def parts(self) -> List["Part"]:
+        return []
+
+    def weight_specs(self) -> List[WeightSpec]:
+        return []
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime):
+        """Take the tensors named by weight_specs (already on the device) and prepare for forward."""
+
+    # helpers over the tree
+    def all_weight_specs(self) -> List[WeightSpec]:
+        out = list(self.weight_specs())
+        for p in self.parts():
+            out.extend(p.all_weight_specs())
+        return out
+
+    def bind_all(self, tensors: Mapping[str, torch.Tensor], rt: Runtime):
+        self.bind(tensors, rt)
+        for p in self.parts():
+            p.bind_all(tensors, rt)
+
+
+class Norm(Part):
+    def forward(self, x: torch.Tensor, branch: Optional[torch.Tensor], branch_scale: float, ctx: StepContext,
+                rows: Optional[torch.Tensor] = None, tag: str = "norm") -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def rotary_params(self) -> Optional[Tuple[torch.Tensor, float]]:
+        """(inv_freq float32 [head_dim/2], magnitude) if this encoding is a rotate-half rotation by
+        position * inv_freq, which the fused kernel applies while it writes the cache; else None."""
+        return None
+
+    def apply(self, q: torch.Tensor, k: Optional[torch.Tensor], ctx: StepContext):
+        """Encode positions into q [n, heads, hd] and k [n, kv_heads, hd] in place (used when
+        rotary_params() is None)."""
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_needs(self) -> CacheNeeds:
+        return CacheNeeds()
+
+    def forward(self, h: torch.Tensor, ctx: StepContext, cache: Optional[CacheView], writes_cache: bool = True
+                ) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, h: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block(Part):
+    mixer: Mixer
+
+    def forward(self, stream: ResidualStream, ctx: StepContext, cache: Optional[CacheView], writes_cache: bool = True):
+        raise NotImplementedError
+
+
+# ---------------------------------------------------------------------------
+# registries: kind name -> constructor
+# ---------------------------------------------------------------------------
+class Registry:
+    def __init__(self, what: str):
+        self.what = what
+        self._items: Dict[str, Callable] = {}
+
+    def register(self, name: str, ctor: Optional[Callable] = None):
+        def deco(c):
+            if name in self._items and self._items[name] is not c:
+                raise ValueError(f"{self.what} '{name}' is already registered")
+            self._items[name] = c
+            return c
+        return deco if ctor is None else deco(ctor)
+
+    def unregister(self, name: str):
+        self._items.pop(name, None)
+
+    def get(self, name: str) -> Callable:
+        try:
+            return self._items[name]
+        except KeyError:
+            raise KeyError(f"unknown {self.what} '{name}' (registered: {sorted(self._items)})") from None
+
+    def build(self, kind: str, /, **params):
+        return self.get(kind)(**params)
+
+    def names(self):
+        return sorted(self._items)
+
+
+NORMS = Registry("norm")
+POSITION_ENCODINGS = Registry("position encoding")
+MIXERS = Registry("mixer")
+FEED_FORWARDS = Registry("feed-forward")
+BLOCKS = Registry("block")
+
+
+@dataclass(frozen=True)
+class PartSpec:
+    """A part chosen by name with its parameters: what a model file writes per layer."""
+    kind: str
+    params: Tuple[Tuple[str, object], ...] = ()
+
+    @staticmethod
+    def of(kind: str, **params) -> "PartSpec":
+        return PartSpec(kind, tuple(sorted(params.items())))
+
+    def build(self, registry: Registry, **extra):
+        return registry.build(self.kind, **dict(self.params), **extra)

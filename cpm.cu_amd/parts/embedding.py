@@ -1,0 +1,58 @@
+"""Token embedding (times its scale) and the output head.
+
+x[t] = E[id_t] * scale_emb (src/model/embedding.cuh:7-20, 49-52); logits =
+(y * head_scale) . W^T with the head reading the unscaled table when the
+embeddings are tied (src/model/linear.cuh:86-105, cpmcu/llm.py:136-137).
+"""
+from __future__ import annotations
+
+from typing import List, Mapping, Optional
+
+import torch
+
+from .. import ops
+from .base import Part, Runtime, StepContext, WeightSpec
+
+
+class TokenEmbedding(Part):
+    def __init__(self, name: str, vocab_size: int, hidden_size: int, scale: float = 1.0):
+        self.name = name
+        self.vocab_size = vocab_size
+        self.hidden_size = hidden_size
+        self.scale = float(scale)
+        self.table: Optional[torch.Tensor] = None
+
+    def weight_specs(self) -> List[WeightSpec]:
+        return [WeightSpec(self.name, (self.vocab_size, self.hidden_size), "table")]
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime):
+        self.table = tensors[self.name].to(rt.dtype).contiguous()
+
+    def forward(self, ctx: StepContext) -> torch.Tensor:
+        x = ctx.ws.get("residual", (ctx.n_tokens, self.hidden_size), torch.float32)
+        ops.embed(self.table, ctx.token_ids, x, self.scale)
+        return x
+
+
+class LMHead(Part):
+    def __init__(self, name: str, vocab_size: int, hidden_size: int, scale: float = 1.0,
+                 tied_to: Optional[TokenEmbedding] = None):
+        self.name = name
+        self.vocab_size = vocab_size
+        self.hidden_size = hidden_size
+        self.scale = float(scale)
+        self.tied_to = tied_to
+        self.weight: Optional[torch.Tensor] = None
+
+    def weight_specs(self) -> List[WeightSpec]:
+        return [] if self.tied_to is not None else [WeightSpec(self.name, (self.vocab_size, self.hidden_size), "table")]
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime):
+        if self.tied_to is None:
+            self.weight = tensors[self.name].to(rt.dtype).contiguous()
+
+    def forward(self, y: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        w = self.tied_to.table if self.tied_to is not None else self.weight
+        logits = ctx.ws.get("logits", (y.shape[0], self.vocab_size), torch.float32)
+        ops.linear(y, w, logits, self.scale)
+        return logits

@@ -1,0 +1,33 @@
+"""SiLU-gated feed-forward: down( silu(x Wg^T) * (x Wu^T) ).
+
+gate and up are one stacked product, gate rows first (src/model/ffn.cuh:31-59,
+77-84); silu(g) * u in float (src/model/activation.cuh:6-18).
+"""
+from __future__ import annotations
+
+from typing import List
+
+import torch
+
+from .. import ops
+from .base import FEED_FORWARDS, FeedForward, Part, StepContext
+from .linear import Linear
+
+
+@FEED_FORWARDS.register("gated_silu")
+class GatedFFN(FeedForward):
+    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int):
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+        self.gate_up = Linear([(prefix + "gate_proj.weight", intermediate_size),
+                               (prefix + "up_proj.weight", intermediate_size)], hidden_size)
+        self.down = Linear([(prefix + "down_proj.weight", hidden_size)], intermediate_size)
+
+    def parts(self) -> List[Part]:
+        return [self.gate_up, self.down]
+
+    def forward(self, h: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        gu = self.gate_up.forward(h, ctx, "ffn.gate_up")
+        act = ctx.ws.get("ffn.act", (h.shape[0], self.intermediate_size), h.dtype)
+        ops.silu_mul(gu, act)
+        return self.down.forward(act, ctx, "ffn.down", out_dtype=torch.float32)

@@ -1,0 +1,41 @@
+"""Linear layer: y = alpha * x . W^T with W [out, in] as in the checkpoint.
+
+Several checkpoint tensors may be stacked on the output axis into one weight
+(q, k, v; gate, up), as the reference lays them out contiguously so that one
+product serves them all (src/model/minicpm4/minicpm4_attn.cuh:48-55,
+src/model/ffn.cuh:44-50).
+"""
+from __future__ import annotations
+
+from typing import List, Mapping, Optional, Sequence, Tuple
+
+import torch
+
+from .. import ops
+from .base import Part, Runtime, StepContext, WeightSpec
+
+
+class Linear(Part):
+    def __init__(self, names: Sequence[Tuple[str, int]], in_features: int, init: str = "matrix"):
+        self.names = list(names)
+        self.in_features = in_features
+        self.out_features = sum(r for _, r in self.names)
+        self.init = init
+        self.weight: Optional[torch.Tensor] = None
+
+    def weight_specs(self) -> List[WeightSpec]:
+        return [WeightSpec(n, (r, self.in_features), self.init) for n, r in self.names]
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime):
+        ws = [tensors[n] for n, _ in self.names]
+        w = ws[0] if len(ws) == 1 else torch.cat(ws, dim=0)
+        self.weight = w.to(rt.dtype).contiguous()
+        self.rt = rt
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, tag: str, out_dtype: Optional[torch.dtype] = None,
+                alpha: float = 1.0, rows: Optional[int] = None) -> torch.Tensor:
+        """x [n, in] -> [n, out] (the first ``rows`` output features only, if given)."""
+        w = self.weight if rows is None else self.weight[:rows]
+        out = ctx.ws.get(tag, (x.shape[0], w.shape[0]), out_dtype or x.dtype)
+        ops.linear(x, w, out, alpha)
+        return out

@@ -1,0 +1,35 @@
+"""RMSNorm with the residual add fused in front of it.
+
+y = x * rsqrt(mean(x^2) + eps) * w  (src/model/norm.cuh:7-51); the branch of the
+previous sub-layer is added into the residual stream by the same kernel
+(src/model/norm.cuh:53-99), here with its scale and in float.
+"""
+from __future__ import annotations
+
+from typing import List, Mapping, Optional
+
+import torch
+
+from .. import ops
+from .base import NORMS, Norm, Runtime, StepContext, WeightSpec
+
+
+@NORMS.register("rms_norm")
+class RMSNorm(Norm):
+    def __init__(self, name: str, hidden_size: int, eps: float):
+        self.name = name
+        self.hidden_size = hidden_size
+        self.eps = float(eps)
+
+    def weight_specs(self) -> List[WeightSpec]:
+        return [WeightSpec(self.name, (self.hidden_size,), "norm")]
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime):
+        self.weight = tensors[self.name].to(torch.float32).contiguous()
+        self.rt = rt
+
+    def forward(self, x, branch, branch_scale, ctx: StepContext, rows=None, tag="norm"):
+        n_out = x.shape[0] if rows is None else rows.shape[0]
+        out = ctx.ws.get(tag, (n_out, self.hidden_size), self.rt.dtype)
+        ops.add_rms_norm(x, branch, branch_scale, self.weight, self.eps, out, rows)
+        return out
