@@ -1,0 +1,123 @@
+"""The generation loop above the step function.
+
+For one prompt the reference loops ``prefill -> sample -> (decode -> sample)*``,
+returns the stop token and ends the sequence on it, and counts the token sampled
+from the prompt's logits toward the length (cpmcu/llm.py:261-376).  Here the
+same loop runs over batches: prompts of unequal length start together in one
+step, every later step carries one token of each sequence still running, a
+sequence that ends gives its slot back at once, and when there are more
+requests than one batch holds, batches run one after another.
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Callable, Dict, Iterable, List, Optional, Sequence
+
+import torch
+
+from ..sampling.sampler import Sampler
+from .engine import Engine, StepEntry
+
+
+@dataclass
+class Completion:
+    tokens: List[int]
+    finish_reason: str                      # 'stop' (a stop token, which is returned) or 'length'
+    prefill_time: float = 0.0
+    decode_time: float = 0.0
+
+
+def plan_batches(prompt_lens: Sequence[int], max_new_tokens: int, max_batch: int, max_tokens: int,
+                 page_size: int, max_seq_len: int) -> List[List[int]]:
+    """Split request indices into batches that run one after another.
+
+    Requests keep their order.  A batch takes requests while it has a slot for each and the
+    cache can hold every one of them at its full length (prompt + max_new_tokens, rounded up
+    to whole pages)."""
+    if max_new_tokens < 1:
+        raise ValueError("max_new_tokens must be at least 1")
+    if max_batch < 1:
+        raise ValueError("max_batch must be at least 1")
+    pages_total = max_tokens // page_size if max_tokens % page_size == 0 else -(-max_tokens // page_size)
+    batches: List[List[int]] = []
+    cur: List[int] = []
+    cur_pages = 0
+    for i, n in enumerate(prompt_lens):
+        if n < 1:
+            raise ValueError(f"request {i}: the prompt is empty")
+        total = n + max_new_tokens - 1      # the last sampled token is never fed back
+        if total > max_seq_len:
+            raise ValueError(f"request {i}: prompt of {n} + {max_new_tokens} new tokens exceeds the longest sequence "
+                             f"the engine holds ({max_seq_len})")
+        pages = -(-total // page_size)
+        if pages > pages_total:
+            raise ValueError(f"request {i}: {total} tokens do not fit the cache of {max_tokens} tokens")
+        if cur and (len(cur) >= max_batch or cur_pages + pages > pages_total):
+            batches.append(cur)
+            cur, cur_pages = [], 0
+        cur.append(i)
+        cur_pages += pages
+    if cur:
+        batches.append(cur)
+    return batches
+
+
+def generate(engine: Engine, prompts: Sequence[Sequence[int]], max_new_tokens: int,
+             stop_token_ids: Iterable[int] = (), temperature: float = 0.0, seed: Optional[int] = None,
+             max_batch: Optional[int] = None, on_token: Optional[Callable[[int, int], None]] = None,
+             on_prefill: Optional[Callable[[str, dict], None]] = None) -> List[Completion]:
+    """Generate up to max_new_tokens for every prompt (lists of token ids).
+
+    ``on_token(request index, token)`` is called for each token as it is chosen."""
+    stop = set(int(t) for t in stop_token_ids)
+    sampler = Sampler(temperature, seed)
+    max_batch = max_batch or engine.cache.max_slots
+    max_batch = min(max_batch, engine.cache.max_slots)
+    batches = plan_batches([len(p) for p in prompts], max_new_tokens, max_batch, engine.options.max_tokens,
+                           engine.cache.page_size, engine.max_seq_len)
+    results: List[Optional[Completion]] = [None] * len(prompts)
+    for batch in batches:
+        _run_batch(engine, prompts, batch, max_new_tokens, stop, sampler, results, on_token, on_prefill)
+    return results  # type: ignore[return-value]
+
+
+def _run_batch(engine, prompts, batch, max_new_tokens, stop, sampler, results, on_token, on_prefill):
+    slots = {i: engine.acquire() for i in batch}
+    out: Dict[int, List[int]] = {i: [] for i in batch}
+    try:
+        torch.cuda.synchronize(engine.device)
+        t0 = time.time()
+        if on_prefill:
+            on_prefill("begin", {"total_tokens": sum(len(prompts[i]) for i in batch)})
+        logits = engine.step([StepEntry(slots[i], list(prompts[i]), [len(prompts[i]) - 1]) for i in batch])
+        tokens = sampler.sample(logits, batch, [0] * len(batch)).tolist()
+        torch.cuda.synchronize(engine.device)
+        prefill_time = time.time() - t0
+        if on_prefill:
+            on_prefill("finish", {"total_time": prefill_time})
+        active = list(batch)
+        t1 = time.time()
+        while True:
+            nxt = []
+            for i, t in zip(active, tokens):
+                out[i].append(t)
+                if on_token:
+                    on_token(i, t)
+                if t in stop:
+                    reason = "stop"
+                elif len(out[i]) >= max_new_tokens:
+                    reason = "length"
+                else:
+                    nxt.append((i, t))
+                    continue
+                results[i] = Completion(out[i], reason, prefill_time, time.time() - t1)
+                engine.release(slots.pop(i))
+            if not nxt:
+                break
+            active = [i for i, _ in nxt]
+            logits = engine.step([StepEntry(slots[i], [t], [0]) for i, t in nxt])
+            tokens = sampler.sample(logits, active, [len(out[i]) for i in active]).tolist()
+    finally:
+        for s in slots.values():
+            engine.release(s)
