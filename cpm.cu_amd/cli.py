@@ -1,0 +1,213 @@
+"""Command line: ``python -m cpmcu_amd.cli --model-path DIR --prompt-text ...``.
+
+The flow is the reference's (cpmcu/cli.py:211-301): resolve the model, build the
+``LLM``, make the input ids (chat template when a tokenizer is there), size the
+storage, load the weights, generate (streaming by default), print the speeds.
+Without a tokenizer the prompt comes as token ids (--prompt-ids / --prompt-lens)
+and the output is printed as ids; --random-weights first writes a model folder
+from --config and --seed.
+"""
+from __future__ import annotations
+
+import dataclasses
+import json
+import os
+import sys
+import tempfile
+from typing import List, Optional
+
+from .args import parse_cli_args
+
+
+def log(msg: str):
+    print(f"[cpmcu_amd] {msg}", file=sys.stderr, flush=True)
+
+
+class TextTokenizer:
+    """tokenizer.json (and the chat template of tokenizer_config.json) if the model folder has them."""
+
+    def __init__(self, model_dir: str):
+        from tokenizers import Tokenizer
+        self.tok = Tokenizer.from_file(os.path.join(model_dir, "tokenizer.json"))
+        self.chat_template = None
+        self.eos_token_id = None
+        cfg_path = os.path.join(model_dir, "tokenizer_config.json")
+        if os.path.isfile(cfg_path):
+            with open(cfg_path, "r", encoding="utf-8") as f:
+                cfg = json.load(f)
+            self.chat_template = cfg.get("chat_template")
+            eos = cfg.get("eos_token")
+            if isinstance(eos, dict):
+                eos = eos.get("content")
+            if isinstance(eos, str):
+                self.eos_token_id = self.tok.token_to_id(eos)
+
+    def encode(self, text: str) -> List[int]:
+        return self.tok.encode(text).ids
+
+    def decode(self, ids: List[int]) -> str:
+        return self.tok.decode(ids, skip_special_tokens=True)
+
+    def apply_chat_template(self, content: str) -> str:
+        if not self.chat_template:
+            raise ValueError("the tokenizer has no chat template")
+        import jinja2
+        env = jinja2.Environment()
+        return env.from_string(self.chat_template).render(
+            messages=[{"role": "user", "content": content}], add_generation_prompt=True, bos_token="", eos_token="")
+
+
+def load_tokenizer(model_dir: str) -> Optional[TextTokenizer]:
+    if os.path.isfile(os.path.join(model_dir, "tokenizer.json")):
+        try:
+            return TextTokenizer(model_dir)
+        except Exception as e:  # a broken tokenizer must not stop id-based runs
+            log(f"tokenizer not usable ({e}); working with token ids")
+    return None
+
+
+def make_prompts(args, tokenizer, vocab_size: int) -> List[List[int]]:
+    """Input ids as the reference makes them (cpmcu/cli.py:47-79), or from ids / random lengths."""
+    if args.prompt_ids:
+        prompts = []
+        with open(args.prompt_ids, "r", encoding="utf-8") as f:
+            for line in f:
+                ids = [int(t) for t in line.replace(",", " ").split()]
+                if ids:
+                    prompts.append(ids)
+        if not prompts:
+            raise ValueError(f"no token ids in {args.prompt_ids}")
+        return prompts
+    if args.prompt_lens:
+        import torch
+        g = torch.Generator().manual_seed(args.seed)
+        return [[int(t) for t in torch.randint(0, vocab_size, (int(n),), generator=g)]
+                for n in args.prompt_lens.split(",")]
+    if tokenizer is None:
+        raise ValueError("the model folder has no tokenizer.json: give the prompt as token ids "
+                         "(--prompt-ids FILE) or ask for random prompts (--prompt-lens 5,11,17)")
+    if args.prompt_file:
+        if not os.path.exists(args.prompt_file):
+            raise FileNotFoundError(f"Prompt file not found: {args.prompt_file}")
+        with open(args.prompt_file, "r", encoding="utf-8") as f:
+            content = f.read().strip()
+    elif args.prompt_text:
+        content = args.prompt_text
+    else:
+        content = "Who are you"
+    prompt = content
+    if args.use_chat_template:
+        try:
+            prompt = tokenizer.apply_chat_template(content)
+        except Exception as e:
+            log(f"Failed to apply chat template: {e}, using raw prompt")
+    log(f"Input prompt: {prompt[:100]!r}{'...' if len(prompt) > 100 else ''}")
+    return [tokenizer.encode(prompt)]
+
+
+def run_generation(args):
+    from . import get_architecture
+    from .config.base import architecture_name, read_config_json
+    from .llm import LLM
+
+    model_path = args.model_path
+    if args.random_weights:
+        if not args.config:
+            raise ValueError("--random-weights needs --config <config.json>")
+        from .weights import write_model_dir
+        with open(args.config, "r", encoding="utf-8") as f:
+            raw = json.load(f)
+        cfg = get_architecture(architecture_name(raw)).config_class.from_dict(raw)
+        model_path = model_path or tempfile.mkdtemp(prefix="cpmcu_amd_random_")
+        log(f"writing random weights (seed {args.seed}) to {model_path}")
+        write_model_dir(cfg, model_path, args.seed)
+    if not model_path:
+        raise ValueError("model_path is required")
+    if not os.path.isdir(model_path):
+        raise FileNotFoundError(f"model folder not found: {model_path} (there is no download: give a local folder)")
+
+    raw = read_config_json(model_path)
+    model_type = args.model_type
+    if model_type == "auto":
+        model_type = "minicpm4" if raw.get("sparse_config") else "minicpm"
+    tokenizer = load_tokenizer(model_path)
+    llm = LLM(model_path, memory_limit=args.memory_limit, chunk_length=args.chunk_length, dtype=args.dtype,
+              cuda_graph=args.hip_graph, apply_sparse=(model_type == "minicpm4"),
+              sink_window_size=args.sink_window_size, block_window_size=args.block_window_size,
+              sparse_topk_k=args.sparse_topk_k, sparse_switch=args.sparse_switch,
+              use_compress_lse=args.use_compress_lse, temperature=args.temperature, random_seed=args.random_seed,
+              max_tokens=args.max_tokens, max_seq_len=args.max_seq_len, max_batch=args.batch)
+    llm.tokenizer = tokenizer
+    llm.perf.enabled = bool(args.perf)
+    if args.minicpm4_yarn:
+        from .config.minicpm4_yarn import MINICPM4_YARN_FACTORS
+        from .config.minicpm import RopeScaling
+        if llm.config.head_dim != 2 * len(MINICPM4_YARN_FACTORS):
+            raise ValueError(f"--minicpm4-yarn holds factors for head_dim {2 * len(MINICPM4_YARN_FACTORS)}, "
+                             f"the model has {llm.config.head_dim}")
+        rs = llm.config.rope_scaling
+        orig = rs.original_max_position_embeddings if rs else llm.config.max_position_embeddings
+        llm.config = dataclasses.replace(llm.config, rope_scaling=RopeScaling(
+            "longrope", MINICPM4_YARN_FACTORS, MINICPM4_YARN_FACTORS, orig))
+    prompts = make_prompts(args, tokenizer, llm.config.vocab_size)
+    log(f"Input tokens: {[len(p) for p in prompts]}")
+    terminators = []
+    if not args.ignore_eos:
+        terminators = list(llm.config.stop_token_ids)
+        if tokenizer is not None and tokenizer.eos_token_id is not None and tokenizer.eos_token_id not in terminators:
+            terminators.append(tokenizer.eos_token_id)
+
+    log("Initializing model storage...")
+    if args.max_tokens is None and args.batch is None:
+        llm.max_batch = len(prompts)
+    max_len = llm.init_storage()
+    log(f"Maximum context length under current memory limit: {max_len} tokens")
+    log("Loading model weights...")
+    llm.load_from_hf()
+    log("Model loading completed!")
+
+    if len(prompts) == 1 and args.use_stream:
+        tokens = []
+        prefill_time = decode_time = 0.0
+        for ev in llm.generate(prompts[0], args.num_generate, terminators, use_stream=True):
+            tokens.append(ev["token"])
+            prefill_time = max(prefill_time, ev["prefill_time"])
+            decode_time = max(decode_time, ev["decode_time"])
+            sys.stdout.write(ev["text"] if tokenizer is not None else f"{ev['token']} ")
+            sys.stdout.flush()
+        sys.stdout.write("\n")
+        stats = [(len(prompts[0]), prefill_time, len(tokens), decode_time)]
+    else:
+        outs = llm.generate(prompts, args.num_generate, terminators)
+        stats = []
+        for i, c in enumerate(outs):
+            text = tokenizer.decode(c.tokens) if tokenizer is not None else " ".join(str(t) for t in c.tokens)
+            print(f"[{i}] ({c.finish_reason}) {text}")
+            stats.append((len(prompts[i]), c.prefill_time, len(c.tokens), c.decode_time))
+    # the figures the reference prints (cpmcu/common/display.py:95-115)
+    n_prompt = sum(s[0] for s in stats)
+    t_prefill = max(s[1] for s in stats)
+    n_dec = sum(max(s[2] - 1, 0) for s in stats)
+    t_dec = max(s[3] for s in stats)
+    log(f"Prefill length: {n_prompt}  time: {t_prefill:.2f} s  speed: {n_prompt / max(t_prefill, 1e-9):.2f} tok/s")
+    log(f"Decode length: {n_dec}  time: {t_dec:.2f} s  speed: {n_dec / max(t_dec, 1e-9):.2f} tok/s")
+    if args.perf:
+        llm.print_perf_summary()
+
+
+def main(argv=None):
+    try:
+        run_generation(parse_cli_args(argv))
+    except (ValueError, FileNotFoundError) as e:
+        log(f"Configuration error: {e}")
+        sys.exit(1)
+    except RuntimeError as e:
+        log(f"Runtime error: {e}")
+        sys.exit(1)
+    except KeyboardInterrupt:
+        log("Generation interrupted by user.")
+        sys.exit(0)
+
+
+if __name__ == "__main__":
+    main()

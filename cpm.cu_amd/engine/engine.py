@@ -81,12 +81,15 @@ class Engine:
 
     # ------------------------------------------------------------------
     @classmethod
-    def from_dir(cls, model_dir: str, options: Optional[EngineOptions] = None) -> "Engine":
-        """Build the model that config.json names and load its weights from the folder."""
+    def from_dir(cls, model_dir: str, options: Optional[EngineOptions] = None,
+                 config: Optional[ModelConfig] = None) -> "Engine":
+        """Build the model that config.json names and load its weights from the folder.
+        ``config`` replaces the typed configuration read from config.json (same architecture)."""
         options = options or EngineOptions()
         raw = read_config_json(model_dir)
         arch = get_architecture(architecture_name(raw))
-        config = arch.config_class.from_dict(raw)
+        if config is None:
+            config = arch.config_class.from_dict(raw)
         tied = None
         if arch.tie_key is not None:
             tied = arch.tie_key not in checkpoint_names(model_dir)

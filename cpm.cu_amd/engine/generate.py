@@ -66,12 +66,12 @@ def plan_batches(prompt_lens: Sequence[int], max_new_tokens: int, max_batch: int
 def generate(engine: Engine, prompts: Sequence[Sequence[int]], max_new_tokens: int,
              stop_token_ids: Iterable[int] = (), temperature: float = 0.0, seed: Optional[int] = None,
              max_batch: Optional[int] = None, on_token: Optional[Callable[[int, int], None]] = None,
-             on_prefill: Optional[Callable[[str, dict], None]] = None) -> List[Completion]:
+             on_prefill: Optional[Callable[[str, dict], None]] = None, sampler=None) -> List[Completion]:
     """Generate up to max_new_tokens for every prompt (lists of token ids).
 
     ``on_token(request index, token)`` is called for each token as it is chosen."""
     stop = set(int(t) for t in stop_token_ids)
-    sampler = Sampler(temperature, seed)
+    sampler = sampler or Sampler(temperature, seed)
     max_batch = max_batch or engine.cache.max_slots
     max_batch = min(max_batch, engine.cache.max_slots)
     batches = plan_batches([len(p) for p in prompts], max_new_tokens, max_batch, engine.options.max_tokens,
@@ -82,17 +82,22 @@ def generate(engine: Engine, prompts: Sequence[Sequence[int]], max_new_tokens: i
     return results  # type: ignore[return-value]
 
 
+def _sync(engine):
+    if getattr(engine, "device", None) is not None and engine.device.type == "cuda":
+        torch.cuda.synchronize(engine.device)
+
+
 def _run_batch(engine, prompts, batch, max_new_tokens, stop, sampler, results, on_token, on_prefill):
     slots = {i: engine.acquire() for i in batch}
     out: Dict[int, List[int]] = {i: [] for i in batch}
     try:
-        torch.cuda.synchronize(engine.device)
+        _sync(engine)
         t0 = time.time()
         if on_prefill:
             on_prefill("begin", {"total_tokens": sum(len(prompts[i]) for i in batch)})
         logits = engine.step([StepEntry(slots[i], list(prompts[i]), [len(prompts[i]) - 1]) for i in batch])
         tokens = sampler.sample(logits, batch, [0] * len(batch)).tolist()
-        torch.cuda.synchronize(engine.device)
+        _sync(engine)
         prefill_time = time.time() - t0
         if on_prefill:
             on_prefill("finish", {"total_time": prefill_time})

@@ -1,0 +1,110 @@
+"""The sequence cache's bookkeeping (CPU): no slot or page lost, held twice or freed twice."""
+import random
+
+import pytest
+import torch
+
+from cpmcu_amd.cache import CacheError, CacheNeeds, SequenceCache, StateSpec, StreamSpec
+
+FULL = CacheNeeds(streams=(("k", StreamSpec(8)), ("v", StreamSpec(8))))
+CK = CacheNeeds(streams=(("k", StreamSpec(8)), ("v", StreamSpec(8)), ("ck", StreamSpec(8, every=4))))
+WIN = CacheNeeds(streams=(("k", StreamSpec(4)),), window=20)
+STATE = CacheNeeds(state=(("h", StateSpec((3, 5), torch.float32)),))
+
+
+def make(needs, max_tokens=256, max_slots=4, max_seq_len=128, page=16):
+    return SequenceCache(needs, max_tokens, max_slots, max_seq_len, page, "cpu", torch.float32)
+
+
+def test_groups_share_storage_shape_and_tables():
+    c = make([FULL, FULL, CK, WIN, STATE])
+    assert len(c.groups) == 4
+    assert c.entry_group[0] == c.entry_group[1] != c.entry_group[2]
+    v0, v2, v3, v4 = c.view(0), c.view(2), c.view(3), c.view(4)
+    assert v0.streams["k"].shape == (16, 16, 8) and v2.streams["ck"].shape == (16, 4, 8)
+    assert v0.page_table is c.view(1).page_table and v0.page_table is not v2.page_table
+    assert v0.streams["k"] is not c.view(1).streams["k"]
+    assert v3.window == 20 and v4.state["h"].shape == (4, 3, 5) and not v4.streams
+
+
+def test_positions_pages_and_release():
+    c = make([FULL])
+    s = c.acquire()
+    assert c.extend(s, 5) == 0 and c.length(s) == 5
+    assert c.extend(s, 30) == 5 and c.length(s) == 35
+    c.sync()
+    g = c.groups[0]
+    assert g.held(s) == 3 and len(g.free_pages) == 13
+    assert len(set(g.table[s, :3].tolist())) == 3
+    c.check()
+    c.release(s)
+    assert len(g.free_pages) == 16
+    c.check()
+    with pytest.raises(CacheError, match="not held"):
+        c.release(s)
+    with pytest.raises(CacheError, match="not held"):
+        c.length(s)
+
+
+def test_limits_are_refused_without_side_effects():
+    c = make([FULL], max_tokens=64, max_slots=2, max_seq_len=40)
+    a, b = c.acquire(), c.acquire()
+    with pytest.raises(CacheError, match="no free slot"):
+        c.acquire()
+    c.extend(a, 33)                       # 3 pages of 4
+    with pytest.raises(CacheError, match="longest sequence"):
+        c.extend(a, 8)
+    with pytest.raises(CacheError, match="cache is full"):
+        c.extend(b, 17)                   # needs 2 pages, 1 is free
+    assert c.length(b) == 0 and c.groups[0].held(b) == 0
+    c.extend(b, 16)
+    c.check()
+
+
+def test_a_window_group_gives_old_pages_back():
+    c = make([FULL, WIN], max_tokens=128, max_seq_len=128)
+    s = c.acquire()
+    c.extend(s, 100)
+    for _ in range(20):
+        c.extend(s, 1)
+    full, win = c.groups[c.entry_group[0]], c.groups[c.entry_group[1]]
+    assert full.held(s) == 8
+    # position 119's window reaches back to 100 -> page 6; pages 0..5 are free again
+    assert win.held(s) == 2 and win.pages[s][:6] == [-1] * 6
+    c.check()
+    c.release(s)
+    c.check()
+
+
+def test_state_is_zeroed_when_a_slot_is_taken_again():
+    c = make([STATE])
+    s = c.acquire()
+    c.view(0).state["h"][s] = 7.0
+    c.release(s)
+    t = c.acquire()
+    assert t == s and float(c.view(0).state["h"][t].abs().sum()) == 0.0
+
+
+def test_random_walk_never_loses_anything():
+    rng = random.Random(0)
+    c = make([FULL, CK, WIN], max_tokens=512, max_slots=6, max_seq_len=200)
+    live = []
+    for _ in range(600):
+        op = rng.random()
+        try:
+            if op < 0.25 and len(live) < 6:
+                live.append(c.acquire())
+            elif op < 0.8 and live:
+                c.extend(rng.choice(live), rng.randint(1, 40))
+            elif live:
+                c.release(live.pop(rng.randrange(len(live))))
+        except CacheError:
+            pass
+        c.check()
+        for g in c.groups:
+            held = [p for s in live for p in g.pages[s] if p >= 0]
+            assert len(held) == len(set(held))
+    for s in live:
+        c.release(s)
+    c.check()
+    assert all(len(g.free_pages) == g.n_pages for g in c.groups) and len(c.free_slots) == 6

@@ -1,0 +1,189 @@
+"""The engine against the plain implementation, in 32-bit and in bfloat16, under several ways of
+cutting the same requests into steps (GPU)."""
+import pytest
+import torch
+
+import plain_minicpm as plain
+import schedules
+import tiny
+
+pytestmark = pytest.mark.gpu
+
+# request lengths: prompt + teacher-forced continuation.  A has max_position 256, B 512 with
+# dense_len 64, blocks of 16 and a window of 32, so that 90/200/300 cross into the pruned regime.
+WORK = {
+    "A": {"lens": {"a": 13, "b": 19, "c": 25, "d": 120, "e": 70}, "prompt": {"a": 5, "b": 11, "c": 17, "d": 90, "e": 33}},
+    "B": {"lens": {"a": 106, "b": 216, "c": 40, "d": 300, "e": 65}, "prompt": {"a": 90, "b": 200, "c": 7, "d": 270, "e": 63}},
+}
+BATCHES = [("a", "b", "c"), ("d", "e"), ("c", "a"), ("e", "b", "d")]
+
+
+def tolerance(dtype, ref):
+    # float32: rounding of a few hundred float operations on logits of size ~1.
+    # bfloat16: activations and weights carry 8 significant bits (2^-9 relative per rounding).
+    return 2e-5 if dtype == "float32" else 0.02 * float(ref.abs().max())
+
+
+@pytest.fixture(scope="module")
+def references(model_dirs):
+    refs = {}
+    for name, d in model_dirs.items():
+        cfg, w = tiny.read_model(d)
+        reqs = {r: tiny.random_tokens(n, cfg["vocab_size"], 1000 + i) for i, (r, n) in enumerate(WORK[name]["lens"].items())}
+        refs[name] = (cfg, w, reqs, {r: plain.forward(cfg, w, t).float() for r, t in reqs.items()})
+    return refs
+
+
+_engines = {}
+
+
+def engine_for(model_dirs, name, dtype, **kw):
+    from cpmcu_amd import Engine, EngineOptions
+    key = (name, dtype, tuple(sorted(kw.items())))
+    if key not in _engines:
+        opts = dict(dtype=dtype, max_tokens=1024, max_slots=3)
+        opts.update(kw)
+        _engines[key] = Engine.from_dir(model_dirs[name], EngineOptions(**opts))
+    return _engines[key]
+
+
+def check(got, refs, dtype, what):
+    for r, ref in refs.items():
+        err = (got[r] - ref).abs()
+        tol = tolerance(dtype, ref)
+        bad = (err.max(dim=1).values > tol).nonzero().flatten()
+        assert bad.numel() == 0, (f"{what}: request {r}: first wrong position {int(bad[0])} of {ref.shape[0]} "
+                                  f"(error {float(err[bad[0]].max()):.3g} > {tol:.3g})")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_each_request_alone_and_whole(model_dirs, references, name, dtype):
+    cfg, w, reqs, refs = references[name]
+    eng = engine_for(model_dirs, name, dtype)
+    check(schedules.whole(eng, reqs), refs, dtype, "whole")
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_last_32_tokens_one_by_one(model_dirs, references, name, dtype):
+    cfg, w, reqs, refs = references[name]
+    eng = engine_for(model_dirs, name, dtype)
+    check(schedules.tail(eng, reqs, 32), refs, dtype, "tail-32")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_unequal_batches_one_after_another(model_dirs, references, name, dtype):
+    cfg, w, reqs, refs = references[name]
+    eng = engine_for(model_dirs, name, dtype)       # 3 slots: every batch takes slots that an earlier one gave back
+    got = schedules.batched(eng, reqs, WORK[name]["prompt"], BATCHES[:2])
+    check(got, refs, dtype, "batched")
+    got = schedules.batched(eng, reqs, WORK[name]["prompt"], BATCHES[2:])
+    check(got, refs, dtype, "batched, slots used again")
+    eng.cache.check()
+    assert not eng.cache.live
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_cutting_changes_nothing_beyond_rounding(model_dirs, references, name):
+    """32-bit: whole, token by token and batched agree far below the tolerance against the plain implementation."""
+    cfg, w, reqs, refs = references[name]
+    eng = engine_for(model_dirs, name, "float32")
+    a = schedules.whole(eng, reqs)
+    b = schedules.tail(eng, reqs, 32)
+    c = schedules.batched(eng, reqs, WORK[name]["prompt"], BATCHES[:2])
+    for r in reqs:
+        assert float((a[r] - b[r]).abs().max()) < 2e-6 and float((a[r] - c[r]).abs().max()) < 2e-6
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_small_forward_passes_equal_one_large(model_dirs, references, name, dtype):
+    """A step cut into forward passes of 7 tokens (sequences split across passes) gives the same logits."""
+    cfg, w, reqs, refs = references[name]
+    eng = engine_for(model_dirs, name, dtype, max_step_tokens=7)
+    check(schedules.whole(eng, reqs), refs, dtype, "chunks of 7")
+    got = schedules.batched(eng, reqs, WORK[name]["prompt"], BATCHES[:2])
+    check(got, refs, dtype, "batched in chunks of 7")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_long_decoding_and_first_tokens(model_dirs, references, name, dtype):
+    cfg, w, _, _ = references[name]
+    n = 250 if name == "A" else 330
+    toks = tiny.random_tokens(n, cfg["vocab_size"], 77)
+    ref = plain.forward(cfg, w, toks).float()
+    eng = engine_for(model_dirs, name, dtype)
+    got = schedules.tail(eng, {"x": toks}, n - 1)["x"]           # a one-token prompt, then everything one by one
+    check({"x": got}, {"x": ref}, dtype, "long decoding")
+    # the very first tokens of a sequence, each way
+    for k in (1, 2, 3):
+        s = eng.acquire()
+        from cpmcu_amd import StepEntry
+        lg = eng.step([StepEntry(s, toks[:k], list(range(k)))]).cpu()
+        eng.release(s)
+        check({"x": lg}, {"x": ref[:k]}, dtype, f"first {k} tokens")
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_through_the_entry_point(model_dirs, references, name):
+    from cpmcu_amd.llm import LLM
+    cfg, w, reqs, _ = references[name]
+    prompts = [reqs["a"][:9], reqs["b"][:70] if name == "B" else reqs["b"][:14], reqs["c"][:3]]
+    want = [plain.greedy(cfg, w, p, 7) for p in prompts]
+    llm = LLM(model_dirs[name], dtype="float32", max_tokens=1024, max_batch=2, apply_sparse=(name == "B"))
+    llm.init_storage()
+    llm.load_from_hf()
+    tokens, decode_time, prefill_time = llm.generate(torch.tensor(prompts[0], dtype=torch.int32), generation_length=7)
+    assert tokens == want[0] and decode_time > 0 and prefill_time > 0
+    outs = llm.generate(prompts, generation_length=7)               # 3 requests, 2 slots: two batches
+    assert [o.tokens for o in outs] == want
+    # a stop token ends its sequence and is returned
+    stop = want[1][2]
+    outs = llm.generate(prompts, generation_length=7, terminators=[stop])
+    for o, wnt in zip(outs, want):
+        cut = wnt.index(stop) + 1 if stop in wnt else len(wnt)
+        assert o.tokens == wnt[:cut] and o.finish_reason == ("stop" if stop in wnt else "length")
+    # streaming yields the same tokens
+    ev = list(llm.generate(prompts[2], generation_length=7, use_stream=True))
+    assert [e["token"] for e in ev] == want[2] and ev[-1]["is_finished"]
+    # bfloat16 through the same entry point: tokens are those of its own replayed logits
+    llm16 = LLM(model_dirs[name], dtype="bfloat16", max_tokens=1024, apply_sparse=(name == "B"))
+    llm16.init_storage()
+    llm16.load_from_hf()
+    toks16, _, _ = llm16.generate(prompts[0], generation_length=7)
+    from cpmcu_amd import StepEntry
+    seq = prompts[0] + toks16[:-1]
+    s = llm16.engine.acquire()
+    lg = llm16.engine.step([StepEntry(s, seq, list(range(len(prompts[0]) - 1, len(seq))))])
+    llm16.engine.release(s)
+    margin = lg.topk(2, dim=-1).values
+    sure = (margin[:, 0] - margin[:, 1]) > 0.02
+    assert [t for t, ok in zip(lg.argmax(-1).tolist(), sure.tolist()) if ok] == [t for t, ok in zip(toks16, sure.tolist()) if ok]
+
+
+def test_steps_that_cannot_run_are_refused_and_change_nothing(model_dirs):
+    from cpmcu_amd import StepEntry, StepError
+    eng = engine_for(model_dirs, "A", "float32")
+    s = eng.acquire()
+    with pytest.raises(StepError, match="outside the vocabulary"):
+        eng.step([StepEntry(s, [1, 512], [0])])
+    with pytest.raises(StepError, match="at least one token"):
+        eng.step([StepEntry(s, [], [])])
+    with pytest.raises(StepError, match="wanted place"):
+        eng.step([StepEntry(s, [1, 2], [2])])
+    with pytest.raises(StepError, match="longest sequence"):
+        eng.step([StepEntry(s, [1] * 257, [])])
+    with pytest.raises(StepError, match="twice"):
+        eng.step([StepEntry(s, [1], []), StepEntry(s, [2], [])])
+    with pytest.raises(StepError, match="not held"):
+        eng.step([StepEntry(2 if s != 2 else 1, [1], [])])
+    with pytest.raises(StepError, match="at least one sequence"):
+        eng.step([])
+    assert eng.length(s) == 0
+    assert eng.step([StepEntry(s, [1, 2, 3], [])]) is None and eng.length(s) == 3
+    eng.release(s)
+    eng.cache.check()

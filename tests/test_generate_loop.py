@@ -1,0 +1,118 @@
+"""The generation loop's decisions, with a stand-in engine and sampler (CPU)."""
+import pytest
+import torch
+
+from cpmcu_amd.engine.generate import generate, plan_batches
+
+
+class FakeCache:
+    page_size = 16
+
+    def __init__(self, slots):
+        self.max_slots = slots
+
+
+class FakeEngine:
+    """Logits that make greedy emit (last token + 1) % vocab; records every step."""
+
+    def __init__(self, vocab=50, slots=4, max_tokens=4096, max_seq_len=512):
+        class O:
+            pass
+        self.options = O()
+        self.options.max_tokens = max_tokens
+        self.cache = FakeCache(slots)
+        self.max_seq_len = max_seq_len
+        self.device = torch.device("cpu")
+        self.vocab = vocab
+        self.free = list(range(slots))
+        self.held = {}
+        self.log = []
+
+    def acquire(self):
+        s = self.free.pop(0)
+        self.held[s] = 0
+        return s
+
+    def release(self, s):
+        assert s in self.held, "slot released twice"
+        del self.held[s]
+        self.free.append(s)
+
+    def step(self, entries):
+        self.log.append([(e.slot, list(e.tokens)) for e in entries])
+        rows = []
+        for e in entries:
+            assert e.slot in self.held
+            self.held[e.slot] += len(e.tokens)
+            for w in e.want:
+                row = torch.zeros(self.vocab)
+                row[(e.tokens[w] + 1) % self.vocab] = 1.0
+                rows.append(row)
+        return torch.stack(rows)
+
+
+class ArgmaxSampler:
+    def sample(self, logits, request_ids, steps):
+        self.last = (list(request_ids), list(steps))
+        return logits.argmax(-1).to(torch.int32)
+
+
+def test_unequal_prompts_stop_tokens_and_early_leavers():
+    eng = FakeEngine()
+    prompts = [[1, 2, 3], [10], [20, 21, 22, 23, 24]]
+    outs = generate(eng, prompts, max_new_tokens=6, stop_token_ids=[13, 27], sampler=ArgmaxSampler())
+    assert outs[0].tokens == [4, 5, 6, 7, 8, 9] and outs[0].finish_reason == "length"
+    assert outs[1].tokens == [11, 12, 13] and outs[1].finish_reason == "stop"       # the stop token is returned
+    assert outs[2].tokens == [25, 26, 27] and outs[2].finish_reason == "stop"
+    # step 0 carries the whole prompts; then one token each; finished sequences leave the batch
+    assert [len(t) for _, t in eng.log[0]] == [3, 1, 5]
+    assert all(len(t) == 1 for step in eng.log[1:] for _, t in step)
+    assert [len(step) for step in eng.log] == [3, 3, 3, 1, 1, 1]
+    assert not eng.held and sorted(eng.free) == [0, 1, 2, 3]
+    # the first sampled token counts toward the length: 6 tokens need 5 single-token steps
+    assert len(eng.log) == 6
+
+
+def test_first_token_can_already_stop():
+    eng = FakeEngine()
+    outs = generate(eng, [[4], [8]], max_new_tokens=5, stop_token_ids=[5], sampler=ArgmaxSampler())
+    assert outs[0].tokens == [5] and outs[0].finish_reason == "stop"
+    assert outs[1].tokens == [9, 10, 11, 12, 13]
+    assert [len(s) for s in eng.log] == [2, 1, 1, 1, 1]
+
+
+def test_more_requests_than_slots_run_as_batches_one_after_another():
+    eng = FakeEngine(slots=2)
+    prompts = [[i] for i in range(5)]
+    s = ArgmaxSampler()
+    outs = generate(eng, prompts, max_new_tokens=2, sampler=s)
+    assert [o.tokens for o in outs] == [[i + 1, i + 2] for i in range(5)]
+    assert [len(step) for step in eng.log] == [2, 2, 2, 2, 1, 1]                      # prompt step, then one decode step
+    assert [t for _, t in eng.log[2]] == [[2], [3]] and [t for _, t in eng.log[4]] == [[4]]
+    assert {slot for step in eng.log for slot, _ in step} == {0, 1}                   # slots are used again
+    assert not eng.held
+    assert s.last == ([4], [1])                                                       # request id and its step
+
+
+def test_plan_batches_respects_slots_cache_and_order():
+    assert plan_batches([5, 11, 17], 8, 8, 4096, 64, 256) == [[0, 1, 2]]
+    assert plan_batches([5, 11, 17, 3], 8, 2, 4096, 64, 256) == [[0, 1], [2, 3]]
+    # 100+29 tokens = 3 pages of 64 each; a cache of 320 tokens (5 pages) holds one such request at a time
+    assert plan_batches([100, 100, 10], 30, 8, 320, 64, 256) == [[0], [1, 2]]
+    with pytest.raises(ValueError, match="longest sequence"):
+        plan_batches([250], 10, 8, 4096, 64, 256)
+    with pytest.raises(ValueError, match="do not fit the cache"):
+        plan_batches([200], 10, 8, 128, 64, 256)
+    with pytest.raises(ValueError, match="empty"):
+        plan_batches([3, 0], 10, 8, 4096, 64, 256)
+
+
+def test_a_failing_step_gives_the_slots_back():
+    eng = FakeEngine()
+
+    def boom(entries):
+        raise RuntimeError("kernel refused")
+    eng.step = boom
+    with pytest.raises(RuntimeError):
+        generate(eng, [[1], [2]], 3, sampler=ArgmaxSampler())
+    assert not eng.held
