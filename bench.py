@@ -1,0 +1,176 @@
+#!/usr/bin/env python3
+"""Benchmark: decode tokens/s of a MiniCPM4-8B-shaped model with random weights on one MI355X.
+
+python bench.py --gpus 1 --steps K --warmup W   prints ONE JSON line.  A step is one decode step
+of the whole batch (default batch 8 at context 4,096, the sizes of BASELINE.json configs[2]).
+The same line carries the prefill of 2,048 tokens, the decode step's memory roofline and
+decode at batch 1 and 64.  Weights are random (N(0, 0.02)), token ids uniform: nothing is
+downloaded.  The engine runs on one GPU only: for --gpus > 1 it says so and exits with 2.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+
+def config_8b(layers=None):
+    import torch
+    g = torch.Generator().manual_seed(1234)
+    fac = lambda: [float(x) for x in (1.0 + 3.0 * torch.rand(64, generator=g, dtype=torch.float64))]
+    return {
+        "architectures": ["MiniCPMForCausalLM"], "model_type": "minicpm",
+        "num_hidden_layers": layers or 32, "hidden_size": 4096, "num_attention_heads": 32, "num_key_value_heads": 2,
+        "head_dim": 128, "intermediate_size": 16384, "vocab_size": 73448, "rms_norm_eps": 1e-6, "rope_theta": 10000.0,
+        "max_position_embeddings": 32768,
+        "rope_scaling": {"rope_type": "longrope", "short_factor": fac(), "long_factor": fac(),
+                         "original_max_position_embeddings": 32768},
+        "scale_emb": 12, "dim_model_base": 256, "scale_depth": 1.4, "tie_word_embeddings": False,
+        "hidden_act": "silu", "torch_dtype": "bfloat16",
+    }
+
+
+def weight_bytes_per_step(cfg, esize):
+    """Bytes of weights a decode step reads once: every layer's matrices and norms, final norm, lm_head."""
+    H, I, V, L = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size, cfg.num_hidden_layers
+    qkv = (cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * cfg.head_dim * H
+    o = H * cfg.num_attention_heads * cfg.head_dim
+    per_layer = (qkv + o + 3 * H * I) * esize + 2 * H * 4
+    return L * per_layer + V * H * esize + H * 4
+
+
+def kv_bytes_per_token(cfg, esize):
+    return cfg.num_hidden_layers * 2 * cfg.num_key_value_heads * cfg.head_dim * esize
+
+
+def prefill_flops(cfg, n):
+    H, I, V, L = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size, cfg.num_hidden_layers
+    nh, nkv, hd = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    lin = L * ((nh + 2 * nkv) * hd * H + H * nh * hd + 3 * H * I)
+    attn = L * nh * hd * 2 * (n * (n + 1) // 2) * 2          # q.k and p.v over the causal half
+    return 2 * n * lin + attn + 2 * V * H
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model's 32 (named in config)")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--hip-graph", type=int, default=1)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported (no multi-GPU path exists)")
+        sys.exit(2)
+
+    import torch
+    import cpmcu_amd
+    from cpmcu_amd import Engine, EngineOptions, StepEntry
+    from cpmcu_amd.config import MiniCPMConfig
+    from cpmcu_amd.weights import random_tensors
+
+    dev = "cuda:0"
+    raw = config_8b(args.layers)
+    cfg = MiniCPMConfig.from_dict(raw)
+    esize = 2 if args.dtype == "bfloat16" else 4
+    t0 = time.time()
+    tensors = random_tensors(cfg, seed=0, device=dev)
+    max_b = max(args.batch, 1 if args.no_points else 64)
+    per_seq = -(-(args.context + args.steps + args.warmup + 64) // 64) * 64
+    eng = Engine.from_tensors(cfg, tensors, EngineOptions(
+        dtype=args.dtype, max_tokens=max(max_b * per_seq, args.prefill_tokens + 64), max_slots=max_b,
+        max_step_tokens=max(args.prefill_tokens, 2048), device=dev, hip_graph=bool(args.hip_graph)))
+    del tensors
+    torch.cuda.synchronize()
+    print(f"[bench] model ready in {time.time() - t0:.1f} s: {cfg.num_hidden_layers} layers, "
+          f"{weight_bytes_per_step(cfg, esize) / 1e9:.2f} GB of weights a step", file=sys.stderr, flush=True)
+    g = torch.Generator().manual_seed(7)
+    rand_ids = lambda n: [int(t) for t in torch.randint(0, cfg.vocab_size, (n,), generator=g)]
+
+    def fill_context(batch, context):
+        """Slots that hold `context - 1` tokens of random keys and values: the state a decode step at that
+        context length starts from (the timed steps do all of their own work; what filled the cache is not timed)."""
+        slots = [eng.acquire() for _ in range(batch)]
+        for s in slots:
+            eng.cache.extend(s, context - 1)
+        eng.cache.sync()
+        for grp in eng.cache.groups:
+            for st in grp.storage.values():
+                for t in st.values():
+                    t.normal_(0.0, 0.5)
+        return slots
+
+    def decode_run(batch, context, steps, warmup):
+        slots = fill_context(batch, context)
+        toks = [rand_ids(batch) for _ in range(steps + warmup)]
+        for i in range(warmup):
+            eng.step([StepEntry(s, [toks[i][j]], [0]) for j, s in enumerate(slots)])
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for i in range(warmup, warmup + steps):
+            eng.step([StepEntry(s, [toks[i][j]], [0]) for j, s in enumerate(slots)])
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t
+        for s in slots:
+            eng.release(s)
+        return dt
+
+    dt = decode_run(args.batch, args.context, args.steps, args.warmup)
+    ms_step = dt / args.steps * 1e3
+    value = args.batch * args.steps / dt
+    step_bytes = weight_bytes_per_step(cfg, esize) + args.batch * (args.context + args.steps // 2) * kv_bytes_per_token(cfg, esize)
+    achieved = step_bytes / (ms_step * 1e-3) / 1e9
+    rec = {
+        "metric": "MiniCPM4-8B decode tok/s @ batch 8, context 4096 (bf16, random weights)",
+        "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+        "config": {"model": "MiniCPM4-8B shape, random weights N(0,0.02)", "layers": cfg.num_hidden_layers,
+                   "layers_full_model": 32, "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads,
+                   "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+                   "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size, "global_batch": args.batch,
+                   "seq_len": args.context, "prefill_tokens": args.prefill_tokens, "parallelism": "1gpu",
+                   "page_size": 64, "hip_graph": bool(args.hip_graph)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+    }
+    if not args.no_prefill:
+        n = args.prefill_tokens
+        times = []
+        for it in range(3):
+            s = eng.acquire()
+            ids = rand_ids(n)
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            eng.step([StepEntry(s, ids, [n - 1])])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t)
+            eng.release(s)
+        pt = min(times[1:])
+        peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
+        rec["prefill"] = {"value": round(n / pt, 1), "tokens": n, "ms": round(pt * 1e3, 3),
+                          "frac": round(prefill_flops(cfg, n) / pt / peak, 4)}
+    if not args.no_points:
+        pts = {}
+        for b in (1, 64):
+            st = max(args.steps // 2, 8)
+            d = decode_run(b, args.context, st, max(args.warmup // 2, 3))
+            pts[f"decode_b{b}"] = round(b * st / d, 2)
+        rec["points"] = pts
+    print(json.dumps(rec), flush=True)
+
+
+if __name__ == "__main__":
+    main()
