@@ -68,10 +68,12 @@ __global__ __launch_bounds__(64) void attention_paged_kernel(
             for (int jj = 0; jj < cnt; ++jj) {
                 const float pj = __shfl(p, jj, 64);
                 const int rj = __shfl(row, jj, 64);
-                const T* vr = vpool + (long)rj * kv_stride + (long)g * hd;
+                // values are transposed inside a page: [page][kv head][d][token of the page]
+                const int pg = rj / pv.page_size;
+                const T* vr = vpool + ((long)pg * kv_stride + (long)g * hd) * pv.page_size + (rj - pg * pv.page_size);
                 for (int i = 0; i < nd; ++i) {
                     const int d = lane + 64 * i;
-                    if (d < hd) acc[i] += pj * to_f32(vr[d]);
+                    if (d < hd) acc[i] += pj * to_f32(vr[(long)d * pv.page_size]);
                 }
             }
         }
@@ -109,5 +111,210 @@ extern "C" const char* cpmcu_attention_plain(const void* q, void* out, int dtype
     else
         CPMCU_FAIL("attention: unknown dtype %d", dtype);
     CPMCU_LAUNCH_CHECK("attention_plain");
+    return nullptr;
+}
+
+// ===========================================================================
+// bf16 attention on the matrix cores, for prompts and single tokens alike.
+//
+// One wavefront owns one query token, one kv head and up to 16 of that kv
+// head's query heads (the 16:1 grouping of MiniCPM4-8B fills an MFMA tile
+// exactly), and a share of that token's keys (split-KV for decode steps, where
+// few tokens must fill 256 CUs).  Keys are visited in chunks of 32:
+//   S^T = K . Q^T      A = 16 keys x head_dim straight from the cache rows,
+//                      B = Q^T held in registers for the whole kernel
+//   P^T = exp2(S^T*c - m) in float, per head (a D column), running max/sum
+//   O^T += V^T . P^T   A = V^T: 16 d x 32 keys, one 16-byte load a lane because
+//                      values are stored transposed inside a page
+// The two key tiles of a chunk take keys {8g..8g+3} and {8g+4..8g+7} of every
+// group of 8 so that a lane's 8 probabilities are 8 consecutive keys, the order
+// the V^T vector has.  No LDS and no barrier is used.
+// Output: out (bf16) when n_splits == 1, else unnormalised partial results
+// part_o[token][head][split][d], part_ml[token][head][split] = (max, sum) for
+// attention_combine_kernel.
+// (reference: src/flash_attn/src/flash_fwd_kernel.h:580-1171 is its kernel of
+// one query token x 16 grouped heads; split and combine :1175-1766, :2320-2501)
+// ===========================================================================
+typedef __bf16 abf16x8_t __attribute__((ext_vector_type(8)));
+typedef float afloatx4_t __attribute__((ext_vector_type(4)));
+
+template <int HD>
+__global__ __launch_bounds__(64) void attention_mfma_kernel(
+    const bf16_t* __restrict__ q, bf16_t* __restrict__ out, float* __restrict__ part_o, float2* __restrict__ part_ml,
+    const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vtpool, PagedView pv,
+    const int* __restrict__ positions, const int* __restrict__ tok_slot, int nh, int nkv, float scale_log2e,
+    const int* __restrict__ sel_blocks, const int* __restrict__ sel_count, int max_sel, int block_size, int n_splits) {
+    constexpr int KSTEPS = (HD + 31) / 32;
+    constexpr int DT = HD / 16;
+    const int t = blockIdx.x;
+    const int kvh = blockIdx.y % nkv, ht = blockIdx.y / nkv;
+    const int split = blockIdx.z;
+    const int lane = threadIdx.x, n = lane & 15, g = lane >> 4;
+    const int G = nh / nkv;
+    const int head = kvh * G + ht * 16 + n;            // the head this lane's D column belongs to
+    const bool head_ok = ht * 16 + n < G;
+    const int pos = positions[t], slot = tok_slot[t];
+    const int* ptab = pv.page_table + (long)slot * pv.table_width;
+
+    abf16x8_t qf[KSTEPS];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+        abf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+        const int d = ks * 32 + g * 8;
+        if (head_ok && d < HD) v = *(const abf16x8_t*)(q + ((long)t * nh + head) * HD + d);
+        qf[ks] = v;
+    }
+
+    // which chunks of 32 keys are this wavefront's
+    const int* sel = nullptr;
+    int total_chunks = pos / 32 + 1;
+    int cpb = 1;
+    if (sel_count) {
+        const int c = sel_count[(long)t * nkv + kvh];
+        if (c >= 0) {
+            sel = sel_blocks + ((long)t * nkv + kvh) * max_sel;
+            cpb = block_size / 32;
+            total_chunks = c * cpb;
+        }
+    }
+    const int per_split = (total_chunks + n_splits - 1) / n_splits;
+    const int c0 = split * per_split, c1 = min(c0 + per_split, total_chunks);
+
+    afloatx4_t acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[dt] = afloatx4_t{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+    const long kv_width = (long)nkv * HD;
+
+    for (int c = c0; c < c1; ++c) {
+        const int key0 = sel ? sel[c / cpb] * block_size + (c % cpb) * 32 : c * 32;
+        if (key0 > pos) continue;
+        const int page = ptab[key0 / pv.page_size];
+        const int po = key0 % pv.page_size;
+        // S^T for two tiles of 16 keys: key slot r of tile u is key0 + r + 4*(r/4) + 4u
+        afloatx4_t st[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            st[u] = afloatx4_t{0.f, 0.f, 0.f, 0.f};
+            const long krow = (long)page * pv.page_size + po + n + 4 * (n >> 2) + 4 * u;
+            const bf16_t* kp = kpool + krow * kv_width + (long)kvh * HD + g * 8;
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks) {
+                abf16x8_t kf = {0, 0, 0, 0, 0, 0, 0, 0};
+                if (ks * 32 + g * 8 < HD) kf = *(const abf16x8_t*)(kp + ks * 32);
+                st[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], st[u], 0, 0, 0);
+            }
+        }
+        // lane (head n, g): st[u][i] is key key0 + 8g + 4u + i
+        float s[8];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = key0 + 8 * g + 4 * u + i;
+                const float v = key <= pos ? st[u][i] * scale_log2e : -INFINITY;
+                s[u * 4 + i] = v;
+                mx = fmaxf(mx, v);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m, mx);
+        const float corr = exp2f(m - m_new);
+        float rs = 0.f;
+        abf16x8_t pb;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float p = exp2f(s[j] - m_new);
+            rs += p;
+            pb[j] = (__bf16)p;
+        }
+        rs += __shfl_xor(rs, 16, 64);
+        rs += __shfl_xor(rs, 32, 64);
+        l = l * corr + rs;
+        m = m_new;
+        // O^T += V^T . P^T ; A operand: lane (d row n, g) holds V^T[d][key0 + 8g .. +8]
+        const bf16_t* vp = vtpool + (((long)page * nkv + kvh) * HD + n) * pv.page_size + po + g * 8;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const abf16x8_t vf = *(const abf16x8_t*)(vp + (long)dt * 16 * pv.page_size);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[dt][i] *= corr;
+            acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb, acc[dt], 0, 0, 0);
+        }
+    }
+    if (!head_ok) return;
+    // lane (head n, g): acc[dt][i] is O[head][dt*16 + 4g + i]
+    if (n_splits == 1) {
+        const float inv = 1.0f / l;
+        bf16_t* o = out + ((long)t * nh + head) * HD;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o[dt * 16 + 4 * g + i] = f32_to_bf16(acc[dt][i] * inv);
+    } else {
+        const long idx = ((long)t * nh + head) * n_splits + split;
+        float* o = part_o + idx * HD;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) *(afloatx4_t*)(o + dt * 16 + 4 * g) = acc[dt];
+        if (g == 0) part_ml[idx] = make_float2(m, l);
+    }
+}
+
+// out[token][head][:] = sum_s 2^(m_s - m) o_s / sum_s 2^(m_s - m) l_s   (splits without keys have l = 0)
+__global__ void attention_combine_kernel(const float* __restrict__ part_o, const float2* __restrict__ part_ml,
+                                         bf16_t* __restrict__ out, int hd, int n_splits) {
+    const long row = blockIdx.x;             // token * nh + head
+    const float2* ml = part_ml + row * n_splits;
+    float m = -INFINITY;
+    for (int s = 0; s < n_splits; ++s)
+        if (ml[s].y > 0.f) m = fmaxf(m, ml[s].x);
+    float denom = 0.f;
+    for (int s = 0; s < n_splits; ++s)
+        if (ml[s].y > 0.f) denom += exp2f(ml[s].x - m) * ml[s].y;
+    const float inv = 1.0f / denom;
+    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+        float a = 0.f;
+        for (int s = 0; s < n_splits; ++s)
+            if (ml[s].y > 0.f) a += exp2f(ml[s].x - m) * part_o[(row * n_splits + s) * hd + d];
+        out[row * hd + d] = f32_to_bf16(a * inv);
+    }
+}
+
+extern "C" const char* cpmcu_attention_mfma(const void* q, void* out, float* part_o, float* part_ml, int n, int nh,
+                                            int nkv, int hd, float scale, const void* kpool, const void* vtpool,
+                                            const int* page_table, int table_width, int page_size,
+                                            const int* positions, const int* tok_slot, const int* sel_blocks,
+                                            const int* sel_count, int max_sel, int block_size, int n_splits,
+                                            hipStream_t stream) {
+    CPMCU_REQUIRE(n > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_mfma: bad shape n=%d heads=%d kv_heads=%d", n, nh, nkv);
+    CPMCU_REQUIRE(hd == 16 || hd == 32 || hd == 64 || hd == 128,
+                  "attention_mfma: head_dim %d has no matrix-core kernel (16, 32, 64, 128 have; the plain kernel takes the rest)", hd);
+    CPMCU_REQUIRE(page_size % 32 == 0, "attention_mfma: a cache page of %d tokens is not a multiple of 32", page_size);
+    CPMCU_REQUIRE(!sel_count || (sel_blocks && max_sel > 0 && block_size > 0 && block_size % 32 == 0),
+                  "attention_mfma: key blocks of %d tokens are not a multiple of 32", block_size);
+    CPMCU_REQUIRE(n_splits >= 1 && n_splits <= 65535 && (n_splits == 1 || (part_o && part_ml)), "attention_mfma: bad split %d", n_splits);
+    const int G = nh / nkv;
+    const int HT = (G + 15) / 16;
+    CPMCU_REQUIRE((long)nkv * HT <= 65535, "attention_mfma: too many head tiles");
+    PagedView pv{page_table, table_width, page_size};
+    dim3 grid(n, nkv * HT, n_splits);
+    const float sl = scale * 1.4426950408889634f;
+#define LAUNCH(HDv)                                                                                                \
+    attention_mfma_kernel<HDv><<<grid, 64, 0, stream>>>((const bf16_t*)q, (bf16_t*)out, part_o, (float2*)part_ml,  \
+                                                        (const bf16_t*)kpool, (const bf16_t*)vtpool, pv, positions, \
+                                                        tok_slot, nh, nkv, sl, sel_blocks, sel_count, max_sel,    \
+                                                        block_size, n_splits)
+    if (hd == 16) LAUNCH(16);
+    else if (hd == 32) LAUNCH(32);
+    else if (hd == 64) LAUNCH(64);
+    else LAUNCH(128);
+#undef LAUNCH
+    CPMCU_LAUNCH_CHECK("attention_mfma");
+    if (n_splits > 1) {
+        attention_combine_kernel<<<(unsigned)((long)n * nh), hd >= 64 ? 64 : hd, 0, stream>>>(
+            part_o, (const float2*)part_ml, (bf16_t*)out, hd, n_splits);
+        CPMCU_LAUNCH_CHECK("attention_combine");
+    }
     return nullptr;
 }

@@ -130,7 +130,8 @@ extern "C" const char* cpmcu_silu_mul(const void* gu, void* out, int dtype, int 
 // to `q_out` (row stride nh*hd).  theta = pos * inv_freq[c];
 // (a, b) = (x[c], x[c+hd/2]) -> (a cos - b sin, a sin + b cos), cos and sin
 // times `mscale` (reference: src/model/rotary.cuh:7-34; cache rows
-// src/model/attn.cuh:14-21).  inv_freq null: no rotation.
+// src/model/attn.cuh:14-21).  inv_freq null: no rotation.  Keys lie [token][kv head][d];
+// values lie transposed inside their page, [page][kv head][d][token of the page].
 // ---------------------------------------------------------------------------
 template <typename IT, typename T>
 __global__ void rope_store_kernel(const IT* __restrict__ qkv, long width, int nparts, long part_stride,
@@ -171,9 +172,13 @@ __global__ void rope_store_kernel(const IT* __restrict__ qkv, long width, int np
         }
     }
     if (write_kv) {
+        // values are kept transposed inside a page, [page][kv head][d][token of the page], so that
+        // attention reads, for one d, the values of consecutive keys as one vector
         const long voff = (long)(nh + nkv) * hd;
-        T* dst = vpool + kv_row * (long)nkv * hd;
-        for (int i = threadIdx.x; i < nkv * hd; i += blockDim.x) dst[i] = from_f32<T>(load(voff + i));
+        const long page = kv_row / pv.page_size;
+        const int in_page = (int)(kv_row - page * pv.page_size);
+        T* dst = vpool + page * (long)pv.page_size * nkv * hd + in_page;
+        for (int i = threadIdx.x; i < nkv * hd; i += blockDim.x) dst[(long)i * pv.page_size] = from_f32<T>(load(voff + i));
     }
 }
 

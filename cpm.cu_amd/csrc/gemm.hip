@@ -76,3 +76,210 @@ extern "C" const char* cpmcu_gemm_nt_plain(const void* X, long ldx, const void* 
     CPMCU_LAUNCH_CHECK("gemm_nt_plain");
     return nullptr;
 }
+
+// ===========================================================================
+// Skinny product for decode steps (bf16, at most 64 rows of X):
+//   Y[m,N] = alpha * X[m,K] . W[N,K]^T
+// The step is bound by reading W once from HBM, so W streams from global memory
+// straight into MFMA operand registers (v_mfma_f32_16x16x32_bf16: 16 rows of W
+// by 32 of K an instruction), four K-blocks of 128 ahead of their use, while X
+// (small, shared by all rows of W) is staged through LDS 512 columns at a time.
+// For the i-th MFMA of a K-block of 128 the lane group g = lane/16 holds columns
+// [32i + 8g, 32i + 8g + 8) of its row, so the four lanes of a row read 64
+// contiguous bytes an instruction; X is read from LDS with the same mapping.
+//   MODE 0: Y (float or bf16) = alpha * product
+//   MODE 1: float partial sums of a K-split, part[blockIdx.y][m][N]
+//   MODE 2: rows come in pairs (gate j, up I+j): Y[m][j] = silu(gate) * up  (bf16)
+// ===========================================================================
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float floatx4_t __attribute__((ext_vector_type(4)));
+
+#define SK_XC 512            // K columns of X staged at a time
+#define SK_XS (SK_XC + 8)    // LDS row stride in elements (16 bytes of padding)
+
+template <int MT, int MODE, typename OT, int SPW, int NW>
+__global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ X, long ldx,
+                                                             const bf16_t* __restrict__ W, long ldw,
+                                                             OT* __restrict__ Y, long ldy, int M, int N, int K, int KS,
+                                                             float alpha, int I, long part_stride) {
+    static_assert(MODE != 2 || SPW == 2, "gated output pairs a gate strip with an up strip");
+    constexpr int NT = NW * 64;
+    constexpr int XV = MT * 16 * 64 / NT;     // 16-byte vectors of X a thread stages per chunk
+    __shared__ __attribute__((aligned(16))) bf16_t xs[MT * 16 * SK_XS];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int r = lane & 15, g = lane >> 4;
+    const int k_begin = blockIdx.y * KS;
+    const int k_end = min(K, k_begin + KS);
+    const int nkb = (k_end - k_begin + 127) / 128;
+
+    // the strips of 16 rows of W this wave owns
+    int out_base[SPW];
+    const bf16_t* wp[SPW];
+    if (MODE == 2) {
+        const int p = blockIdx.x * (NW * 16) + wave * 16;
+        out_base[0] = out_base[SPW - 1] = p;
+        const int pr = min(p + r, I - 1);
+        wp[0] = W + (long)pr * ldw;
+        wp[SPW - 1] = W + ((long)I + pr) * ldw;
+    } else {
+        const int n0 = blockIdx.x * (NW * SPW * 16) + wave * (SPW * 16);
+#pragma unroll
+        for (int s = 0; s < SPW; ++s) {
+            out_base[s] = n0 + s * 16;
+            wp[s] = W + (long)min(n0 + s * 16 + r, N - 1) * ldw;
+        }
+    }
+
+    bf16x8_t a[4][SPW][4];
+    auto load_w = [&](int kb, bf16x8_t (&dst)[SPW][4]) {
+        const int k = k_begin + kb * 128 + g * 8;
+#pragma unroll
+        for (int s = 0; s < SPW; ++s)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                bf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+                if (kb < nkb && k + i * 32 < k_end) v = __builtin_nontemporal_load((const bf16x8_t*)(wp[s] + k + i * 32));
+                dst[s][i] = v;
+            }
+    };
+    bf16x8_t xr[XV];
+    auto load_x = [&](int chunk) {
+        const int k0 = k_begin + chunk * SK_XC;
+#pragma unroll
+        for (int v = 0; v < XV; ++v) {
+            const int idx = tid + v * NT;
+            const int xrow = idx >> 6, vec = idx & 63;
+            bf16x8_t val = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (xrow < M && k0 + vec * 8 < k_end) val = *(const bf16x8_t*)(X + (long)xrow * ldx + k0 + vec * 8);
+            xr[v] = val;
+        }
+    };
+    auto store_x = [&]() {
+#pragma unroll
+        for (int v = 0; v < XV; ++v) {
+            const int idx = tid + v * NT;
+            const int xrow = idx >> 6, vec = idx & 63;
+            *(bf16x8_t*)(xs + xrow * SK_XS + vec * 8) = xr[v];
+        }
+    };
+
+    floatx4_t acc[SPW][MT];
+#pragma unroll
+    for (int s = 0; s < SPW; ++s)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[s][t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+    for (int j = 0; j < 4; ++j) load_w(j, a[j]);
+    load_x(0);
+    const int nchunk = (nkb + 3) / 4;
+    for (int c = 0; c < nchunk; ++c) {
+        __syncthreads();
+        store_x();
+        __syncthreads();
+        if (c + 1 < nchunk) load_x(c + 1);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                const bf16_t* xrow = xs + (t * 16 + r) * SK_XS + j * 128 + g * 8;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const bf16x8_t b = *(const bf16x8_t*)(xrow + i * 32);
+#pragma unroll
+                    for (int s = 0; s < SPW; ++s)
+                        acc[s][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j][s][i], b, acc[s][t], 0, 0, 0);
+                }
+            }
+            load_w(c * 4 + j + 4, a[j]);
+        }
+    }
+
+    // lane (r, g) of tile t holds token t*16 + r, rows 4g .. 4g+3 of each strip
+    OT* Yp = Y + (MODE == 1 ? (long)blockIdx.y * part_stride : 0);
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        const int tok = t * 16 + r;
+        if (tok >= M) continue;
+        if (MODE == 2) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int col = out_base[0] + 4 * g + i;
+                if (col < I) {
+                    const float gt = acc[0][t][i], up = acc[SPW - 1][t][i];
+                    Yp[(long)tok * ldy + col] = from_f32<OT>(gt / (1.0f + expf(-gt)) * up);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < SPW; ++s)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int col = out_base[s] + 4 * g + i;
+                    if (col < N) Yp[(long)tok * ldy + col] = from_f32<OT>(alpha * acc[s][t][i]);
+                }
+        }
+    }
+}
+
+// out_mode: 0 = Y[m,N] in out_dtype; 1 = float partial sums Y[ksplit][m][N]; 2 = gated (N = 2*I rows of W, Y[m,I] bf16)
+// variant: 0 = 4 waves x 2 strips, 1 = 8 waves x 1 strip, 2 = 4 waves x 1 strip; gated: 4, 2, 1 waves x a pair
+extern "C" const char* cpmcu_gemm_skinny_v(const void* X, long ldx, const void* W, long ldw, void* Y, long ldy,
+                                           int out_dtype, int out_mode, int M, int N, int K, int ksplit, float alpha,
+                                           int variant, hipStream_t stream) {
+    CPMCU_REQUIRE(M > 0 && M <= 64, "gemm_skinny: %d rows (1..64 are taken; more rows belong to the tiled product)", M);
+    CPMCU_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "gemm_skinny: K=%d must be a positive multiple of 8 (N=%d)", K, N);
+    CPMCU_REQUIRE(ldx % 8 == 0 && ldw % 8 == 0 && ldx >= K && ldw >= K, "gemm_skinny: leading dimensions %ld %ld must be multiples of 8 and >= K", ldx, ldw);
+    CPMCU_REQUIRE(((uintptr_t)X % 16 == 0) && ((uintptr_t)W % 16 == 0), "gemm_skinny: operands must be 16-byte aligned");
+    CPMCU_REQUIRE(ksplit >= 1 && (out_mode == 1 || ksplit == 1), "gemm_skinny: a K-split (%d) needs partial-sum output", ksplit);
+    CPMCU_REQUIRE(out_mode != 2 || N % 2 == 0, "gemm_skinny: gated output needs an even number of rows, got %d", N);
+    int KS = (K + ksplit - 1) / ksplit;
+    KS = (KS + 127) / 128 * 128;
+    const int splits = (K + KS - 1) / KS;
+    CPMCU_REQUIRE(splits == ksplit, "gemm_skinny: K=%d cannot be cut into %d slices of whole 128-blocks (would be %d)", K, ksplit, splits);
+    const int MT = (M + 15) / 16 == 3 ? 4 : (M + 15) / 16;
+    const int I = N / 2;
+    const long part_stride = (long)M * ldy;
+#define LAUNCH(MTv, MODEv, OT, SPW, NW)                                                                           \
+    do {                                                                                                          \
+        const int rows_wg = (MODEv == 2) ? NW * 16 : NW * SPW * 16;                                               \
+        dim3 grid(((MODEv == 2 ? I : N) + rows_wg - 1) / rows_wg, ksplit);                                        \
+        gemm_skinny_kernel<MTv, MODEv, OT, SPW, NW><<<grid, NW * 64, 0, stream>>>(                                \
+            (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (OT*)Y, ldy, M, N, K, KS, alpha, I, part_stride);       \
+    } while (0)
+#define BY_VAR(MTv, MODEv, OT)                                  \
+    do {                                                        \
+        if (MODEv == 2) {                                       \
+            if (variant == 1) LAUNCH(MTv, MODEv, OT, 2, 2);     \
+            else if (variant == 2) LAUNCH(MTv, MODEv, OT, 2, 1);\
+            else LAUNCH(MTv, MODEv, OT, 2, 4);                  \
+        } else if (variant == 1) LAUNCH(MTv, (MODEv == 2 ? 0 : MODEv), OT, 1, 8); \
+        else if (variant == 2) LAUNCH(MTv, (MODEv == 2 ? 0 : MODEv), OT, 1, 4);   \
+        else LAUNCH(MTv, (MODEv == 2 ? 0 : MODEv), OT, 2, 4);   \
+    } while (0)
+#define BY_MT(MODEv, OT)                         \
+    do {                                         \
+        if (MT == 1) BY_VAR(1, MODEv, OT);       \
+        else if (MT == 2) BY_VAR(2, MODEv, OT);  \
+        else BY_VAR(4, MODEv, OT);               \
+    } while (0)
+    if (out_mode == 0 && out_dtype == CPMCU_F32) BY_MT(0, float);
+    else if (out_mode == 0 && out_dtype == CPMCU_BF16) BY_MT(0, bf16_t);
+    else if (out_mode == 1) BY_MT(1, float);
+    else if (out_mode == 2) BY_MT(2, bf16_t);
+    else CPMCU_FAIL("gemm_skinny: unknown output mode %d / dtype %d", out_mode, out_dtype);
+#undef BY_MT
+#undef BY_VAR
+#undef LAUNCH
+    CPMCU_LAUNCH_CHECK("gemm_skinny");
+    return nullptr;
+}
+
+// The variant that measured best on the MI355X for each shape: one strip a wave (more, smaller
+// workgroups balance better over 256 CUs); gated output with 2 waves a workgroup up to 16 rows.
+extern "C" const char* cpmcu_gemm_skinny(const void* X, long ldx, const void* W, long ldw, void* Y, long ldy,
+                                         int out_dtype, int out_mode, int M, int N, int K, int ksplit, float alpha,
+                                         hipStream_t stream) {
+    const int variant = out_mode == 2 ? (M <= 16 ? 1 : 0) : 2;
+    return cpmcu_gemm_skinny_v(X, ldx, W, ldw, Y, ldy, out_dtype, out_mode, M, N, K, ksplit, alpha, variant, stream);
+}

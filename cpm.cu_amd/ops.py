@@ -189,6 +189,53 @@ def attention_plain(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hd: i
         _p(sel_blocks), _p(sel_count), c_int(max_sel), c_int(block_size), _stream()))
 
 
+MFMA_HEAD_DIMS = (16, 32, 64, 128)
+
+
+def attention_mfma_ok(q: torch.Tensor, hd: int, page_size: int, block_size: int = 0) -> bool:
+    return (q.dtype == torch.bfloat16 and hd in MFMA_HEAD_DIMS and page_size % 32 == 0
+            and (block_size == 0 or block_size % 32 == 0))
+
+
+def attention_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hd: int, scale: float,
+                   kpool: torch.Tensor, vpool: torch.Tensor, page_table: torch.Tensor, page_size: int,
+                   positions: torch.Tensor, tok_slot: torch.Tensor, n_splits: int = 1,
+                   part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None,
+                   sel_blocks: Optional[torch.Tensor] = None, sel_count: Optional[torch.Tensor] = None,
+                   block_size: int = 0):
+    """bf16 attention on the matrix cores (head_dim 16, 32, 64 or 128; pages and key blocks multiples of 32).
+    With n_splits > 1 every token's keys are shared among n_splits wavefronts and merged afterwards;
+    part_o float32 [n, nh, n_splits, hd] and part_ml float32 [n, nh, n_splits, 2] are its scratch."""
+    _need(q, "attention q", torch.bfloat16, (None, nh * hd))
+    n = q.shape[0]
+    _need(out, "attention out", torch.bfloat16, (n, nh * hd))
+    _need(kpool, "attention key pool", torch.bfloat16, (None, page_size, nkv * hd))
+    _need(vpool, "attention value pool", torch.bfloat16, tuple(kpool.shape))
+    _need(page_table, "attention page table", torch.int32, (None, None))
+    _need(positions, "attention positions", torch.int32, (n,))
+    _need(tok_slot, "attention token slots", torch.int32, (n,))
+    max_sel = 0
+    if sel_count is not None:
+        _need(sel_count, "attention block counts", torch.int32, (n, nkv))
+        _need(sel_blocks, "attention block list", torch.int32, (n, nkv, None))
+        max_sel = sel_blocks.shape[2]
+    if n_splits > 1:
+        _need(part_o, "attention partial outputs", torch.float32, (n, nh, n_splits, hd))
+        _need(part_ml, "attention partial max/sum", torch.float32, (n, nh, n_splits, 2))
+    _check(_fn("attention", "cpmcu_attention_mfma")(
+        _p(q), _p(out), _p(part_o), _p(part_ml), c_int(n), c_int(nh), c_int(nkv), c_int(hd), c_float(scale),
+        _p(kpool), _p(vpool), _p(page_table), c_int(page_table.shape[1]), c_int(page_size), _p(positions),
+        _p(tok_slot), _p(sel_blocks), _p(sel_count), c_int(max_sel), c_int(block_size), c_int(n_splits), _stream()))
+
+
+def attention_splits(n_tokens: int, nkv: int, group: int, max_keys: int) -> int:
+    """Shares of a token's keys: enough wavefronts (about 2048) to fill 256 CUs when a step has few
+    tokens, each with at least 128 keys."""
+    waves = n_tokens * nkv * -(-group // 16)
+    s = max(1, min(2048 // max(waves, 1), max_keys // 128, 64))
+    return s
+
+
 def compress_keys(kpool: torch.Tensor, ckpool: torch.Tensor, page_table: torch.Tensor, page_size: int,
                   positions: torch.Tensor, tok_slot: torch.Tensor, kernel_size: int, kernel_stride: int):
     """Write the compressed keys (means of kernel_size keys, every kernel_stride) that the step's tokens complete."""
@@ -251,16 +298,79 @@ def sample(logits: torch.Tensor, temperature: float, seed: int, request_ids: tor
                                        _p(u_out), _stream()))
 
 
+def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, alpha: float = 1.0, mode: str = "plain"):
+    """bf16 product for at most 64 rows of x on the matrix cores, streaming w once.
+    mode 'plain': out [m,N] float32 or bfloat16; 'partial': out float32 [S,m,N], S slices of K to be summed by
+    the consumer; 'gated': w holds gate rows then up rows, out bfloat16 [m,N/2] = silu(gate) * up."""
+    _need(x, "gemm x", torch.bfloat16, (None, None))
+    M, K = x.shape
+    _need(w, "gemm weight", torch.bfloat16, (None, K))
+    N = w.shape[0]
+    ksplit, omode = 1, 0
+    if mode == "plain":
+        _need(out, "gemm out", shape=(M, N))
+        ldy = N
+    elif mode == "partial":
+        _need(out, "gemm partial sums", torch.float32, (None, M, N))
+        ksplit, omode, ldy = out.shape[0], 1, N
+    elif mode == "gated":
+        _need(out, "gemm gated out", torch.bfloat16, (M, N // 2))
+        omode, ldy = 2, N // 2
+    else:
+        raise KernelError(f"gemm_skinny: unknown mode '{mode}'")
+    _check(_fn("gemm", "cpmcu_gemm_skinny")(_p(x), c_long(K), _p(w), c_long(K), _p(out), c_long(ldy),
+                                            c_int(_code(out)), c_int(omode), c_int(M), c_int(N), c_int(K),
+                                            c_int(ksplit), c_float(alpha), _stream()))
+
+
+SKINNY_MAX_ROWS = 64
+
+
+def skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+    return x.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 8 == 0
+
+
+def skinny_split(M: int, N: int, K: int) -> int:
+    """Slices of K for a skinny product whose consumer sums partial results.  A workgroup streams 64 rows
+    of the weight; about 1024 workgroups balance well over the 256 CUs, every slice should still stream 512
+    columns, and more rows make the partial sums themselves cost traffic (measured on the MI355X)."""
+    wgs = -(-N // 64)
+    cap = 16 if M <= 16 else (8 if M <= 32 else 4)
+    want = 1
+    while want * 2 <= cap and wgs * want * 2 <= 1280 and K // (want * 2) >= 512:
+        want *= 2
+    if want <= 1:
+        return 1
+    ks = -(-(-(-K // want)) // 128) * 128
+    return -(-K // ks)
+
+
 # ---------------------------------------------------------------------------
 # dispatchers: choose the kernel for a shape and element type
 # ---------------------------------------------------------------------------
 def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, alpha: float = 1.0):
     """out = alpha * x . w^T with the kernel that suits the element type and the number of rows."""
-    gemm_nt_plain(x, w, out, alpha)
+    if skinny_ok(x, w):
+        gemm_skinny(x, w, out, alpha)
+    else:
+        gemm_nt_plain(x, w, out, alpha)
 
 
 def attention(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, ctx,
               sel_blocks=None, sel_count=None, block_size=0):
     """Attention of the step's queries over the cache, with the kernel that suits the step."""
+    if attention_mfma_ok(q, hd, page_size, block_size if sel_count is not None else 0):
+        n = q.shape[0]
+        keys = ctx.max_pos + 1
+        if sel_count is not None:
+            keys = min(keys, sel_blocks.shape[2] * block_size)
+        splits = attention_splits(n, nkv, nh // nkv, keys)
+        part_o = part_ml = None
+        if splits > 1:
+            part_o = ctx.ws.get("attn.part_o", (n, nh, splits, hd), torch.float32)
+            part_ml = ctx.ws.get("attn.part_ml", (n, nh, splits, 2), torch.float32)
+        attention_mfma(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, ctx.positions, ctx.tok_slot,
+                       splits, part_o, part_ml, sel_blocks, sel_count, block_size)
+        return
     attention_plain(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, ctx.positions, ctx.tok_slot,
                     sel_blocks, sel_count, block_size)

@@ -56,7 +56,8 @@ class GQAAttention(Mixer):
     def project_and_store(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool) -> torch.Tensor:
         n = h.shape[0]
         nh, nkv, hd = self.nh, self.nkv, self.hd
-        qkv = self.qkv.forward(h, ctx, "attn.qkv", rows=None if writes_cache else nh * hd)
+        plain_rotation = self.position is None or self.position.rotary_params() is not None
+        qkv = self.qkv.forward(h, ctx, "attn.qkv", rows=None if writes_cache else nh * hd, partials=plain_rotation)
         rot = self.position.rotary_params() if self.position is not None else None
         inv_freq, mag = (rot if rot is not None else (None, 1.0))
         if self.position is not None and rot is None:
@@ -79,7 +80,7 @@ class GQAAttention(Mixer):
     def forward(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool = True) -> torch.Tensor:
         q = self.project_and_store(h, ctx, cache, writes_cache)
         a = self.attend(q, ctx, cache)
-        return self.o.forward(a, ctx, "attn.o", out_dtype=torch.float32)
+        return self.o.forward(a, ctx, "attn.o", out_dtype=torch.float32, partials=True)
 
 
 @MIXERS.register("infllm_v2_attention")
@@ -117,4 +118,4 @@ class InfLLMv2Attention(GQAAttention):
                               sel_blocks, sel_count)
             sel = (sel_blocks, sel_count, self.bs)
         a = self.attend(q, ctx, cache, sel)
-        return self.o.forward(a, ctx, "attn.o", out_dtype=torch.float32)
+        return self.o.forward(a, ctx, "attn.o", out_dtype=torch.float32, partials=True)

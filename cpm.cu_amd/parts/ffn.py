@@ -27,7 +27,5 @@ class GatedFFN(FeedForward):
         return [self.gate_up, self.down]
 
     def forward(self, h: torch.Tensor, ctx: StepContext) -> torch.Tensor:
-        gu = self.gate_up.forward(h, ctx, "ffn.gate_up")
-        act = ctx.ws.get("ffn.act", (h.shape[0], self.intermediate_size), h.dtype)
-        ops.silu_mul(gu, act)
-        return self.down.forward(act, ctx, "ffn.down", out_dtype=torch.float32)
+        act = self.gate_up.forward_gated(h, ctx, "ffn.gate_up")
+        return self.down.forward(act, ctx, "ffn.down", out_dtype=torch.float32, partials=True)

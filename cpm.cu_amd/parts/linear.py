@@ -33,9 +33,29 @@ class Linear(Part):
         self.rt = rt
 
     def forward(self, x: torch.Tensor, ctx: StepContext, tag: str, out_dtype: Optional[torch.dtype] = None,
-                alpha: float = 1.0, rows: Optional[int] = None) -> torch.Tensor:
-        """x [n, in] -> [n, out] (the first ``rows`` output features only, if given)."""
+                alpha: float = 1.0, rows: Optional[int] = None, partials: bool = False) -> torch.Tensor:
+        """x [n, in] -> [n, out] (the first ``rows`` output features only, if given).  With ``partials`` the
+        result may come as float32 partial sums [S, n, out] over slices of the input axis, for a consumer
+        that adds them up (the norm and the position-encoding kernels do)."""
         w = self.weight if rows is None else self.weight[:rows]
-        out = ctx.ws.get(tag, (x.shape[0], w.shape[0]), out_dtype or x.dtype)
+        n, N = x.shape[0], w.shape[0]
+        if partials and ops.skinny_ok(x, w):
+            S = ops.skinny_split(n, N, self.in_features)
+            if S > 1:
+                out = ctx.ws.get(tag, (S, n, N), torch.float32)
+                ops.gemm_skinny(x, w, out, alpha, mode="partial")
+                return out
+        out = ctx.ws.get(tag, (n, N), out_dtype or x.dtype)
         ops.linear(x, w, out, alpha)
         return out
+
+    def forward_gated(self, x: torch.Tensor, ctx: StepContext, tag: str) -> torch.Tensor:
+        """For a weight of gate rows stacked on up rows: silu(x Wg^T) * (x Wu^T), [n, out/2]."""
+        n, half = x.shape[0], self.out_features // 2
+        act = ctx.ws.get(tag + ".act", (n, half), x.dtype)
+        if ops.skinny_ok(x, self.weight):
+            ops.gemm_skinny(x, self.weight, act, mode="gated")
+        else:
+            gu = self.forward(x, ctx, tag)
+            ops.silu_mul(gu, act)
+        return act

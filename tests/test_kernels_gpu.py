@@ -1,0 +1,301 @@
+"""Each kernel alone against a plain float reference, at sizes other than the engine's (GPU)."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def rnd(*shape, seed=0, dtype=torch.float32, scale=1.0):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+# ---------------------------------------------------------------------------- products
+@pytest.mark.parametrize("M,N,K", [(1, 40, 64), (7, 129, 96), (64, 512, 160), (65, 100, 72), (200, 333, 50), (3, 17, 5)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_plain_product(M, N, K, dtype):
+    from cpmcu_amd import ops
+    x, w = rnd(M, K, seed=1, dtype=dtype), rnd(N, K, seed=2, dtype=dtype)
+    ref = 0.5 * (x.double() @ w.double().T)
+    for out_dtype in ([torch.float32] if dtype == torch.float32 else [torch.float32, torch.bfloat16]):
+        out = torch.empty(M, N, dtype=out_dtype, device=DEV)
+        ops.gemm_nt_plain(x, w, out, 0.5)
+        tol = 1e-5 * math.sqrt(K) if out_dtype == torch.float32 else 2 ** -8 * float(ref.abs().max())
+        assert float((out.double() - ref).abs().max()) <= tol
+
+
+@pytest.mark.parametrize("M", [1, 5, 16, 17, 33, 48, 64])
+@pytest.mark.parametrize("N,K", [(96, 64), (136, 160), (1000, 96), (4608, 1024), (250, 520), (73448 // 8 + 3, 256)])
+def test_skinny_product_all_modes(M, N, K):
+    """bf16 operands are exact in float, so the matrix-core product must match a float64 product of the same
+    bf16 values up to float32 accumulation."""
+    from cpmcu_amd import ops
+    x, w = rnd(M, K, seed=3, dtype=torch.bfloat16), rnd(N, K, seed=4, dtype=torch.bfloat16, scale=0.1)
+    ref = x.double() @ w.double().T
+    tol = 2e-6 * math.sqrt(K) * float(ref.abs().max() + 1)
+    out = torch.empty(M, N, dtype=torch.float32, device=DEV)
+    ops.gemm_skinny(x, w, out, 1.0)
+    assert float((out.double() - ref).abs().max()) <= tol
+    ops.gemm_skinny(x, w, out, 0.25)
+    assert float((out.double() - 0.25 * ref).abs().max()) <= tol
+    out16 = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    ops.gemm_skinny(x, w, out16, 1.0)
+    assert float((out16.double() - ref).abs().max()) <= 2 ** -8 * float(ref.abs().max())
+    for S in (2, 3):                                    # slices of K, summed by the consumer
+        ks = -(-(-(-K // S)) // 128) * 128
+        S_real = -(-K // ks)
+        part = torch.full((S_real, M, N), float("nan"), dtype=torch.float32, device=DEV)
+        ops.gemm_skinny(x, w, part, 1.0, mode="partial")
+        assert float((part.double().sum(0) - ref).abs().max()) <= tol
+    if N % 2 == 0:
+        I = N // 2
+        act = torch.empty(M, I, dtype=torch.bfloat16, device=DEV)
+        ops.gemm_skinny(x, w, act, mode="gated")
+        want = F.silu(ref[:, :I]) * ref[:, I:]
+        assert float((act.double() - want).abs().max()) <= 2 ** -8 * float(want.abs().max()) + tol
+
+
+def test_skinny_split_heuristic_matches_what_the_kernel_accepts():
+    from cpmcu_amd import ops
+    for M in (1, 8, 64):
+        for N, K in [(4608, 4096), (4096, 4096), (4096, 16384), (73448, 4096), (64, 64), (96, 160), (1000, 96)]:
+            S = ops.skinny_split(M, N, K)
+            x, w = torch.zeros(M, K, dtype=torch.bfloat16, device=DEV), torch.zeros(N, K, dtype=torch.bfloat16, device=DEV)
+            if S > 1:
+                ops.gemm_skinny(x, w, torch.empty(S, M, N, dtype=torch.float32, device=DEV), mode="partial")
+
+
+def test_products_refuse_what_they_do_not_take():
+    from cpmcu_amd import ops
+    x, w = torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ops.KernelError, match="1..64"):
+        ops.gemm_skinny(x, w, torch.empty(65, 32, dtype=torch.float32, device=DEV))
+    with pytest.raises(ops.KernelError, match="multiple of 8"):
+        ops.gemm_skinny(torch.zeros(2, 20, dtype=torch.bfloat16, device=DEV), torch.zeros(8, 20, dtype=torch.bfloat16, device=DEV),
+                        torch.empty(2, 8, dtype=torch.float32, device=DEV))
+    with pytest.raises(ops.KernelError, match="GPU tensor"):
+        ops.gemm_nt_plain(torch.zeros(2, 8), torch.zeros(4, 8), torch.zeros(2, 4))
+    with pytest.raises(ops.KernelError, match="shape"):
+        ops.gemm_nt_plain(x, w, torch.empty(65, 33, dtype=torch.float32, device=DEV))
+
+
+# ---------------------------------------------------------------------------- row-wise kernels
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embedding(dtype):
+    from cpmcu_amd import ops
+    table = rnd(37, 50, dtype=dtype)
+    ids = torch.tensor([0, 36, 5, 5, 17], dtype=torch.int32, device=DEV)
+    out = torch.empty(5, 50, dtype=torch.float32, device=DEV)
+    ops.embed(table, ids, out, 12.0)
+    assert torch.equal(out, table.float()[ids.long()] * 12.0)
+
+
+@pytest.mark.parametrize("H", [24, 100, 1000, 4096 + 8])
+@pytest.mark.parametrize("bdtype,odtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                           (torch.float32, torch.bfloat16)])
+def test_add_rms_norm(H, bdtype, odtype):
+    from cpmcu_amd import ops
+    n, eps = 6, 1e-5
+    x0, w = rnd(n, H, seed=1), rnd(H, seed=2) + 1.0
+    otol = 1e-5 if odtype == torch.float32 else 2 ** -8
+    # plain norm
+    x = x0.clone()
+    out = torch.empty(n, H, dtype=odtype, device=DEV)
+    ops.add_rms_norm(x, None, 1.0, w, eps, out)
+    ref = F.rms_norm(x0.double(), (H,), w.double(), eps)
+    assert torch.equal(x, x0) and float((out.double() - ref).abs().max()) <= otol * float(ref.abs().max())
+    # with a branch, as one tensor and as 3 partial sums
+    for parts in (1, 3):
+        b = rnd(parts, n, H, seed=3, dtype=bdtype)
+        x = x0.clone()
+        ops.add_rms_norm(x, b if parts > 1 else b[0], 0.7, w, eps, out)
+        xs = x0.double() + 0.7 * b.double().sum(0)
+        assert float((x.double() - xs).abs().max()) <= 1e-5
+        ref = F.rms_norm(xs, (H,), w.double(), eps)
+        assert float((out.double() - ref).abs().max()) <= otol * float(ref.abs().max())
+        # chosen rows only (one of them twice): x stays as it was
+        rows = torch.tensor([4, 0, 4], dtype=torch.int32, device=DEV)
+        x = x0.clone()
+        out_r = torch.empty(3, H, dtype=odtype, device=DEV)
+        ops.add_rms_norm(x, b if parts > 1 else b[0], 0.7, w, eps, out_r, rows)
+        assert torch.equal(x, x0)
+        assert float((out_r.double() - ref[rows.long()]).abs().max()) <= otol * float(ref.abs().max())
+    # eps inside the root: a tiny constant row
+    c = 3e-3
+    x = torch.full((1, H), c, device=DEV)
+    o = torch.empty(1, H, dtype=torch.float32, device=DEV)
+    ops.add_rms_norm(x, None, 1.0, torch.ones(H, device=DEV), eps, o)
+    assert float((o - c / math.sqrt(c * c + eps)).abs().max()) < 1e-6
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_silu_mul(dtype):
+    from cpmcu_amd import ops
+    gu = rnd(5, 2 * 77, dtype=dtype, scale=3.0)
+    out = torch.empty(5, 77, dtype=dtype, device=DEV)
+    ops.silu_mul(gu, out)
+    ref = F.silu(gu[:, :77].double()) * gu[:, 77:].double()
+    tol = 1e-6 if dtype == torch.float32 else 2 ** -8
+    assert float((out.double() - ref).abs().max()) <= tol * float(ref.abs().max() + 1)
+
+
+# ---------------------------------------------------------------------------- attention over the paged cache
+def paged_setup(lens, nkv, hd, page, dtype, seed=0, scramble=True):
+    """Sequences of the given lengths in a paged cache whose pages are handed out in a scrambled order.
+    Returns keys/values per sequence (float64) and the pools/page table as the kernels want them."""
+    g = torch.Generator().manual_seed(seed)
+    n_pages_seq = [-(-L // page) for L in lens]
+    total = sum(n_pages_seq) + 3
+    perm = torch.randperm(total, generator=g).tolist() if scramble else list(range(total))
+    table = torch.zeros(len(lens), max(n_pages_seq), dtype=torch.int32)
+    kpool = torch.zeros(total, page, nkv * hd, dtype=dtype)
+    vpool = torch.zeros(total, page, nkv * hd, dtype=dtype)            # [page][kv head][d][token]: same bytes
+    ks, vs = [], []
+    it = iter(perm)
+    for s, L in enumerate(lens):
+        k = torch.randn(L, nkv, hd, generator=g).to(dtype)
+        v = torch.randn(L, nkv, hd, generator=g).to(dtype)
+        ks.append(k.double())
+        vs.append(v.double())
+        for pn in range(n_pages_seq[s]):
+            pg = next(it)
+            table[s, pn] = pg
+            a, b = pn * page, min((pn + 1) * page, L)
+            kpool[pg, :b - a] = k[a:b].reshape(b - a, nkv * hd)
+            vt = vpool[pg].view(nkv, hd, page)
+            vt[:, :, :b - a] = v[a:b].permute(1, 2, 0)
+    return ks, vs, kpool.to(DEV), vpool.to(DEV), table.to(DEV)
+
+
+def attention_reference(qs, ks, vs, positions, seq_of, nh, scale, allowed=None):
+    out = []
+    nkv = ks[0].shape[1]
+    G = nh // nkv
+    for t, (p, s) in enumerate(zip(positions, seq_of)):
+        k, v = ks[s][:p + 1], vs[s][:p + 1]
+        row = []
+        for h in range(nh):
+            sc = (k[:, h // G] @ qs[t, h]) * scale
+            if allowed is not None:
+                sc = sc.masked_fill(~allowed[t][h // G][:p + 1], float("-inf"))
+            row.append(torch.softmax(sc, 0) @ v[:, h // G])
+        out.append(torch.stack(row))
+    return torch.stack(out)
+
+
+@pytest.mark.parametrize("nh,nkv,hd", [(4, 2, 16), (3, 1, 32), (6, 3, 64), (32, 2, 128), (20, 1, 32), (2, 2, 48), (4, 1, 256)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_over_scrambled_pages(nh, nkv, hd, dtype):
+    """Prompt tokens and single tokens of three sequences at once; plain kernel, and the matrix-core kernel
+    with 1, 3 and 8 shares of the keys where it takes the head size."""
+    from cpmcu_amd import ops
+    page = 64
+    lens = [300, 70, 1]
+    ks, vs, kpool, vpool, table = paged_setup(lens, nkv, hd, page, dtype, seed=hd)
+    # queries: the last 40 positions of sequence 0, the last of sequence 1, the only one of sequence 2
+    positions = list(range(260, 300)) + [69, 0]
+    seq_of = [0] * 40 + [1, 2]
+    n = len(positions)
+    q = rnd(n, nh, hd, seed=5, dtype=dtype)
+    scale = hd ** -0.5
+    ref = attention_reference(q.double().cpu(), ks, vs, positions, seq_of, nh, scale)
+    pos_t = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    slot_t = torch.tensor(seq_of, dtype=torch.int32, device=DEV)
+    tol = 2e-6 if dtype == torch.float32 else 2 ** -7
+    out = torch.empty(n, nh * hd, dtype=dtype, device=DEV)
+    ops.attention_plain(q.view(n, -1), out, nh, nkv, hd, scale, kpool, vpool, table, page, pos_t, slot_t)
+    assert float((out.double().cpu().view(n, nh, hd) - ref).abs().max()) <= tol
+    if dtype == torch.bfloat16 and hd in ops.MFMA_HEAD_DIMS:
+        for splits in (1, 3, 8):
+            out.fill_(float("nan"))
+            po = torch.full((n, nh, splits, hd), float("nan"), device=DEV) if splits > 1 else None
+            pm = torch.full((n, nh, splits, 2), float("nan"), device=DEV) if splits > 1 else None
+            ops.attention_mfma(q.view(n, -1), out, nh, nkv, hd, scale, kpool, vpool, table, page, pos_t, slot_t,
+                               splits, po, pm)
+            assert float((out.double().cpu().view(n, nh, hd) - ref).abs().max()) <= tol, f"splits={splits}"
+    elif dtype == torch.bfloat16:
+        assert not ops.attention_mfma_ok(q.view(n, -1), hd, page)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_finds_one_far_key_among_hundreds(dtype):
+    """One key far back is made to stand out: the output must be its value (a kernel that skips or misplaces
+    a page, or mixes up the transposed values, fails this)."""
+    from cpmcu_amd import ops
+    nh, nkv, hd, page = 16, 1, 64, 64
+    L = 1000
+    ks, vs, kpool, vpool, table = paged_setup([L], nkv, hd, page, dtype, seed=3)
+    for far in (0, 63, 64, 517, 998, 999):
+        k = ks[0].clone()
+        q = torch.zeros(1, nh, hd, dtype=torch.float64)
+        q[0, :, 5] = 40.0
+        pg, off = int(table[0, far // page]), far % page
+        saved = kpool[pg, off].clone()
+        kpool[pg, off] = 0
+        kpool[pg, off, 5] = 40.0
+        pos_t = torch.tensor([L - 1], dtype=torch.int32, device=DEV)
+        slot_t = torch.zeros(1, dtype=torch.int32, device=DEV)
+        qd = q.to(dtype).to(DEV).view(1, -1)
+        outs = []
+        out = torch.empty(1, nh * hd, dtype=dtype, device=DEV)
+        ops.attention_plain(qd, out, nh, nkv, hd, hd ** -0.5, kpool, vpool, table, page, pos_t, slot_t)
+        outs.append(out.clone())
+        if dtype == torch.bfloat16:
+            for splits in (1, 5):
+                po = torch.empty(1, nh, splits, hd, device=DEV)
+                pm = torch.empty(1, nh, splits, 2, device=DEV)
+                ops.attention_mfma(qd, out, nh, nkv, hd, hd ** -0.5, kpool, vpool, table, page, pos_t, slot_t, splits, po, pm)
+                outs.append(out.clone())
+        for o in outs:
+            assert float((o.double().cpu().view(nh, hd) - vs[0][far, 0]).abs().max()) < 1e-2, far
+        kpool[pg, off] = saved
+
+
+@pytest.mark.parametrize("bs", [16, 32, 64])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_with_block_lists(bs, dtype):
+    """Only the listed key blocks are attended to; a count of -1 means all keys."""
+    from cpmcu_amd import ops
+    nh, nkv, hd, page = 6, 2, 32, 64
+    L = 400
+    ks, vs, kpool, vpool, table = paged_setup([L], nkv, hd, page, dtype, seed=9)
+    positions = [399, 250, 131, 64]
+    n = len(positions)
+    q = rnd(n, nh, hd, seed=2, dtype=dtype)
+    max_sel = 6
+    sel_blocks = torch.zeros(n, nkv, max_sel, dtype=torch.int32)
+    sel_count = torch.zeros(n, nkv, dtype=torch.int32)
+    allowed = torch.zeros(n, nkv, L, dtype=torch.bool)
+    g = torch.Generator().manual_seed(1)
+    for t, p in enumerate(positions):
+        for h in range(nkv):
+            if t == 2 and h == 1:
+                sel_count[t, h] = -1
+                allowed[t, h] = True
+                continue
+            own = p // bs
+            cand = torch.randperm(own, generator=g)[:4].tolist() if own > 0 else []
+            blocks = sorted(set(cand + [own]))
+            sel_count[t, h] = len(blocks)
+            sel_blocks[t, h, :len(blocks)] = torch.tensor(blocks, dtype=torch.int32)
+            for b in blocks:
+                allowed[t, h, b * bs:(b + 1) * bs] = True
+    ref = attention_reference(q.double().cpu(), ks, vs, positions, [0] * n, nh, hd ** -0.5, allowed)
+    pos_t = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    slot_t = torch.zeros(n, dtype=torch.int32, device=DEV)
+    out = torch.empty(n, nh * hd, dtype=dtype, device=DEV)
+    tol = 2e-6 if dtype == torch.float32 else 2 ** -7
+    ops.attention_plain(q.view(n, -1), out, nh, nkv, hd, hd ** -0.5, kpool, vpool, table, page, pos_t, slot_t,
+                        sel_blocks.to(DEV), sel_count.to(DEV), bs)
+    assert float((out.double().cpu().view(n, nh, hd) - ref).abs().max()) <= tol
+    if dtype == torch.bfloat16 and bs % 32 == 0:
+        for splits in (1, 4):
+            po = torch.empty(n, nh, splits, hd, device=DEV)
+            pm = torch.empty(n, nh, splits, 2, device=DEV)
+            ops.attention_mfma(q.view(n, -1), out, nh, nkv, hd, hd ** -0.5, kpool, vpool, table, page, pos_t, slot_t,
+                               splits, po, pm, sel_blocks.to(DEV), sel_count.to(DEV), bs)
+            assert float((out.double().cpu().view(n, nh, hd) - ref).abs().max()) <= tol
