@@ -128,7 +128,8 @@ extern "C" const char* cpmcu_attention_plain(const void* q, void* out, int dtype
 //                      values are stored transposed inside a page
 // The two key tiles of a chunk take keys {8g..8g+3} and {8g+4..8g+7} of every
 // group of 8 so that a lane's 8 probabilities are 8 consecutive keys, the order
-// the V^T vector has.  No LDS and no barrier is used.
+// the V^T vector has.  With 4 wavefronts a workgroup (decode steps) the wavefronts take
+// the workgroup's chunks in turn and merge their running results through LDS at the end.
 // Output: out (bf16) when n_splits == 1, else unnormalised partial results
 // part_o[token][head][split][d], part_ml[token][head][split] = (max, sum) for
 // attention_combine_kernel.
@@ -138,8 +139,8 @@ extern "C" const char* cpmcu_attention_plain(const void* q, void* out, int dtype
 typedef __bf16 abf16x8_t __attribute__((ext_vector_type(8)));
 typedef float afloatx4_t __attribute__((ext_vector_type(4)));
 
-template <int HD>
-__global__ __launch_bounds__(64) void attention_mfma_kernel(
+template <int HD, int NW>
+__global__ __launch_bounds__(NW * 64) void attention_mfma_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, float* __restrict__ part_o, float2* __restrict__ part_ml,
     const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vtpool, PagedView pv,
     const int* __restrict__ positions, const int* __restrict__ tok_slot, int nh, int nkv, float scale_log2e,
@@ -149,7 +150,7 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
     const int t = blockIdx.x;
     const int kvh = blockIdx.y % nkv, ht = blockIdx.y / nkv;
     const int split = blockIdx.z;
-    const int lane = threadIdx.x, n = lane & 15, g = lane >> 4;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
     const int G = nh / nkv;
     const int head = kvh * G + ht * 16 + n;            // the head this lane's D column belongs to
     const bool head_ok = ht * 16 + n < G;
@@ -165,16 +166,16 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
         qf[ks] = v;
     }
 
-    // which chunks of 32 keys are this wavefront's
+    // which chunks of 32 keys are this workgroup's; its wavefronts take them in turn
     const int* sel = nullptr;
     int total_chunks = pos / 32 + 1;
     int cpb = 1;
     if (sel_count) {
-        const int c = sel_count[(long)t * nkv + kvh];
-        if (c >= 0) {
+        const int cnt = sel_count[(long)t * nkv + kvh];
+        if (cnt >= 0) {
             sel = sel_blocks + ((long)t * nkv + kvh) * max_sel;
             cpb = block_size / 32;
-            total_chunks = c * cpb;
+            total_chunks = cnt * cpb;
         }
     }
     const int per_split = (total_chunks + n_splits - 1) / n_splits;
@@ -186,97 +187,189 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(
     float m = -INFINITY, l = 0.f;
     const long kv_width = (long)nkv * HD;
 
-    for (int c = c0; c < c1; ++c) {
-        const int key0 = sel ? sel[c / cpb] * block_size + (c % cpb) * 32 : c * 32;
-        if (key0 > pos) continue;
-        const int page = ptab[key0 / pv.page_size];
-        const int po = key0 % pv.page_size;
-        // S^T for two tiles of 16 keys: key slot r of tile u is key0 + r + 4*(r/4) + 4u
-        afloatx4_t st[2];
+    auto chunk_key0 = [&](int c) { return sel ? sel[c / cpb] * block_size + (c % cpb) * 32 : c * 32; };
+    // key slot r of tile u is key0 + r + 4*(r/4) + 4u
+    auto load_k = [&](int page, int po, abf16x8_t (&kf)[2][KSTEPS]) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            st[u] = afloatx4_t{0.f, 0.f, 0.f, 0.f};
             const long krow = (long)page * pv.page_size + po + n + 4 * (n >> 2) + 4 * u;
             const bf16_t* kp = kpool + krow * kv_width + (long)kvh * HD + g * 8;
 #pragma unroll
             for (int ks = 0; ks < KSTEPS; ++ks) {
-                abf16x8_t kf = {0, 0, 0, 0, 0, 0, 0, 0};
-                if (ks * 32 + g * 8 < HD) kf = *(const abf16x8_t*)(kp + ks * 32);
-                st[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], st[u], 0, 0, 0);
+                abf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+                if (ks * 32 + g * 8 < HD) v = *(const abf16x8_t*)(kp + ks * 32);
+                kf[u][ks] = v;
             }
         }
-        // lane (head n, g): st[u][i] is key key0 + 8g + 4u + i
-        float s[8];
-        float mx = -INFINITY;
+    };
+
+    int c = c0 + wave;
+    abf16x8_t kf[2][KSTEPS];
+    int key0 = 0, page = 0, po = 0;
+    if (c < c1) {
+        key0 = chunk_key0(c);
+        page = ptab[key0 / pv.page_size];
+        po = key0 % pv.page_size;
+        load_k(page, po, kf);
+    }
+    while (c < c1) {
+        // this chunk's values and the next chunk's keys are asked for before this chunk's arithmetic
+        abf16x8_t vf[DT];
+        {
+            const bf16_t* vp = vtpool + (((long)page * nkv + kvh) * HD + n) * pv.page_size + po + g * 8;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const abf16x8_t*)(vp + (long)dt * 16 * pv.page_size);
+        }
+        const int cn = c + NW;
+        abf16x8_t kn[2][KSTEPS];
+        int key0n = 0, pagen = 0, pon = 0;
+        if (cn < c1) {
+            key0n = chunk_key0(cn);
+            pagen = ptab[key0n / pv.page_size];
+            pon = key0n % pv.page_size;
+            load_k(pagen, pon, kn);
+        }
+        if (key0 <= pos) {
+            afloatx4_t st[2];
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                st[u] = afloatx4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < KSTEPS; ++ks)
+                    st[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][ks], qf[ks], st[u], 0, 0, 0);
+            }
+            // lane (head n, g): st[u][i] is key key0 + 8g + 4u + i
+            float sc[8];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int key = key0 + 8 * g + 4 * u + i;
+                    const float v = key <= pos ? st[u][i] * scale_log2e : -INFINITY;
+                    sc[u * 4 + i] = v;
+                    mx = fmaxf(mx, v);
+                }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m, mx);
+            const float corr = exp2f(m - m_new);
+            float rs = 0.f;
+            abf16x8_t pb;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float p = exp2f(sc[j] - m_new);
+                rs += p;
+                pb[j] = (__bf16)p;
+            }
+            rs += __shfl_xor(rs, 16, 64);
+            rs += __shfl_xor(rs, 32, 64);
+            l = l * corr + rs;
+            m = m_new;
+            // O^T += V^T . P^T ; A operand: lane (d row n, g) holds V^T[d][key0 + 8g .. +8]
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[dt][i] *= corr;
+                acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pb, acc[dt], 0, 0, 0);
+            }
+        }
+        c = cn;
+        key0 = key0n;
+        page = pagen;
+        po = pon;
 #pragma unroll
         for (int u = 0; u < 2; ++u)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int key = key0 + 8 * g + 4 * u + i;
-                const float v = key <= pos ? st[u][i] * scale_log2e : -INFINITY;
-                s[u * 4 + i] = v;
-                mx = fmaxf(mx, v);
-            }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m, mx);
-        const float corr = exp2f(m - m_new);
-        float rs = 0.f;
-        abf16x8_t pb;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const float p = exp2f(s[j] - m_new);
-            rs += p;
-            pb[j] = (__bf16)p;
+            for (int ks = 0; ks < KSTEPS; ++ks) kf[u][ks] = kn[u][ks];
+    }
+
+    if (NW > 1) {
+        // merge the wavefronts' running results: wavefront w then finishes the d tiles w, w+NW, ...
+        __shared__ float ml_s[NW][16][2];
+        __shared__ float acc_s[NW * DT * 4 * 64];
+        if (g == 0) {
+            ml_s[wave][n][0] = m;
+            ml_s[wave][n][1] = l;
         }
-        rs += __shfl_xor(rs, 16, 64);
-        rs += __shfl_xor(rs, 32, 64);
-        l = l * corr + rs;
-        m = m_new;
-        // O^T += V^T . P^T ; A operand: lane (d row n, g) holds V^T[d][key0 + 8g .. +8]
-        const bf16_t* vp = vtpool + (((long)page * nkv + kvh) * HD + n) * pv.page_size + po + g * 8;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc_s[((wave * DT + dt) * 4 + i) * 64 + lane] = acc[dt][i];
+        __syncthreads();
+        float m_all = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < NW; ++w)
+            if (ml_s[w][n][1] > 0.f) m_all = fmaxf(m_all, ml_s[w][n][0]);
+        float l_all = 0.f;
+        float sw[NW];
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            sw[w] = ml_s[w][n][1] > 0.f ? exp2f(ml_s[w][n][0] - m_all) : 0.f;
+            l_all += sw[w] * ml_s[w][n][1];
+        }
+        m = m_all;
+        l = l_all;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-            const abf16x8_t vf = *(const abf16x8_t*)(vp + (long)dt * 16 * pv.page_size);
+            if (dt % NW != wave) continue;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) acc[dt][i] *= corr;
-            acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb, acc[dt], 0, 0, 0);
+            for (int i = 0; i < 4; ++i) {
+                float a = 0.f;
+#pragma unroll
+                for (int w = 0; w < NW; ++w) a += sw[w] * acc_s[((w * DT + dt) * 4 + i) * 64 + lane];
+                acc[dt][i] = a;
+            }
         }
     }
     if (!head_ok) return;
-    // lane (head n, g): acc[dt][i] is O[head][dt*16 + 4g + i]
+    // lane (head n, g): acc[dt][i] is O[head][dt*16 + 4g + i]; with NW > 1 this wavefront owns d tiles dt % NW == wave
     if (n_splits == 1) {
         const float inv = 1.0f / l;
         bf16_t* o = out + ((long)t * nh + head) * HD;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
+        for (int dt = 0; dt < DT; ++dt) {
+            if (NW > 1 && dt % NW != wave) continue;
 #pragma unroll
             for (int i = 0; i < 4; ++i) o[dt * 16 + 4 * g + i] = f32_to_bf16(acc[dt][i] * inv);
+        }
     } else {
         const long idx = ((long)t * nh + head) * n_splits + split;
         float* o = part_o + idx * HD;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) *(afloatx4_t*)(o + dt * 16 + 4 * g) = acc[dt];
-        if (g == 0) part_ml[idx] = make_float2(m, l);
+        for (int dt = 0; dt < DT; ++dt) {
+            if (NW > 1 && dt % NW != wave) continue;
+            *(afloatx4_t*)(o + dt * 16 + 4 * g) = acc[dt];
+        }
+        if (g == 0 && wave == 0) part_ml[idx] = make_float2(m, l);
     }
 }
 
 // out[token][head][:] = sum_s 2^(m_s - m) o_s / sum_s 2^(m_s - m) l_s   (splits without keys have l = 0)
 __global__ void attention_combine_kernel(const float* __restrict__ part_o, const float2* __restrict__ part_ml,
                                          bf16_t* __restrict__ out, int hd, int n_splits) {
+    __shared__ float wgt[64];
     const long row = blockIdx.x;             // token * nh + head
     const float2* ml = part_ml + row * n_splits;
     float m = -INFINITY;
-    for (int s = 0; s < n_splits; ++s)
-        if (ml[s].y > 0.f) m = fmaxf(m, ml[s].x);
+    for (int s = 0; s < n_splits; ++s) {
+        const float2 v = ml[s];
+        if (v.y > 0.f) m = fmaxf(m, v.x);
+    }
     float denom = 0.f;
-    for (int s = 0; s < n_splits; ++s)
-        if (ml[s].y > 0.f) denom += exp2f(ml[s].x - m) * ml[s].y;
+    for (int s = 0; s < n_splits; ++s) {
+        const float2 v = ml[s];
+        const float wv = v.y > 0.f ? exp2f(v.x - m) : 0.f;
+        denom += wv * v.y;
+        if (threadIdx.x == 0) wgt[s] = wv;
+    }
+    __syncthreads();
     const float inv = 1.0f / denom;
+    const float* po = part_o + row * n_splits * hd;
     for (int d = threadIdx.x; d < hd; d += blockDim.x) {
         float a = 0.f;
-        for (int s = 0; s < n_splits; ++s)
-            if (ml[s].y > 0.f) a += exp2f(ml[s].x - m) * part_o[(row * n_splits + s) * hd + d];
+#pragma unroll 8
+        for (int s = 0; s < n_splits; ++s) a += wgt[s] * po[(long)s * hd + d];
         out[row * hd + d] = f32_to_bf16(a * inv);
     }
 }
@@ -286,29 +379,38 @@ extern "C" const char* cpmcu_attention_mfma(const void* q, void* out, float* par
                                             const int* page_table, int table_width, int page_size,
                                             const int* positions, const int* tok_slot, const int* sel_blocks,
                                             const int* sel_count, int max_sel, int block_size, int n_splits,
-                                            hipStream_t stream) {
+                                            int waves_per_group, hipStream_t stream) {
     CPMCU_REQUIRE(n > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_mfma: bad shape n=%d heads=%d kv_heads=%d", n, nh, nkv);
     CPMCU_REQUIRE(hd == 16 || hd == 32 || hd == 64 || hd == 128,
                   "attention_mfma: head_dim %d has no matrix-core kernel (16, 32, 64, 128 have; the plain kernel takes the rest)", hd);
     CPMCU_REQUIRE(page_size % 32 == 0, "attention_mfma: a cache page of %d tokens is not a multiple of 32", page_size);
     CPMCU_REQUIRE(!sel_count || (sel_blocks && max_sel > 0 && block_size > 0 && block_size % 32 == 0),
                   "attention_mfma: key blocks of %d tokens are not a multiple of 32", block_size);
-    CPMCU_REQUIRE(n_splits >= 1 && n_splits <= 65535 && (n_splits == 1 || (part_o && part_ml)), "attention_mfma: bad split %d", n_splits);
+    CPMCU_REQUIRE(n_splits >= 1 && n_splits <= 64 && (n_splits == 1 || (part_o && part_ml)),
+                  "attention_mfma: %d shares of the keys (1..64 are taken)", n_splits);
     const int G = nh / nkv;
     const int HT = (G + 15) / 16;
     CPMCU_REQUIRE((long)nkv * HT <= 65535, "attention_mfma: too many head tiles");
     PagedView pv{page_table, table_width, page_size};
     dim3 grid(n, nkv * HT, n_splits);
     const float sl = scale * 1.4426950408889634f;
-#define LAUNCH(HDv)                                                                                                \
-    attention_mfma_kernel<HDv><<<grid, 64, 0, stream>>>((const bf16_t*)q, (bf16_t*)out, part_o, (float2*)part_ml,  \
-                                                        (const bf16_t*)kpool, (const bf16_t*)vtpool, pv, positions, \
-                                                        tok_slot, nh, nkv, sl, sel_blocks, sel_count, max_sel,    \
-                                                        block_size, n_splits)
-    if (hd == 16) LAUNCH(16);
-    else if (hd == 32) LAUNCH(32);
-    else if (hd == 64) LAUNCH(64);
-    else LAUNCH(128);
+    // few tokens (decode steps): 4 wavefronts share a workgroup's keys; many tokens (prompts): one each
+    const int nw = waves_per_group > 0 ? waves_per_group : (n <= 256 ? 4 : 1);
+    CPMCU_REQUIRE(nw == 1 || nw == 4, "attention_mfma: %d wavefronts a workgroup (1 or 4 are built)", nw);
+#define LAUNCH(HDv, NWv)                                                                                           \
+    attention_mfma_kernel<HDv, NWv><<<grid, NWv * 64, 0, stream>>>(                                               \
+        (const bf16_t*)q, (bf16_t*)out, part_o, (float2*)part_ml, (const bf16_t*)kpool, (const bf16_t*)vtpool, pv, \
+        positions, tok_slot, nh, nkv, sl, sel_blocks, sel_count, max_sel, block_size, n_splits)
+#define BY_NW(HDv)                 \
+    do {                           \
+        if (nw == 4) LAUNCH(HDv, 4); \
+        else LAUNCH(HDv, 1);       \
+    } while (0)
+    if (hd == 16) BY_NW(16);
+    else if (hd == 32) BY_NW(32);
+    else if (hd == 64) BY_NW(64);
+    else BY_NW(128);
+#undef BY_NW
 #undef LAUNCH
     CPMCU_LAUNCH_CHECK("attention_mfma");
     if (n_splits > 1) {

@@ -73,11 +73,74 @@ __global__ void add_rms_norm_kernel(float* __restrict__ x, const BT* __restrict_
     }
 }
 
+// The same with 4 columns a thread and 16-byte accesses (H a multiple of 4, float branch or none):
+// the decode steps' norms have few rows and up to 16 partial sums to add, so the row's work
+// is spread over up to 1024 threads.
+template <typename OT>
+__global__ __launch_bounds__(1024) void add_rms_norm_vec4_kernel(float* __restrict__ x, const float* __restrict__ branch,
+                                                                 int nparts, long part_stride, float bscale,
+                                                                 const float* __restrict__ w, float eps,
+                                                                 OT* __restrict__ out, const int* __restrict__ rows, int H) {
+    __shared__ float red[17];
+    const long r_out = blockIdx.x;
+    const long r = rows ? rows[r_out] : r_out;
+    float* xr = x + r * H;
+    const int H4 = H / 4;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < H4; c += blockDim.x) {
+        float4 v = *(const float4*)(xr + 4 * c);
+        if (branch) {
+            float4 b = make_float4(0.f, 0.f, 0.f, 0.f);
+            for (int p = 0; p < nparts; ++p) {
+                const float4 t = *(const float4*)(branch + p * part_stride + r * H + 4 * c);
+                b.x += t.x; b.y += t.y; b.z += t.z; b.w += t.w;
+            }
+            v.x += bscale * b.x; v.y += bscale * b.y; v.z += bscale * b.z; v.w += bscale * b.w;
+            if (!rows) *(float4*)(xr + 4 * c) = v;
+        }
+        ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+    }
+    ss = block_sum(ss, red);
+    const float rs = 1.0f / sqrtf(ss / (float)H + eps);
+    OT* o = out + r_out * H;
+    for (int c = threadIdx.x; c < H4; c += blockDim.x) {
+        float4 v = *(const float4*)(xr + 4 * c);
+        if (branch && rows) {
+            float4 b = make_float4(0.f, 0.f, 0.f, 0.f);
+            for (int p = 0; p < nparts; ++p) {
+                const float4 t = *(const float4*)(branch + p * part_stride + r * H + 4 * c);
+                b.x += t.x; b.y += t.y; b.z += t.z; b.w += t.w;
+            }
+            v.x += bscale * b.x; v.y += bscale * b.y; v.z += bscale * b.z; v.w += bscale * b.w;
+        }
+        const float4 wv = *(const float4*)(w + 4 * c);
+        o[4 * c + 0] = from_f32<OT>(v.x * rs * wv.x);
+        o[4 * c + 1] = from_f32<OT>(v.y * rs * wv.y);
+        o[4 * c + 2] = from_f32<OT>(v.z * rs * wv.z);
+        o[4 * c + 3] = from_f32<OT>(v.w * rs * wv.w);
+    }
+}
+
 extern "C" const char* cpmcu_add_rms_norm(float* x, const void* branch, int branch_dtype, int nparts,
                                           long part_stride, float bscale, const float* w, float eps, void* out,
                                           int out_dtype, const int* rows, int n_out, int H, hipStream_t stream) {
     CPMCU_REQUIRE(n_out > 0 && H > 0, "add_rms_norm: empty shape rows=%d H=%d", n_out, H);
     CPMCU_REQUIRE(!branch || nparts >= 1, "add_rms_norm: nparts=%d", nparts);
+    if (H % 4 == 0 && (!branch || branch_dtype == CPMCU_F32) && ((uintptr_t)x % 16 == 0) &&
+        (!branch || ((uintptr_t)branch % 16 == 0 && part_stride % 4 == 0)) && ((uintptr_t)w % 16 == 0)) {
+        const int h4 = H / 4;
+        const int vblock = h4 >= 1024 ? 1024 : (h4 >= 512 ? 512 : (h4 >= 256 ? 256 : (h4 >= 128 ? 128 : 64)));
+        if (out_dtype == CPMCU_F32)
+            add_rms_norm_vec4_kernel<float><<<n_out, vblock, 0, stream>>>(x, (const float*)branch, nparts, part_stride,
+                                                                          bscale, w, eps, (float*)out, rows, H);
+        else if (out_dtype == CPMCU_BF16)
+            add_rms_norm_vec4_kernel<bf16_t><<<n_out, vblock, 0, stream>>>(x, (const float*)branch, nparts, part_stride,
+                                                                           bscale, w, eps, (bf16_t*)out, rows, H);
+        else
+            CPMCU_FAIL("add_rms_norm: unknown output dtype %d", out_dtype);
+        CPMCU_LAUNCH_CHECK("add_rms_norm");
+        return nullptr;
+    }
     const int block = H >= 2048 ? 512 : (H >= 512 ? 256 : 64);
 #define LAUNCH(BT, OT)                                                                                         \
     add_rms_norm_kernel<BT, OT><<<n_out, block, 0, stream>>>(x, (const BT*)branch, nparts, part_stride, bscale, \
@@ -138,47 +201,40 @@ __global__ void rope_store_kernel(const IT* __restrict__ qkv, long width, int np
                                   T* __restrict__ q_out, int nh, int nkv, int hd, const int* __restrict__ positions,
                                   const int* __restrict__ tok_slot, const float* __restrict__ inv_freq, float mscale,
                                   T* __restrict__ kpool, T* __restrict__ vpool, PagedView pv, int write_kv) {
+    // one block per (token, head): heads [0, nh) are queries, then nkv key heads, then nkv value heads
     const long t = blockIdx.x;
+    const int head = blockIdx.y;
     const int half = hd / 2;
     const int pos = positions[t];
-    const IT* row = qkv + t * width;
-    auto load = [&](long i) {
+    const IT* row = qkv + t * width + (long)head * hd;
+    auto load = [&](int i) {
         float s = 0.f;
         for (int p = 0; p < nparts; ++p) s += to_f32(row[p * part_stride + i]);
         return s;
     };
     long kv_row = 0;
-    if (write_kv) kv_row = paged_row(pv, tok_slot[t], pos);
-    const int n_rot = (nh + (write_kv ? nkv : 0)) * half;
-    for (int i = threadIdx.x; i < n_rot; i += blockDim.x) {
-        const int head = i / half, c = i - head * half;
-        float cs = 1.f, sn = 0.f;
-        if (inv_freq) {
-            const float ang = (float)pos * inv_freq[c];
-            cs = cosf(ang) * mscale;
-            sn = sinf(ang) * mscale;
+    if (head >= nh) kv_row = paged_row(pv, tok_slot[t], pos);
+    if (head < nh + nkv) {
+        T* dst = head < nh ? q_out + (t * nh + head) * (long)hd
+                           : kpool + kv_row * (long)nkv * hd + (long)(head - nh) * hd;
+        for (int c = threadIdx.x; c < half; c += blockDim.x) {
+            float cs = 1.f, sn = 0.f;
+            if (inv_freq) {
+                const float ang = (float)pos * inv_freq[c];
+                cs = cosf(ang) * mscale;
+                sn = sinf(ang) * mscale;
+            }
+            const float a = load(c), b = load(c + half);
+            dst[c] = from_f32<T>(a * cs - b * sn);
+            dst[c + half] = from_f32<T>(a * sn + b * cs);
         }
-        const long off = (long)head * hd + c;
-        const float a = load(off), b = load(off + half);
-        const float ra = a * cs - b * sn, rb = a * sn + b * cs;
-        if (head < nh) {
-            T* dst = q_out + t * (long)nh * hd + off;
-            dst[0] = from_f32<T>(ra);
-            dst[half] = from_f32<T>(rb);
-        } else {
-            T* dst = kpool + kv_row * (long)nkv * hd + (off - (long)nh * hd);
-            dst[0] = from_f32<T>(ra);
-            dst[half] = from_f32<T>(rb);
-        }
-    }
-    if (write_kv) {
+    } else {
         // values are kept transposed inside a page, [page][kv head][d][token of the page], so that
         // attention reads, for one d, the values of consecutive keys as one vector
-        const long voff = (long)(nh + nkv) * hd;
         const long page = kv_row / pv.page_size;
         const int in_page = (int)(kv_row - page * pv.page_size);
-        T* dst = vpool + page * (long)pv.page_size * nkv * hd + in_page;
-        for (int i = threadIdx.x; i < nkv * hd; i += blockDim.x) dst[(long)i * pv.page_size] = from_f32<T>(load(voff + i));
+        T* dst = vpool + (page * nkv + (head - nh - nkv)) * (long)hd * pv.page_size + in_page;
+        for (int d = threadIdx.x; d < hd; d += blockDim.x) dst[(long)d * pv.page_size] = from_f32<T>(load(d));
     }
 }
 
@@ -196,9 +252,11 @@ extern "C" const char* cpmcu_rope_store(const void* qkv, long row_width, int in_
                   "rope_store: a row of %ld elements cannot hold %d query%s heads of %d", row_width, nh,
                   write_kv ? " and key/value" : "", hd);
     PagedView pv{page_table, table_width, page_size};
-    const int block = 256;
+    const int block = hd >= 128 ? 64 : (hd / 2 > 32 ? 64 : 32);
+    CPMCU_REQUIRE(nh + 2 * nkv <= 65535, "rope_store: %d heads exceed the launch grid", nh + 2 * nkv);
+    dim3 grid(n, nh + (write_kv ? 2 * nkv : 0));
 #define LAUNCH(IT, T)                                                                                          \
-    rope_store_kernel<IT, T><<<n, block, 0, stream>>>((const IT*)qkv, row_width, nparts, part_stride, (T*)q_out, nh, nkv, \
+    rope_store_kernel<IT, T><<<grid, block, 0, stream>>>((const IT*)qkv, row_width, nparts, part_stride, (T*)q_out, nh, nkv, \
                                                       hd, positions, tok_slot, inv_freq, mscale, (T*)kpool,   \
                                                       (T*)vpool, pv, write_kv)
     if (in_dtype == CPMCU_F32 && dtype == CPMCU_F32) LAUNCH(float, float);

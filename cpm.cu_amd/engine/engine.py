@@ -78,6 +78,10 @@ class Engine:
         self._meta = torch.zeros(cap, dtype=torch.int32, device=self.device)
         self.vocab_size = model.vocab_size
         self.steps_run = 0
+        self._graphs: Dict[Tuple[int, int], tuple] = {}
+        self._stage = [torch.empty(cap, dtype=torch.int32).pin_memory() for _ in range(4)]
+        self._stage_ev: List[Optional[torch.cuda.Event]] = [None] * 4
+        self._stage_i = 0
 
     # ------------------------------------------------------------------
     @classmethod
@@ -195,6 +199,8 @@ class Engine:
         B = len(chunk)
         q_lens = [b - a for _, a, b in chunk]
         n = sum(q_lens)
+        single = n == B
+        graph = bool(self.options.hip_graph) and single
         tok = np.empty(n, dtype=np.int32)
         pos = np.empty(n, dtype=np.int32)
         tslot = np.empty(n, dtype=np.int32)
@@ -222,24 +228,74 @@ class Engine:
                         dest.append(r)
             o += q
         cache.sync()
-        R = len(rows)
-        host = np.concatenate([tok, pos, tslot, cu, sslot, slen, np.asarray(rows, dtype=np.int32)])
-        if host.size > self._meta.numel():
-            self._meta = torch.zeros(host.size * 2, dtype=torch.int32, device=self.device)
-        meta = self._meta
-        meta[:host.size].copy_(torch.from_numpy(host))
-        o1, o2, o3 = n, 2 * n, 3 * n
-        o4 = o3 + B + 1
-        o5 = o4 + B
-        o6 = o5 + B
-        ctx = StepContext(
-            n_tokens=n, n_seqs=B, token_ids=meta[0:o1], positions=meta[o1:o2], tok_slot=meta[o2:o3],
-            cu_q=meta[o3:o4], seq_slot=meta[o4:o5], seq_len=meta[o5:o6], q_lens=q_lens,
-            kv_lens=[int(x) for x in slen], max_pos=int(pos.max()), single_token=all(q == 1 for q in q_lens),
-            ws=self.workspace, cache=cache, logit_rows=meta[o6:o6 + R] if R else None)
-        logits = self.model.forward(ctx)
-        if R:
-            result.index_copy_(0, torch.tensor(dest, dtype=torch.long, device=self.device), logits)
+        max_pos = int(pos.max())
+        if graph:
+            # a captured step computes the logits of all its rows, and sizes its launches for the largest
+            # position of a whole range of steps, so that one capture serves all of them
+            bound = 256
+            while bound < max_pos + 1:
+                bound *= 2
+            max_pos = min(bound, self.max_seq_len) - 1
+            want_rows = np.arange(B, dtype=np.int32)
+        else:
+            want_rows = np.asarray(rows, dtype=np.int32)
+        R = int(want_rows.size)
+        host = np.concatenate([tok, pos, tslot, cu, sslot, slen, want_rows])
+        key = (B, max_pos)
+        entry = self._graphs.get(key) if graph else None
+        if entry is not None and entry[3] != self.workspace.generation:
+            self._graphs.clear()            # scratch buffers moved: what was captured points at freed memory
+            entry = None
+        if graph:
+            meta = entry[1] if entry is not None else torch.zeros(host.size, dtype=torch.int32, device=self.device)
+        else:
+            if host.size > self._meta.numel():
+                self._meta = torch.zeros(host.size * 2, dtype=torch.int32, device=self.device)
+            meta = self._meta
+        self._upload(host, meta)
+        if entry is not None:
+            entry[0].replay()
+            logits = entry[2]
+        else:
+            o1, o2, o3 = n, 2 * n, 3 * n
+            o4 = o3 + B + 1
+            o5 = o4 + B
+            o6 = o5 + B
+            ctx = StepContext(
+                n_tokens=n, n_seqs=B, token_ids=meta[0:o1], positions=meta[o1:o2], tok_slot=meta[o2:o3],
+                cu_q=meta[o3:o4], seq_slot=meta[o4:o5], seq_len=meta[o5:o6], q_lens=q_lens,
+                kv_lens=[int(x) for x in slen], max_pos=max_pos, single_token=single,
+                ws=self.workspace, cache=cache, logit_rows=meta[o6:o6 + R] if R else None)
+            logits = self.model.forward(ctx)
+            if graph:
+                # the eager run above did this step's work and sized the scratch buffers; recording the same
+                # launches executes nothing and serves the following steps of this batch size
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    captured = self.model.forward(ctx)
+                self._graphs[key] = (g, meta, captured, self.workspace.generation)
+        if rows:
+            dest_t = torch.tensor([dest, rows], dtype=torch.long).to(self.device, non_blocking=True)
+            if graph:
+                result.index_copy_(0, dest_t[0], logits.index_select(0, dest_t[1]))
+            else:
+                result.index_copy_(0, dest_t[0], logits)
+
+    def _upload(self, host: np.ndarray, dst: torch.Tensor):
+        """Step metadata to the device through pinned memory, without waiting for the GPU."""
+        if host.size > self._stage[0].numel():
+            self._stage = [torch.empty(host.size * 2, dtype=torch.int32).pin_memory() for _ in self._stage]
+            self._stage_ev = [None] * len(self._stage)
+        i = self._stage_i
+        self._stage_i = (i + 1) % len(self._stage)
+        if self._stage_ev[i] is not None:
+            self._stage_ev[i].synchronize()      # the copy that last used this staging buffer has finished
+        st = self._stage[i][:host.size]
+        st.numpy()[:] = host
+        dst[:host.size].copy_(st, non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        self._stage_ev[i] = ev
 
     # ------------------------------------------------------------------
     def memory_report(self) -> Dict[str, int]:

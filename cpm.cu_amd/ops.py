@@ -202,7 +202,7 @@ def attention_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hd: in
                    positions: torch.Tensor, tok_slot: torch.Tensor, n_splits: int = 1,
                    part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None,
                    sel_blocks: Optional[torch.Tensor] = None, sel_count: Optional[torch.Tensor] = None,
-                   block_size: int = 0):
+                   block_size: int = 0, waves_per_group: int = 0):
     """bf16 attention on the matrix cores (head_dim 16, 32, 64 or 128; pages and key blocks multiples of 32).
     With n_splits > 1 every token's keys are shared among n_splits wavefronts and merged afterwards;
     part_o float32 [n, nh, n_splits, hd] and part_ml float32 [n, nh, n_splits, 2] are its scratch."""
@@ -225,15 +225,17 @@ def attention_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hd: in
     _check(_fn("attention", "cpmcu_attention_mfma")(
         _p(q), _p(out), _p(part_o), _p(part_ml), c_int(n), c_int(nh), c_int(nkv), c_int(hd), c_float(scale),
         _p(kpool), _p(vpool), _p(page_table), c_int(page_table.shape[1]), c_int(page_size), _p(positions),
-        _p(tok_slot), _p(sel_blocks), _p(sel_count), c_int(max_sel), c_int(block_size), c_int(n_splits), _stream()))
+        _p(tok_slot), _p(sel_blocks), _p(sel_count), c_int(max_sel), c_int(block_size), c_int(n_splits),
+        c_int(waves_per_group), _stream()))
 
 
 def attention_splits(n_tokens: int, nkv: int, group: int, max_keys: int) -> int:
-    """Shares of a token's keys: enough wavefronts (about 2048) to fill 256 CUs when a step has few
-    tokens, each with at least 128 keys."""
-    waves = n_tokens * nkv * -(-group // 16)
-    s = max(1, min(2048 // max(waves, 1), max_keys // 128, 64))
-    return s
+    """Shares of a token's keys for steps of few tokens: about 512 workgroups of 4 wavefronts fill the 256
+    CUs; a share should still hold 512 keys (4 chunks of 32 for each wavefront)."""
+    if n_tokens > 256:
+        return 1
+    groups = n_tokens * nkv * -(-group // 16)
+    return max(1, min(512 // max(groups, 1), max_keys // 512, 64))
 
 
 def compress_keys(kpool: torch.Tensor, ckpool: torch.Tensor, page_table: torch.Tensor, page_size: int,

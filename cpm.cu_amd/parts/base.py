@@ -56,6 +56,7 @@ class Workspace:
     def __init__(self, device):
         self.device = torch.device(device)
         self._buf: Dict[str, torch.Tensor] = {}
+        self.generation = 0           # counts the times a buffer moved (captured graphs hold the old address)
 
     def get(self, name: str, shape: Sequence[int], dtype: torch.dtype) -> torch.Tensor:
         n = 1
@@ -64,6 +65,8 @@ class Workspace:
         nbytes = n * torch.empty((), dtype=dtype).element_size()
         buf = self._buf.get(name)
         if buf is None or buf.numel() < nbytes:
+            if buf is not None:
+                self.generation += 1
             buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=self.device)
             self._buf[name] = buf
         return buf[:nbytes].view(dtype).view(*shape)

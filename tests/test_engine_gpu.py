@@ -187,3 +187,20 @@ def test_steps_that_cannot_run_are_refused_and_change_nothing(model_dirs):
     assert eng.step([StepEntry(s, [1, 2, 3], [])]) is None and eng.length(s) == 3
     eng.release(s)
     eng.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_captured_decode_steps_equal_eager_ones(model_dirs, references, name, dtype):
+    """Single-token steps replayed from a captured graph: every replay is checked, with eager work (prompts of
+    other batches, larger batches that move scratch buffers) and synchronisations between the replays."""
+    cfg, w, reqs, refs = references[name]
+    eng = engine_for(model_dirs, name, dtype, hip_graph=True)
+    for rnd_ in range(2):
+        got = schedules.batched(eng, reqs, WORK[name]["prompt"], BATCHES[:2] if rnd_ == 0 else BATCHES[2:])
+        check(got, refs, dtype, f"graph round {rnd_}")
+        torch.cuda.synchronize()
+    assert eng._graphs, "no decode step was captured"
+    got = schedules.tail(eng, {"d": reqs["d"]}, 40)
+    check(got, {"d": refs["d"]}, dtype, "graph tail")
+    eng.cache.check()

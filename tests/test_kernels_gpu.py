@@ -210,13 +210,13 @@ def test_attention_over_scrambled_pages(nh, nkv, hd, dtype):
     ops.attention_plain(q.view(n, -1), out, nh, nkv, hd, scale, kpool, vpool, table, page, pos_t, slot_t)
     assert float((out.double().cpu().view(n, nh, hd) - ref).abs().max()) <= tol
     if dtype == torch.bfloat16 and hd in ops.MFMA_HEAD_DIMS:
-        for splits in (1, 3, 8):
+        for splits, nw in ((1, 1), (1, 4), (3, 1), (3, 4), (8, 4)):
             out.fill_(float("nan"))
             po = torch.full((n, nh, splits, hd), float("nan"), device=DEV) if splits > 1 else None
             pm = torch.full((n, nh, splits, 2), float("nan"), device=DEV) if splits > 1 else None
             ops.attention_mfma(q.view(n, -1), out, nh, nkv, hd, scale, kpool, vpool, table, page, pos_t, slot_t,
-                               splits, po, pm)
-            assert float((out.double().cpu().view(n, nh, hd) - ref).abs().max()) <= tol, f"splits={splits}"
+                               splits, po, pm, waves_per_group=nw)
+            assert float((out.double().cpu().view(n, nh, hd) - ref).abs().max()) <= tol, f"splits={splits} waves={nw}"
     elif dtype == torch.bfloat16:
         assert not ops.attention_mfma_ok(q.view(n, -1), hd, page)
 
@@ -245,10 +245,11 @@ def test_attention_finds_one_far_key_among_hundreds(dtype):
         ops.attention_plain(qd, out, nh, nkv, hd, hd ** -0.5, kpool, vpool, table, page, pos_t, slot_t)
         outs.append(out.clone())
         if dtype == torch.bfloat16:
-            for splits in (1, 5):
+            for splits, nw in ((1, 1), (1, 4), (5, 4), (5, 1)):
                 po = torch.empty(1, nh, splits, hd, device=DEV)
                 pm = torch.empty(1, nh, splits, 2, device=DEV)
-                ops.attention_mfma(qd, out, nh, nkv, hd, hd ** -0.5, kpool, vpool, table, page, pos_t, slot_t, splits, po, pm)
+                ops.attention_mfma(qd, out, nh, nkv, hd, hd ** -0.5, kpool, vpool, table, page, pos_t, slot_t, splits,
+                                   po, pm, waves_per_group=nw)
                 outs.append(out.clone())
         for o in outs:
             assert float((o.double().cpu().view(nh, hd) - vs[0][far, 0]).abs().max()) < 1e-2, far
@@ -293,9 +294,9 @@ def test_attention_with_block_lists(bs, dtype):
                         sel_blocks.to(DEV), sel_count.to(DEV), bs)
     assert float((out.double().cpu().view(n, nh, hd) - ref).abs().max()) <= tol
     if dtype == torch.bfloat16 and bs % 32 == 0:
-        for splits in (1, 4):
+        for splits, nw in ((1, 1), (4, 4), (1, 4)):
             po = torch.empty(n, nh, splits, hd, device=DEV)
             pm = torch.empty(n, nh, splits, 2, device=DEV)
             ops.attention_mfma(q.view(n, -1), out, nh, nkv, hd, hd ** -0.5, kpool, vpool, table, page, pos_t, slot_t,
-                               splits, po, pm, sel_blocks.to(DEV), sel_count.to(DEV), bs)
+                               splits, po, pm, sel_blocks.to(DEV), sel_count.to(DEV), bs, waves_per_group=nw)
             assert float((out.double().cpu().view(n, nh, hd) - ref).abs().max()) <= tol
