@@ -350,12 +350,27 @@ def skinny_split(M: int, N: int, K: int) -> int:
 # ---------------------------------------------------------------------------
 # dispatchers: choose the kernel for a shape and element type
 # ---------------------------------------------------------------------------
+def library_gemm_ok(x: torch.Tensor, out_dtype: torch.dtype) -> bool:
+    """Many rows in bf16 with bf16 output: the library's matrix product (the reference calls its vendor's
+    library for every linear layer, src/model/linear.cuh:9-37)."""
+    return x.dtype == torch.bfloat16 and out_dtype == torch.bfloat16 and x.shape[0] > SKINNY_MAX_ROWS
+
+
 def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, alpha: float = 1.0):
     """out = alpha * x . w^T with the kernel that suits the element type and the number of rows."""
-    if skinny_ok(x, w):
-        gemm_skinny(x, w, out, alpha)
-    else:
-        gemm_nt_plain(x, w, out, alpha)
+    M = x.shape[0]
+    if x.dtype == torch.bfloat16 and x.shape[1] % 8 == 0:
+        if M <= SKINNY_MAX_ROWS:
+            gemm_skinny(x, w, out, alpha)
+            return
+        if out.dtype == torch.bfloat16 and alpha == 1.0:
+            torch.mm(x, w.t(), out=out)
+            return
+        # float output for many rows (logits of many positions): the skinny kernel, 64 rows at a time
+        for r in range(0, M, SKINNY_MAX_ROWS):
+            gemm_skinny(x[r:r + SKINNY_MAX_ROWS], w, out[r:r + SKINNY_MAX_ROWS], alpha)
+        return
+    gemm_nt_plain(x, w, out, alpha)
 
 
 def attention(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, ctx,

@@ -45,7 +45,10 @@ class Linear(Part):
                 out = ctx.ws.get(tag, (S, n, N), torch.float32)
                 ops.gemm_skinny(x, w, out, alpha, mode="partial")
                 return out
-        out = ctx.ws.get(tag, (n, N), out_dtype or x.dtype)
+        out_dtype = out_dtype or x.dtype
+        if partials and alpha == 1.0 and ops.library_gemm_ok(x, x.dtype):
+            out_dtype = x.dtype         # many rows: the branch comes back in bf16 from the library product
+        out = ctx.ws.get(tag, (n, N), out_dtype)
         ops.linear(x, w, out, alpha)
         return out
 
