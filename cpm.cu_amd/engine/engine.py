@@ -41,6 +41,7 @@ class EngineOptions:
     device: str = "cuda:0"
     hip_graph: bool = False                 # replay single-token steps from a captured graph
     sparse: bool = True                     # honour sparse_config (False: dense attention everywhere)
+    tiled_weights: bool = True              # second copy of the linear weights laid out for decode steps (bf16)
 
 
 @dataclass
@@ -66,7 +67,7 @@ class Engine:
         max_seq_len = options.max_seq_len or getattr(config, "max_position_embeddings", None) or options.max_tokens
         self.max_seq_len = int(max_seq_len)
         self.workspace = Workspace(self.device)
-        self.runtime = Runtime(self.device, self.dtype, self.workspace, self.max_seq_len)
+        self.runtime = Runtime(self.device, self.dtype, self.workspace, self.max_seq_len, options.tiled_weights)
         with torch.cuda.device(self.device):
             model.bind_all(tensors, self.runtime)
         n_pages = -(-options.max_tokens // options.page_size)

@@ -300,14 +300,38 @@ def sample(logits: torch.Tensor, temperature: float, seed: int, request_ids: tor
                                        _p(u_out), _stream()))
 
 
-def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, alpha: float = 1.0, mode: str = "plain"):
-    """bf16 product for at most 64 rows of x on the matrix cores, streaming w once.
+class TiledWeight:
+    """A weight [N, K] re-laid for the skinny product: [strip of 16 rows][K-block of 128][MFMA i][lane][8],
+    lane = 16*g + r holding row 16*strip + r, columns 128*block + 32*i + 8*g .. +8; zero padded."""
+
+    def __init__(self, w: torch.Tensor):
+        _need(w, "weight to tile", torch.bfloat16, (None, None))
+        N, K = w.shape
+        Np, Kp = -(-N // 16) * 16, -(-K // 128) * 128
+        if (Np, Kp) != (N, K):
+            wp = torch.zeros((Np, Kp), dtype=w.dtype, device=w.device)
+            wp[:N, :K] = w
+        else:
+            wp = w
+        self.data = wp.view(Np // 16, 16, Kp // 128, 4, 4, 8).permute(0, 2, 3, 4, 1, 5).contiguous()
+        self.N, self.K = N, K
+
+
+def gemm_skinny(x: torch.Tensor, w, out: torch.Tensor, alpha: float = 1.0, mode: str = "plain"):
+    """bf16 product for at most 64 rows of x on the matrix cores, streaming w once; w is [N, K] as in the
+    checkpoint or a TiledWeight.
     mode 'plain': out [m,N] float32 or bfloat16; 'partial': out float32 [S,m,N], S slices of K to be summed by
     the consumer; 'gated': w holds gate rows then up rows, out bfloat16 [m,N/2] = silu(gate) * up."""
     _need(x, "gemm x", torch.bfloat16, (None, None))
     M, K = x.shape
-    _need(w, "gemm weight", torch.bfloat16, (None, K))
-    N = w.shape[0]
+    tiled = isinstance(w, TiledWeight)
+    if tiled:
+        if w.K != K:
+            raise KernelError(f"gemm weight: tiled for K={w.K}, x has {K} columns")
+        N, wt = w.N, w.data
+    else:
+        _need(w, "gemm weight", torch.bfloat16, (None, K))
+        N, wt = w.shape[0], w
     ksplit, omode = 1, 0
     if mode == "plain":
         _need(out, "gemm out", shape=(M, N))
@@ -320,15 +344,15 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, alpha: floa
         omode, ldy = 2, N // 2
     else:
         raise KernelError(f"gemm_skinny: unknown mode '{mode}'")
-    _check(_fn("gemm", "cpmcu_gemm_skinny")(_p(x), c_long(K), _p(w), c_long(K), _p(out), c_long(ldy),
+    _check(_fn("gemm", "cpmcu_gemm_skinny")(_p(x), c_long(K), _p(wt), c_long(K), _p(out), c_long(ldy),
                                             c_int(_code(out)), c_int(omode), c_int(M), c_int(N), c_int(K),
-                                            c_int(ksplit), c_float(alpha), _stream()))
+                                            c_int(ksplit), c_float(alpha), c_int(1 if tiled else 0), _stream()))
 
 
 SKINNY_MAX_ROWS = 64
 
 
-def skinny_ok(x: torch.Tensor, w: torch.Tensor) -> bool:
+def skinny_ok(x: torch.Tensor, w=None) -> bool:
     return x.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 8 == 0
 
 
@@ -356,19 +380,19 @@ def library_gemm_ok(x: torch.Tensor, out_dtype: torch.dtype) -> bool:
     return x.dtype == torch.bfloat16 and out_dtype == torch.bfloat16 and x.shape[0] > SKINNY_MAX_ROWS
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, alpha: float = 1.0):
+def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, alpha: float = 1.0, w_tiled=None):
     """out = alpha * x . w^T with the kernel that suits the element type and the number of rows."""
     M = x.shape[0]
     if x.dtype == torch.bfloat16 and x.shape[1] % 8 == 0:
         if M <= SKINNY_MAX_ROWS:
-            gemm_skinny(x, w, out, alpha)
+            gemm_skinny(x, w_tiled if w_tiled is not None else w, out, alpha)
             return
         if out.dtype == torch.bfloat16 and alpha == 1.0:
             torch.mm(x, w.t(), out=out)
             return
         # float output for many rows (logits of many positions): the skinny kernel, 64 rows at a time
         for r in range(0, M, SKINNY_MAX_ROWS):
-            gemm_skinny(x[r:r + SKINNY_MAX_ROWS], w, out[r:r + SKINNY_MAX_ROWS], alpha)
+            gemm_skinny(x[r:r + SKINNY_MAX_ROWS], w_tiled if w_tiled is not None else w, out[r:r + SKINNY_MAX_ROWS], alpha)
         return
     gemm_nt_plain(x, w, out, alpha)
 

@@ -82,6 +82,7 @@ class Runtime:
     dtype: torch.dtype            # element type of activations, weights and cache: float32 or bfloat16
     workspace: Workspace
     max_seq_len: int              # longest sequence the engine holds
+    tiled_weights: bool = True    # keep a second copy of linear weights in the decode product's layout
 
 
 @dataclass

@@ -50,9 +50,13 @@ class LMHead(Part):
     def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime):
         if self.tied_to is None:
             self.weight = tensors[self.name].to(rt.dtype).contiguous()
+        self.rt = rt
+        self.tiled = None
 
     def forward(self, y: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         w = self.tied_to.table if self.tied_to is not None else self.weight
+        if self.tiled is None and self.rt.dtype == torch.bfloat16 and self.rt.tiled_weights:
+            self.tiled = ops.TiledWeight(w)
         logits = ctx.ws.get("logits", (y.shape[0], self.vocab_size), torch.float32)
-        ops.linear(y, w, logits, self.scale)
+        ops.linear(y, w, logits, self.scale, w_tiled=self.tiled)
         return logits

@@ -31,6 +31,8 @@ class Linear(Part):
         w = ws[0] if len(ws) == 1 else torch.cat(ws, dim=0)
         self.weight = w.to(rt.dtype).contiguous()
         self.rt = rt
+        # a second copy laid out for the decode product (bf16 engine; costs the weight's size again)
+        self.tiled = ops.TiledWeight(self.weight) if (rt.dtype == torch.bfloat16 and rt.tiled_weights) else None
 
     def forward(self, x: torch.Tensor, ctx: StepContext, tag: str, out_dtype: Optional[torch.dtype] = None,
                 alpha: float = 1.0, rows: Optional[int] = None, partials: bool = False) -> torch.Tensor:
@@ -38,26 +40,27 @@ class Linear(Part):
         result may come as float32 partial sums [S, n, out] over slices of the input axis, for a consumer
         that adds them up (the norm and the position-encoding kernels do)."""
         w = self.weight if rows is None else self.weight[:rows]
+        wt = self.tiled if rows is None else None
         n, N = x.shape[0], w.shape[0]
-        if partials and ops.skinny_ok(x, w):
+        if partials and ops.skinny_ok(x):
             S = ops.skinny_split(n, N, self.in_features)
             if S > 1:
                 out = ctx.ws.get(tag, (S, n, N), torch.float32)
-                ops.gemm_skinny(x, w, out, alpha, mode="partial")
+                ops.gemm_skinny(x, wt if wt is not None else w, out, alpha, mode="partial")
                 return out
         out_dtype = out_dtype or x.dtype
         if partials and alpha == 1.0 and ops.library_gemm_ok(x, x.dtype):
             out_dtype = x.dtype         # many rows: the branch comes back in bf16 from the library product
         out = ctx.ws.get(tag, (n, N), out_dtype)
-        ops.linear(x, w, out, alpha)
+        ops.linear(x, w, out, alpha, w_tiled=wt)
         return out
 
     def forward_gated(self, x: torch.Tensor, ctx: StepContext, tag: str) -> torch.Tensor:
         """For a weight of gate rows stacked on up rows: silu(x Wg^T) * (x Wu^T), [n, out/2]."""
         n, half = x.shape[0], self.out_features // 2
         act = ctx.ws.get(tag + ".act", (n, half), x.dtype)
-        if ops.skinny_ok(x, self.weight):
-            ops.gemm_skinny(x, self.weight, act, mode="gated")
+        if ops.skinny_ok(x) and (self.tiled is None or half % 16 == 0):
+            ops.gemm_skinny(x, self.tiled if self.tiled is not None else self.weight, act, mode="gated")
         else:
             gu = self.forward(x, ctx, tag)
             ops.silu_mul(gu, act)

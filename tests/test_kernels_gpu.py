@@ -57,6 +57,20 @@ def test_skinny_product_all_modes(M, N, K):
         ops.gemm_skinny(x, w, act, mode="gated")
         want = F.silu(ref[:, :I]) * ref[:, I:]
         assert float((act.double() - want).abs().max()) <= 2 ** -8 * float(want.abs().max()) + tol
+    # the same from the weight re-laid for this kernel
+    wt = ops.TiledWeight(w)
+    out.fill_(float("nan"))
+    ops.gemm_skinny(x, wt, out, 0.25)
+    assert float((out.double() - 0.25 * ref).abs().max()) <= tol
+    ks = -(-(-(-K // 2)) // 128) * 128
+    part = torch.full((-(-K // ks), M, N), float("nan"), dtype=torch.float32, device=DEV)
+    ops.gemm_skinny(x, wt, part, 1.0, mode="partial")
+    assert float((part.double().sum(0) - ref).abs().max()) <= tol
+    if N % 32 == 0:
+        act = torch.full((M, N // 2), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.gemm_skinny(x, wt, act, mode="gated")
+        want = F.silu(ref[:, :N // 2]) * ref[:, N // 2:]
+        assert float((act.double() - want).abs().max()) <= 2 ** -8 * float(want.abs().max()) + tol
 
 
 def test_skinny_split_heuristic_matches_what_the_kernel_accepts():
