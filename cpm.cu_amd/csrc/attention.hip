@@ -420,3 +420,205 @@ extern "C" const char* cpmcu_attention_mfma(const void* q, void* out, float* par
     }
     return nullptr;
 }
+
+// ===========================================================================
+// bf16 attention for prompts on the matrix cores (dense, causal).
+//
+// One wavefront owns R row tiles of 16 rows for one kv head: a row is one
+// (token, query head) pair, a tile holds the grouped heads of one token (or of
+// several tokens when the group is smaller than 16), and the tokens of a
+// wavefront are consecutive positions of one sequence.  For every chunk of 32
+// keys the K and V^T operands are loaded once and used by all R tiles, which
+// divides the cache traffic of a prompt by the tokens a wavefront holds.  The
+// arithmetic of a tile is that of attention_mfma_kernel; the causal mask is per
+// row, and a tile is skipped for chunks that lie behind all of its rows.
+// `tiles` holds, per wavefront, the first packed token and the number of tokens.
+// ===========================================================================
+template <int HD, int R>
+__global__ __launch_bounds__(64) void attention_prefill_mfma_kernel(
+    const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ kpool,
+    const bf16_t* __restrict__ vtpool, PagedView pv, const int* __restrict__ tiles,
+    const int* __restrict__ positions, const int* __restrict__ tok_slot, int nh, int nkv, float scale_log2e,
+    int rows_per_token, int tokens_per_tile) {
+    constexpr int KSTEPS = (HD + 31) / 32;
+    constexpr int DT = HD / 16;
+    const int tile_id = blockIdx.x;
+    const int kvh = blockIdx.y % nkv, ht = blockIdx.y / nkv;
+    const int lane = threadIdx.x, n = lane & 15, g = lane >> 4;
+    const int G = nh / nkv;
+    const int t0 = tiles[2 * tile_id], n_tok = tiles[2 * tile_id + 1];
+    const int slot = tok_slot[t0];
+    const int* ptab = pv.page_table + (long)slot * pv.table_width;
+    const int pos0 = positions[t0];
+
+    // this lane's row in each tile: token and head; rows beyond the tile's tokens repeat its first token
+    int row_tok[R], row_pos[R], row_head[R];
+    bool row_ok[R];
+    int tile_last_pos[R];
+    abf16x8_t qf[R][KSTEPS];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int tk = r * tokens_per_tile + n / rows_per_token;
+        const int hh = ht * 16 + n % rows_per_token;        // head inside the group (rows_per_token = min(G,16) or 16)
+        const bool ok = tk < n_tok && hh < G && (n / rows_per_token) < tokens_per_tile;
+        row_ok[r] = ok;
+        row_tok[r] = t0 + (tk < n_tok ? tk : 0);
+        row_pos[r] = pos0 + (tk < n_tok ? tk : 0);
+        row_head[r] = kvh * G + (hh < G ? hh : 0);
+        tile_last_pos[r] = pos0 + min((r + 1) * tokens_per_tile, n_tok) - 1;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+            abf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+            const int d = ks * 32 + g * 8;
+            if (d < HD) v = *(const abf16x8_t*)(q + ((long)row_tok[r] * nh + row_head[r]) * HD + d);
+            qf[r][ks] = v;
+        }
+    }
+    const int n_tiles_used = (n_tok + tokens_per_tile - 1) / tokens_per_tile;
+    const int last_pos = pos0 + n_tok - 1;
+    const int total_chunks = last_pos / 32 + 1;
+
+    afloatx4_t acc[R][DT];
+    float m[R], l[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        m[r] = -INFINITY;
+        l[r] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) acc[r][dt] = afloatx4_t{0.f, 0.f, 0.f, 0.f};
+    }
+    const long kv_width = (long)nkv * HD;
+    auto load_k = [&](int page, int po, abf16x8_t (&kf)[2][KSTEPS]) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const long krow = (long)page * pv.page_size + po + n + 4 * (n >> 2) + 4 * u;
+            const bf16_t* kp = kpool + krow * kv_width + (long)kvh * HD + g * 8;
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks) {
+                abf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+                if (ks * 32 + g * 8 < HD) v = *(const abf16x8_t*)(kp + ks * 32);
+                kf[u][ks] = v;
+            }
+        }
+    };
+    abf16x8_t kf[2][KSTEPS];
+    int page = ptab[0], po = 0;
+    load_k(page, po, kf);
+    for (int c = 0; c < total_chunks; ++c) {
+        const int key0 = c * 32;
+        abf16x8_t vf[DT];
+        {
+            const bf16_t* vp = vtpool + (((long)page * nkv + kvh) * HD + n) * pv.page_size + po + g * 8;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const abf16x8_t*)(vp + (long)dt * 16 * pv.page_size);
+        }
+        abf16x8_t kn[2][KSTEPS];
+        int pagen = 0, pon = 0;
+        if (c + 1 < total_chunks) {
+            pagen = ptab[(key0 + 32) / pv.page_size];
+            pon = (key0 + 32) % pv.page_size;
+            load_k(pagen, pon, kn);
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if (r >= n_tiles_used || key0 > tile_last_pos[r]) continue;
+            afloatx4_t st[2];
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                st[u] = afloatx4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < KSTEPS; ++ks)
+                    st[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][ks], qf[r][ks], st[u], 0, 0, 0);
+            }
+            float sc[8];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int key = key0 + 8 * g + 4 * u + i;
+                    const float v = key <= row_pos[r] ? st[u][i] * scale_log2e : -INFINITY;
+                    sc[u * 4 + i] = v;
+                    mx = fmaxf(mx, v);
+                }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            // a row whose position lies before this chunk sees none of its keys: nothing changes for it
+            const float m_new = fmaxf(m[r], mx);
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;
+            const float corr = exp2f(m[r] - m_use);
+            float rs = 0.f;
+            abf16x8_t pb;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float p = exp2f(sc[j] - m_use);
+                rs += p;
+                pb[j] = (__bf16)p;
+            }
+            rs += __shfl_xor(rs, 16, 64);
+            rs += __shfl_xor(rs, 32, 64);
+            l[r] = l[r] * corr + rs;
+            m[r] = m_new;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[r][dt][i] *= corr;
+                acc[r][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pb, acc[r][dt], 0, 0, 0);
+            }
+        }
+        page = pagen;
+        po = pon;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks) kf[u][ks] = kn[u][ks];
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        if (!row_ok[r]) continue;
+        const float inv = 1.0f / l[r];
+        bf16_t* o = out + ((long)row_tok[r] * nh + row_head[r]) * HD;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o[dt * 16 + 4 * g + i] = f32_to_bf16(acc[r][dt][i] * inv);
+    }
+}
+
+extern "C" int cpmcu_attention_prefill_tokens_per_wave(int nh, int nkv) {
+    const int G = nh / nkv;
+    const int rpt = (G < 16 && 16 % G == 0) ? G : 16;
+    return 4 * (16 / rpt);
+}
+
+// tiles: int32 [n_tiles, 2] = (first packed token, tokens) with tokens <= cpmcu_attention_prefill_tokens_per_wave
+extern "C" const char* cpmcu_attention_prefill_mfma(const void* q, void* out, int n_tiles, const int* tiles, int nh,
+                                                    int nkv, int hd, float scale, const void* kpool,
+                                                    const void* vtpool, const int* page_table, int table_width,
+                                                    int page_size, const int* positions, const int* tok_slot,
+                                                    hipStream_t stream) {
+    CPMCU_REQUIRE(n_tiles > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_prefill: bad shape tiles=%d heads=%d kv_heads=%d", n_tiles, nh, nkv);
+    CPMCU_REQUIRE(hd == 16 || hd == 32 || hd == 64 || hd == 128,
+                  "attention_prefill: head_dim %d has no matrix-core kernel (16, 32, 64, 128 have)", hd);
+    CPMCU_REQUIRE(page_size % 32 == 0, "attention_prefill: a cache page of %d tokens is not a multiple of 32", page_size);
+    const int G = nh / nkv;
+    const int rpt = (G < 16 && 16 % G == 0) ? G : 16;
+    const int tpt = 16 / rpt;
+    const int HT = (G + 15) / 16;
+    CPMCU_REQUIRE((long)nkv * HT <= 65535, "attention_prefill: too many head tiles");
+    PagedView pv{page_table, table_width, page_size};
+    dim3 grid(n_tiles, nkv * HT);
+    const float sl = scale * 1.4426950408889634f;
+#define LAUNCH(HDv)                                                                                             \
+    attention_prefill_mfma_kernel<HDv, 4><<<grid, 64, 0, stream>>>((const bf16_t*)q, (bf16_t*)out,              \
+                                                                   (const bf16_t*)kpool, (const bf16_t*)vtpool, \
+                                                                   pv, tiles, positions, tok_slot, nh, nkv, sl, \
+                                                                   rpt, tpt)
+    if (hd == 16) LAUNCH(16);
+    else if (hd == 32) LAUNCH(32);
+    else if (hd == 64) LAUNCH(64);
+    else LAUNCH(128);
+#undef LAUNCH
+    CPMCU_LAUNCH_CHECK("attention_prefill_mfma");
+    return nullptr;
+}

@@ -229,6 +229,43 @@ def attention_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hd: in
         c_int(waves_per_group), _stream()))
 
 
+def attention_prefill_tokens_per_wave(nh: int, nkv: int) -> int:
+    lib = _build.load("attention")
+    lib.cpmcu_attention_prefill_tokens_per_wave.restype = c_int
+    return int(lib.cpmcu_attention_prefill_tokens_per_wave(c_int(nh), c_int(nkv)))
+
+
+def attention_prefill_mfma(q: torch.Tensor, out: torch.Tensor, tiles: torch.Tensor, nh: int, nkv: int, hd: int,
+                           scale: float, kpool: torch.Tensor, vpool: torch.Tensor, page_table: torch.Tensor,
+                           page_size: int, positions: torch.Tensor, tok_slot: torch.Tensor):
+    """Dense causal bf16 attention for prompts: tiles int32 [T, 2] = (first packed token, tokens), each a run of
+    consecutive tokens of one sequence, at most attention_prefill_tokens_per_wave(nh, nkv) long."""
+    _need(q, "attention q", torch.bfloat16, (None, nh * hd))
+    n = q.shape[0]
+    _need(out, "attention out", torch.bfloat16, (n, nh * hd))
+    _need(tiles, "attention tiles", torch.int32, (None, 2))
+    _need(kpool, "attention key pool", torch.bfloat16, (None, page_size, nkv * hd))
+    _need(vpool, "attention value pool", torch.bfloat16, tuple(kpool.shape))
+    _need(page_table, "attention page table", torch.int32, (None, None))
+    _need(positions, "attention positions", torch.int32, (n,))
+    _need(tok_slot, "attention token slots", torch.int32, (n,))
+    _check(_fn("attention", "cpmcu_attention_prefill_mfma")(
+        _p(q), _p(out), c_int(tiles.shape[0]), _p(tiles), c_int(nh), c_int(nkv), c_int(hd), c_float(scale),
+        _p(kpool), _p(vpool), _p(page_table), c_int(page_table.shape[1]), c_int(page_size), _p(positions),
+        _p(tok_slot), _stream()))
+
+
+def prefill_tiles(q_lens: Sequence[int], tokens_per_wave: int, device) -> torch.Tensor:
+    """Runs of at most tokens_per_wave consecutive tokens of one sequence, covering the packed batch."""
+    tiles = []
+    start = 0
+    for q in q_lens:
+        for a in range(0, q, tokens_per_wave):
+            tiles.append((start + a, min(tokens_per_wave, q - a)))
+        start += q
+    return torch.tensor(tiles, dtype=torch.int32).to(device)
+
+
 def attention_splits(n_tokens: int, nkv: int, group: int, max_keys: int) -> int:
     """Shares of a token's keys for steps of few tokens: about 512 workgroups of 4 wavefronts fill the 256
     CUs; a share should still hold 512 keys (4 chunks of 32 for each wavefront)."""
@@ -400,6 +437,15 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, alpha: float = 1
 def attention(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, ctx,
               sel_blocks=None, sel_count=None, block_size=0):
     """Attention of the step's queries over the cache, with the kernel that suits the step."""
+    if sel_count is None and not ctx.single_token and attention_mfma_ok(q, hd, page_size):
+        tpw = attention_prefill_tokens_per_wave(nh, nkv)
+        key = ("prefill_tiles", tpw)
+        tiles = ctx.extras.get(key)
+        if tiles is None:
+            tiles = ctx.extras[key] = prefill_tiles(ctx.q_lens, tpw, q.device)
+        attention_prefill_mfma(q, out, tiles, nh, nkv, hd, scale, kpool, vpool, page_table, page_size,
+                               ctx.positions, ctx.tok_slot)
+        return
     if attention_mfma_ok(q, hd, page_size, block_size if sel_count is not None else 0):
         n = q.shape[0]
         keys = ctx.max_pos + 1

@@ -231,8 +231,43 @@ def test_attention_over_scrambled_pages(nh, nkv, hd, dtype):
             ops.attention_mfma(q.view(n, -1), out, nh, nkv, hd, scale, kpool, vpool, table, page, pos_t, slot_t,
                                splits, po, pm, waves_per_group=nw)
             assert float((out.double().cpu().view(n, nh, hd) - ref).abs().max()) <= tol, f"splits={splits} waves={nw}"
+        # the prompt kernel: runs of consecutive tokens of one sequence share a wavefront
+        tpw = ops.attention_prefill_tokens_per_wave(nh, nkv)
+        tiles = ops.prefill_tiles([40, 1, 1], tpw, DEV)
+        out.fill_(float("nan"))
+        ops.attention_prefill_mfma(q.view(n, -1), out, tiles, nh, nkv, hd, scale, kpool, vpool, table, page, pos_t, slot_t)
+        assert float((out.double().cpu().view(n, nh, hd) - ref).abs().max()) <= tol, "prompt kernel"
     elif dtype == torch.bfloat16:
         assert not ops.attention_mfma_ok(q.view(n, -1), hd, page)
+
+
+@pytest.mark.parametrize("nh,nkv,hd", [(16, 1, 64), (8, 1, 32), (4, 2, 128), (5, 5, 16), (40, 2, 32)])
+def test_prompt_attention_from_position_zero_and_continued(nh, nkv, hd):
+    """Whole prompts from position 0 (where early tiles stop before late chunks) and a chunk that continues
+    a sequence already in the cache, several sequences packed."""
+    from cpmcu_amd import ops
+    page, dtype = 64, torch.bfloat16
+    lens = [150, 37, 64]
+    ks, vs, kpool, vpool, table = paged_setup(lens, nkv, hd, page, dtype, seed=nh)
+    starts = [0, 0, 41]                       # the third sequence already holds 41 tokens
+    positions, seq_of, q_lens = [], [], []
+    for s, (L, a) in enumerate(zip(lens, starts)):
+        positions += list(range(a, L))
+        seq_of += [s] * (L - a)
+        q_lens.append(L - a)
+    n = len(positions)
+    q = rnd(n, nh, hd, seed=8, dtype=dtype)
+    scale = hd ** -0.5
+    ref = attention_reference(q.double().cpu(), ks, vs, positions, seq_of, nh, scale)
+    pos_t = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    slot_t = torch.tensor(seq_of, dtype=torch.int32, device=DEV)
+    tiles = ops.prefill_tiles(q_lens, ops.attention_prefill_tokens_per_wave(nh, nkv), DEV)
+    out = torch.full((n, nh * hd), float("nan"), dtype=dtype, device=DEV)
+    ops.attention_prefill_mfma(q.view(n, -1), out, tiles, nh, nkv, hd, scale, kpool, vpool, table, page, pos_t, slot_t)
+    # the output is rounded to bf16 (8 significant bits): allow its half ulp at the size of each token's values
+    err = (out.double().cpu().view(n, nh, hd) - ref).abs().amax(dim=(1, 2))
+    bad = (err > 2 ** -7 * ref.abs().amax(dim=(1, 2)).clamp(min=1.0)).nonzero().flatten()
+    assert bad.numel() == 0, f"first wrong token {int(bad[0])} (position {positions[int(bad[0])]})"
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
