@@ -501,23 +501,26 @@ __global__ __launch_bounds__(64) void attention_prefill_mfma_kernel(
             }
         }
     };
-    abf16x8_t kf[2][KSTEPS];
-    int page = ptab[0], po = 0;
-    load_k(page, po, kf);
+    auto load_v = [&](int page, int po, abf16x8_t (&vf)[DT]) {
+        const bf16_t* vp = vtpool + (((long)page * nkv + kvh) * HD + n) * pv.page_size + po + g * 8;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const abf16x8_t*)(vp + (long)dt * 16 * pv.page_size);
+    };
+    // keys and values of chunk c+1 are asked for before the arithmetic of chunk c
+    abf16x8_t kf[2][KSTEPS], vf[DT];
+    {
+        const int page = ptab[0];
+        load_k(page, 0, kf);
+        load_v(page, 0, vf);
+    }
     for (int c = 0; c < total_chunks; ++c) {
         const int key0 = c * 32;
-        abf16x8_t vf[DT];
-        {
-            const bf16_t* vp = vtpool + (((long)page * nkv + kvh) * HD + n) * pv.page_size + po + g * 8;
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const abf16x8_t*)(vp + (long)dt * 16 * pv.page_size);
-        }
-        abf16x8_t kn[2][KSTEPS];
-        int pagen = 0, pon = 0;
+        abf16x8_t kn[2][KSTEPS], vn[DT];
         if (c + 1 < total_chunks) {
-            pagen = ptab[(key0 + 32) / pv.page_size];
-            pon = (key0 + 32) % pv.page_size;
+            const int pagen = ptab[(key0 + 32) / pv.page_size];
+            const int pon = (key0 + 32) % pv.page_size;
             load_k(pagen, pon, kn);
+            load_v(pagen, pon, vn);
         }
 #pragma unroll
         for (int r = 0; r < R; ++r) {
@@ -566,12 +569,12 @@ __global__ __launch_bounds__(64) void attention_prefill_mfma_kernel(
                 acc[r][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pb, acc[r][dt], 0, 0, 0);
             }
         }
-        page = pagen;
-        po = pon;
 #pragma unroll
         for (int u = 0; u < 2; ++u)
 #pragma unroll
             for (int ks = 0; ks < KSTEPS; ++ks) kf[u][ks] = kn[u][ks];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) vf[dt] = vn[dt];
     }
 #pragma unroll
     for (int r = 0; r < R; ++r) {

@@ -76,8 +76,19 @@ __global__ void add_rms_norm_kernel(float* __restrict__ x, const BT* __restrict_
 // The same with 4 columns a thread and 16-byte accesses (H a multiple of 4, float branch or none):
 // the decode steps' norms have few rows and up to 16 partial sums to add, so the row's work
 // is spread over up to 1024 threads.
-template <typename OT>
-__global__ __launch_bounds__(1024) void add_rms_norm_vec4_kernel(float* __restrict__ x, const float* __restrict__ branch,
+__device__ inline float4 load4(const float* p) { return *(const float4*)p; }
+__device__ inline float4 load4(const bf16_t* p) {
+    const uint2 u = *(const uint2*)p;
+    float4 r;
+    r.x = __uint_as_float(u.x << 16);
+    r.y = __uint_as_float(u.x & 0xffff0000u);
+    r.z = __uint_as_float(u.y << 16);
+    r.w = __uint_as_float(u.y & 0xffff0000u);
+    return r;
+}
+
+template <typename BT, typename OT>
+__global__ __launch_bounds__(1024) void add_rms_norm_vec4_kernel(float* __restrict__ x, const BT* __restrict__ branch,
                                                                  int nparts, long part_stride, float bscale,
                                                                  const float* __restrict__ w, float eps,
                                                                  OT* __restrict__ out, const int* __restrict__ rows, int H) {
@@ -92,7 +103,7 @@ __global__ __launch_bounds__(1024) void add_rms_norm_vec4_kernel(float* __restri
         if (branch) {
             float4 b = make_float4(0.f, 0.f, 0.f, 0.f);
             for (int p = 0; p < nparts; ++p) {
-                const float4 t = *(const float4*)(branch + p * part_stride + r * H + 4 * c);
+                const float4 t = load4(branch + p * part_stride + r * H + 4 * c);
                 b.x += t.x; b.y += t.y; b.z += t.z; b.w += t.w;
             }
             v.x += bscale * b.x; v.y += bscale * b.y; v.z += bscale * b.z; v.w += bscale * b.w;
@@ -108,7 +119,7 @@ __global__ __launch_bounds__(1024) void add_rms_norm_vec4_kernel(float* __restri
         if (branch && rows) {
             float4 b = make_float4(0.f, 0.f, 0.f, 0.f);
             for (int p = 0; p < nparts; ++p) {
-                const float4 t = *(const float4*)(branch + p * part_stride + r * H + 4 * c);
+                const float4 t = load4(branch + p * part_stride + r * H + 4 * c);
                 b.x += t.x; b.y += t.y; b.z += t.z; b.w += t.w;
             }
             v.x += bscale * b.x; v.y += bscale * b.y; v.z += bscale * b.z; v.w += bscale * b.w;
@@ -126,18 +137,22 @@ extern "C" const char* cpmcu_add_rms_norm(float* x, const void* branch, int bran
                                           int out_dtype, const int* rows, int n_out, int H, hipStream_t stream) {
     CPMCU_REQUIRE(n_out > 0 && H > 0, "add_rms_norm: empty shape rows=%d H=%d", n_out, H);
     CPMCU_REQUIRE(!branch || nparts >= 1, "add_rms_norm: nparts=%d", nparts);
-    if (H % 4 == 0 && (!branch || branch_dtype == CPMCU_F32) && ((uintptr_t)x % 16 == 0) &&
-        (!branch || ((uintptr_t)branch % 16 == 0 && part_stride % 4 == 0)) && ((uintptr_t)w % 16 == 0)) {
+    if (H % 4 == 0 && ((uintptr_t)x % 16 == 0) && (!branch || ((uintptr_t)branch % 16 == 0 && part_stride % 4 == 0)) &&
+        ((uintptr_t)w % 16 == 0) && (out_dtype == CPMCU_F32 || out_dtype == CPMCU_BF16) &&
+        (branch_dtype == CPMCU_F32 || branch_dtype == CPMCU_BF16)) {
         const int h4 = H / 4;
-        const int vblock = h4 >= 1024 ? 1024 : (h4 >= 512 ? 512 : (h4 >= 256 ? 256 : (h4 >= 128 ? 128 : 64)));
-        if (out_dtype == CPMCU_F32)
-            add_rms_norm_vec4_kernel<float><<<n_out, vblock, 0, stream>>>(x, (const float*)branch, nparts, part_stride,
-                                                                          bscale, w, eps, (float*)out, rows, H);
-        else if (out_dtype == CPMCU_BF16)
-            add_rms_norm_vec4_kernel<bf16_t><<<n_out, vblock, 0, stream>>>(x, (const float*)branch, nparts, part_stride,
-                                                                           bscale, w, eps, (bf16_t*)out, rows, H);
-        else
-            CPMCU_FAIL("add_rms_norm: unknown output dtype %d", out_dtype);
+        // many rows: smaller blocks keep more rows in flight on a CU; few rows: spread a row over many threads
+        const int cap = n_out >= 512 ? 256 : 1024;
+        int vblock = 64;
+        while (vblock < cap && vblock < h4) vblock *= 2;
+#define VLAUNCH(BT, OT)                                                                                             \
+        add_rms_norm_vec4_kernel<BT, OT><<<n_out, vblock, 0, stream>>>(x, (const BT*)branch, nparts, part_stride,   \
+                                                                       bscale, w, eps, (OT*)out, rows, H)
+        if (branch_dtype == CPMCU_F32 && out_dtype == CPMCU_F32) VLAUNCH(float, float);
+        else if (branch_dtype == CPMCU_F32) VLAUNCH(float, bf16_t);
+        else if (out_dtype == CPMCU_F32) VLAUNCH(bf16_t, float);
+        else VLAUNCH(bf16_t, bf16_t);
+#undef VLAUNCH
         CPMCU_LAUNCH_CHECK("add_rms_norm");
         return nullptr;
     }
@@ -171,8 +186,38 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, l
     }
 }
 
+// bf16, I a multiple of 8: 8 columns a thread with 16-byte accesses
+__global__ void silu_mul_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, long n, int I) {
+    const int I8 = I / 8;
+    const long total = n * I8;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+        const long r = i / I8;
+        const int c = (int)(i - r * I8) * 8;
+        const uint4 g4 = *(const uint4*)(gu + r * 2 * I + c);
+        const uint4 u4 = *(const uint4*)(gu + r * 2 * I + I + c);
+        const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, uw[4] = {u4.x, u4.y, u4.z, u4.w};
+        uint32_t ow[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float g0 = __uint_as_float(gw[j] << 16), g1 = __uint_as_float(gw[j] & 0xffff0000u);
+            const float u0 = __uint_as_float(uw[j] << 16), u1 = __uint_as_float(uw[j] & 0xffff0000u);
+            const bf16_t a = f32_to_bf16(g0 / (1.0f + expf(-g0)) * u0);
+            const bf16_t b = f32_to_bf16(g1 / (1.0f + expf(-g1)) * u1);
+            ow[j] = (uint32_t)a.v | ((uint32_t)b.v << 16);
+        }
+        *(uint4*)(out + r * I + c) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+    }
+}
+
 extern "C" const char* cpmcu_silu_mul(const void* gu, void* out, int dtype, int n, int I, hipStream_t stream) {
     CPMCU_REQUIRE(n > 0 && I > 0, "silu_mul: empty shape n=%d I=%d", n, I);
+    if (dtype == CPMCU_BF16 && I % 8 == 0 && (uintptr_t)gu % 16 == 0 && (uintptr_t)out % 16 == 0) {
+        const long total8 = (long)n * (I / 8);
+        const int grid8 = (int)((total8 + 255) / 256 < 65535 * 8 ? (total8 + 255) / 256 : 65535 * 8);
+        silu_mul_bf16x8_kernel<<<grid8, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, n, I);
+        CPMCU_LAUNCH_CHECK("silu_mul");
+        return nullptr;
+    }
     const long total = (long)n * I;
     const int block = 256;
     const int grid = (int)((total + block - 1) / block < 65535 * 16 ? (total + block - 1) / block : 65535 * 16);

@@ -108,12 +108,12 @@ def test_embedding(dtype):
     assert torch.equal(out, table.float()[ids.long()] * 12.0)
 
 
-@pytest.mark.parametrize("H", [24, 100, 1000, 4096 + 8])
+@pytest.mark.parametrize("H,n", [(24, 6), (100, 6), (1000, 6), (4096 + 8, 6), (7, 3), (66, 3), (96, 600)])
 @pytest.mark.parametrize("bdtype,odtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
-                                           (torch.float32, torch.bfloat16)])
-def test_add_rms_norm(H, bdtype, odtype):
+                                           (torch.float32, torch.bfloat16), (torch.bfloat16, torch.float32)])
+def test_add_rms_norm(H, n, bdtype, odtype):
     from cpmcu_amd import ops
-    n, eps = 6, 1e-5
+    eps = 1e-5
     x0, w = rnd(n, H, seed=1), rnd(H, seed=2) + 1.0
     otol = 1e-5 if odtype == torch.float32 else 2 ** -8
     # plain norm
@@ -132,7 +132,7 @@ def test_add_rms_norm(H, bdtype, odtype):
         ref = F.rms_norm(xs, (H,), w.double(), eps)
         assert float((out.double() - ref).abs().max()) <= otol * float(ref.abs().max())
         # chosen rows only (one of them twice): x stays as it was
-        rows = torch.tensor([4, 0, 4], dtype=torch.int32, device=DEV)
+        rows = torch.tensor([n - 2, 0, n - 2], dtype=torch.int32, device=DEV)
         x = x0.clone()
         out_r = torch.empty(3, H, dtype=odtype, device=DEV)
         ops.add_rms_norm(x, b if parts > 1 else b[0], 0.7, w, eps, out_r, rows)
@@ -146,13 +146,14 @@ def test_add_rms_norm(H, bdtype, odtype):
     assert float((o - c / math.sqrt(c * c + eps)).abs().max()) < 1e-6
 
 
+@pytest.mark.parametrize("I", [77, 160, 1000])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_silu_mul(dtype):
+def test_silu_mul(dtype, I):
     from cpmcu_amd import ops
-    gu = rnd(5, 2 * 77, dtype=dtype, scale=3.0)
-    out = torch.empty(5, 77, dtype=dtype, device=DEV)
+    gu = rnd(5, 2 * I, dtype=dtype, scale=3.0)
+    out = torch.empty(5, I, dtype=dtype, device=DEV)
     ops.silu_mul(gu, out)
-    ref = F.silu(gu[:, :77].double()) * gu[:, 77:].double()
+    ref = F.silu(gu[:, :I].double()) * gu[:, I:].double()
     tol = 1e-6 if dtype == torch.float32 else 2 ** -8
     assert float((out.double() - ref).abs().max()) <= tol * float(ref.abs().max() + 1)
 
