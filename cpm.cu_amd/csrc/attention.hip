@@ -139,6 +139,10 @@ extern "C" const char* cpmcu_attention_plain(const void* q, void* out, int dtype
 typedef __bf16 abf16x8_t __attribute__((ext_vector_type(8)));
 typedef float afloatx4_t __attribute__((ext_vector_type(4)));
 
+// 2^x for x <= 0 (probabilities and rescale factors): the bare hardware instruction; results below the
+// normal range come out as 0, which is what a probability that small contributes anyway
+__device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
 template <int HD, int NW>
 __global__ __launch_bounds__(NW * 64) void attention_mfma_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, float* __restrict__ part_o, float2* __restrict__ part_ml,
@@ -253,26 +257,30 @@ __global__ __launch_bounds__(NW * 64) void attention_mfma_kernel(
             mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
             const float m_new = fmaxf(m, mx);
-            const float corr = exp2f(m - m_new);
+            const float corr = fast_exp2(m - m_new);
             float rs = 0.f;
             abf16x8_t pb;
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                const float p = exp2f(sc[j] - m_new);
+                const float p = fast_exp2(sc[j] - m_new);
                 rs += p;
                 pb[j] = (__bf16)p;
             }
             rs += __shfl_xor(rs, 16, 64);
             rs += __shfl_xor(rs, 32, 64);
             l = l * corr + rs;
+            // the accumulators are rescaled only when some row's maximum moved (rare after the first chunks)
+            if (__builtin_amdgcn_ballot_w64(m_new != m) != 0) {
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[dt][i] *= corr;
+            }
             m = m_new;
             // O^T += V^T . P^T ; A operand: lane (d row n, g) holds V^T[d][key0 + 8g .. +8]
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[dt][i] *= corr;
+            for (int dt = 0; dt < DT; ++dt)
                 acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pb, acc[dt], 0, 0, 0);
-            }
         }
         c = cn;
         key0 = key0n;
@@ -442,7 +450,7 @@ __global__ __launch_bounds__(64) void attention_prefill_mfma_kernel(
     int rows_per_token, int tokens_per_tile) {
     constexpr int KSTEPS = (HD + 31) / 32;
     constexpr int DT = HD / 16;
-    const int tile_id = blockIdx.x;
+    const int tile_id = gridDim.x - 1 - blockIdx.x;      // later tiles of a prompt see more keys: start them first
     const int kvh = blockIdx.y % nkv, ht = blockIdx.y / nkv;
     const int lane = threadIdx.x, n = lane & 15, g = lane >> 4;
     const int G = nh / nkv;
@@ -454,7 +462,7 @@ __global__ __launch_bounds__(64) void attention_prefill_mfma_kernel(
     // this lane's row in each tile: token and head; rows beyond the tile's tokens repeat its first token
     int row_tok[R], row_pos[R], row_head[R];
     bool row_ok[R];
-    int tile_last_pos[R];
+    int tile_last_pos[R], tile_first_pos[R];
     abf16x8_t qf[R][KSTEPS];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -466,6 +474,7 @@ __global__ __launch_bounds__(64) void attention_prefill_mfma_kernel(
         row_pos[r] = pos0 + (tk < n_tok ? tk : 0);
         row_head[r] = kvh * G + (hh < G ? hh : 0);
         tile_last_pos[r] = pos0 + min((r + 1) * tokens_per_tile, n_tok) - 1;
+        tile_first_pos[r] = pos0 + min(r * tokens_per_tile, n_tok - 1);
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) {
             abf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -506,7 +515,8 @@ __global__ __launch_bounds__(64) void attention_prefill_mfma_kernel(
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const abf16x8_t*)(vp + (long)dt * 16 * pv.page_size);
     };
-    // keys and values of chunk c+1 are asked for before the arithmetic of chunk c
+    // one buffer each for keys and values: the next chunk's keys are asked for as soon as the last tile's
+    // scores are issued, its values as soon as the last tile's P.V is, so both arrive behind other work
     abf16x8_t kf[2][KSTEPS], vf[DT];
     {
         const int page = ptab[0];
@@ -515,66 +525,74 @@ __global__ __launch_bounds__(64) void attention_prefill_mfma_kernel(
     }
     for (int c = 0; c < total_chunks; ++c) {
         const int key0 = c * 32;
-        abf16x8_t kn[2][KSTEPS], vn[DT];
-        if (c + 1 < total_chunks) {
-            const int pagen = ptab[(key0 + 32) / pv.page_size];
-            const int pon = (key0 + 32) % pv.page_size;
-            load_k(pagen, pon, kn);
-            load_v(pagen, pon, vn);
+        const bool more = c + 1 < total_chunks;
+        int pagen = 0, pon = 0;
+        if (more) {
+            pagen = ptab[(key0 + 32) / pv.page_size];
+            pon = (key0 + 32) % pv.page_size;
         }
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            if (r >= n_tiles_used || key0 > tile_last_pos[r]) continue;
+            const bool active = r < n_tiles_used && key0 <= tile_last_pos[r];
             afloatx4_t st[2];
+            if (active) {
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                st[u] = afloatx4_t{0.f, 0.f, 0.f, 0.f};
+                for (int u = 0; u < 2; ++u) {
+                    st[u] = afloatx4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int ks = 0; ks < KSTEPS; ++ks)
-                    st[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][ks], qf[r][ks], st[u], 0, 0, 0);
-            }
-            float sc[8];
-            float mx = -INFINITY;
-#pragma unroll
-            for (int u = 0; u < 2; ++u)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int key = key0 + 8 * g + 4 * u + i;
-                    const float v = key <= row_pos[r] ? st[u][i] * scale_log2e : -INFINITY;
-                    sc[u * 4 + i] = v;
-                    mx = fmaxf(mx, v);
+                    for (int ks = 0; ks < KSTEPS; ++ks)
+                        st[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][ks], qf[r][ks], st[u], 0, 0, 0);
                 }
-            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            // a row whose position lies before this chunk sees none of its keys: nothing changes for it
-            const float m_new = fmaxf(m[r], mx);
-            const float m_use = m_new == -INFINITY ? 0.f : m_new;
-            const float corr = exp2f(m[r] - m_use);
-            float rs = 0.f;
-            abf16x8_t pb;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const float p = exp2f(sc[j] - m_use);
-                rs += p;
-                pb[j] = (__bf16)p;
             }
-            rs += __shfl_xor(rs, 16, 64);
-            rs += __shfl_xor(rs, 32, 64);
-            l[r] = l[r] * corr + rs;
-            m[r] = m_new;
+            if (r == R - 1 && more) load_k(pagen, pon, kf);      // the last tile's scores are issued: keys are free
+            if (active) {
+                // raw scores; only a chunk that reaches past a row's position needs the causal mask
+                float sc[8];
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
+                for (int u = 0; u < 2; ++u)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) acc[r][dt][i] *= corr;
-                acc[r][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pb, acc[r][dt], 0, 0, 0);
+                    for (int i = 0; i < 4; ++i) sc[u * 4 + i] = st[u][i];
+                if (key0 + 31 > tile_first_pos[r]) {
+#pragma unroll
+                    for (int u = 0; u < 2; ++u)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            if (key0 + 8 * g + 4 * u + i > row_pos[r]) sc[u * 4 + i] = -INFINITY;
+                }
+                float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
+                                 fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+                mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                // running maximum in units of scaled scores (scale > 0); a row whose position lies before
+                // this chunk sees none of its keys: nothing changes for it
+                const float m_new = fmaxf(m[r], mx * scale_log2e);
+                const float m_use = m_new == -INFINITY ? 0.f : m_new;
+                const float corr = fast_exp2(m[r] - m_use);
+                float rs = 0.f;
+                abf16x8_t pb;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float p = fast_exp2(fmaf(sc[j], scale_log2e, -m_use));
+                    rs += p;
+                    pb[j] = (__bf16)p;
+                }
+                rs += __shfl_xor(rs, 16, 64);
+                rs += __shfl_xor(rs, 32, 64);
+                l[r] = l[r] * corr + rs;
+                // the accumulators are rescaled only when some row's maximum moved (rare after the first chunks)
+                if (__builtin_amdgcn_ballot_w64(m_new != m[r]) != 0) {
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) acc[r][dt][i] *= corr;
+                }
+                m[r] = m_new;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+                    acc[r][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pb, acc[r][dt], 0, 0, 0);
             }
         }
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-#pragma unroll
-            for (int ks = 0; ks < KSTEPS; ++ks) kf[u][ks] = kn[u][ks];
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) vf[dt] = vn[dt];
+        if (more) load_v(pagen, pon, vf);
     }
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -588,14 +606,16 @@ __global__ __launch_bounds__(64) void attention_prefill_mfma_kernel(
     }
 }
 
-extern "C" int cpmcu_attention_prefill_tokens_per_wave(int nh, int nkv) {
+// tokens a wavefront holds: `tiles_per_wave` (2 or 4) tiles of 16 rows
+extern "C" int cpmcu_attention_prefill_tokens_per_wave(int nh, int nkv, int tiles_per_wave) {
     const int G = nh / nkv;
     const int rpt = (G < 16 && 16 % G == 0) ? G : 16;
-    return 4 * (16 / rpt);
+    return tiles_per_wave * (16 / rpt);
 }
 
 // tiles: int32 [n_tiles, 2] = (first packed token, tokens) with tokens <= cpmcu_attention_prefill_tokens_per_wave
-extern "C" const char* cpmcu_attention_prefill_mfma(const void* q, void* out, int n_tiles, const int* tiles, int nh,
+extern "C" const char* cpmcu_attention_prefill_mfma(const void* q, void* out, int n_tiles, const int* tiles,
+                                                    int tiles_per_wave, int nh,
                                                     int nkv, int hd, float scale, const void* kpool,
                                                     const void* vtpool, const int* page_table, int table_width,
                                                     int page_size, const int* positions, const int* tok_slot,
@@ -612,15 +632,22 @@ extern "C" const char* cpmcu_attention_prefill_mfma(const void* q, void* out, in
     PagedView pv{page_table, table_width, page_size};
     dim3 grid(n_tiles, nkv * HT);
     const float sl = scale * 1.4426950408889634f;
-#define LAUNCH(HDv)                                                                                             \
-    attention_prefill_mfma_kernel<HDv, 4><<<grid, 64, 0, stream>>>((const bf16_t*)q, (bf16_t*)out,              \
-                                                                   (const bf16_t*)kpool, (const bf16_t*)vtpool, \
-                                                                   pv, tiles, positions, tok_slot, nh, nkv, sl, \
-                                                                   rpt, tpt)
-    if (hd == 16) LAUNCH(16);
-    else if (hd == 32) LAUNCH(32);
-    else if (hd == 64) LAUNCH(64);
-    else LAUNCH(128);
+    CPMCU_REQUIRE(tiles_per_wave == 2 || tiles_per_wave == 4, "attention_prefill: %d tiles a wavefront (2 or 4 are built)", tiles_per_wave);
+#define LAUNCH(HDv, Rv)                                                                                          \
+    attention_prefill_mfma_kernel<HDv, Rv><<<grid, 64, 0, stream>>>((const bf16_t*)q, (bf16_t*)out,              \
+                                                                    (const bf16_t*)kpool, (const bf16_t*)vtpool, \
+                                                                    pv, tiles, positions, tok_slot, nh, nkv, sl, \
+                                                                    rpt, tpt)
+#define BY_R(HDv)                                \
+    do {                                         \
+        if (tiles_per_wave == 4) LAUNCH(HDv, 4); \
+        else LAUNCH(HDv, 2);                     \
+    } while (0)
+    if (hd == 16) BY_R(16);
+    else if (hd == 32) BY_R(32);
+    else if (hd == 64) BY_R(64);
+    else BY_R(128);
+#undef BY_R
 #undef LAUNCH
     CPMCU_LAUNCH_CHECK("attention_prefill_mfma");
     return nullptr;
