@@ -354,3 +354,83 @@ def test_attention_with_block_lists(bs, dtype):
             ops.attention_mfma(q.view(n, -1), out, nh, nkv, hd, hd ** -0.5, kpool, vpool, table, page, pos_t, slot_t,
                                splits, po, pm, sel_blocks.to(DEV), sel_count.to(DEV), bs, waves_per_group=nw)
             assert float((out.double().cpu().view(n, nh, hd) - ref).abs().max()) <= tol
+
+
+# ---------------------------------------------------------------------------- InfLLM-v2 kernels
+@pytest.mark.parametrize("ks,st", [(8, 4), (32, 16), (16, 16), (12, 4)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_compressed_keys_are_means_written_when_their_last_key_arrives(ks, st, dtype):
+    from cpmcu_amd import ops
+    nkv, hd, page = 2, 16, 64
+    lens = [150, 37]
+    kseq, vs, kpool, vpool, table = paged_setup(lens, nkv, hd, page, dtype, seed=ks)
+    ck = torch.zeros(kpool.shape[0], page // st, nkv * hd, dtype=dtype, device=DEV)
+    # two steps: first the tokens up to 100 / 20, then the rest (compressed keys that straddle the cut
+    # are completed by the second step)
+    for a0, b0, a1, b1 in ((0, 100, 0, 20), (100, 150, 20, 37)):
+        positions = list(range(a0, b0)) + list(range(a1, b1))
+        slots = [0] * (b0 - a0) + [1] * (b1 - a1)
+        ops.compress_keys(kpool, ck, table, page, torch.tensor(positions, dtype=torch.int32, device=DEV),
+                          torch.tensor(slots, dtype=torch.int32, device=DEV), ks, st)
+    for s, L in enumerate(lens):
+        ref = F.avg_pool1d(kseq[s].reshape(L, -1).T[None], ks, st)[0].T        # [n_ck, nkv*hd]
+        got = torch.stack([ck[int(table[s, (st * j) // page]), ((st * j) % page) // st] for j in range(ref.shape[0])])
+        tol = 1e-6 if dtype == torch.float32 else 2 ** -8
+        assert float((got.double().cpu() - ref).abs().max()) <= tol * float(ref.abs().max() + 1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("ks,st,bs,init,topk,window,dense_len", [(8, 4, 16, 1, 4, 32, 64), (32, 16, 64, 1, 3, 128, 0),
+                                                              (8, 8, 32, 2, 2, 32, 100), (16, 4, 16, 0, 5, 16, 0)])
+def test_block_selection_equals_the_plain_selection(dtype, ks, st, bs, init, topk, window, dense_len):
+    """Positions at block edges, window edges, just past dense_len and where compressed keys become visible."""
+    import plain_minicpm as plain
+    from cpmcu_amd import ops
+    nh, nkv, hd, page = 6, 2, 16, 64
+    L = 460
+    kseq, vs, kpool, vpool, table = paged_setup([L], nkv, hd, page, dtype, seed=bs + topk)
+    ck = torch.zeros(kpool.shape[0], page // st, nkv * hd, dtype=dtype, device=DEV)
+    allpos = torch.arange(L, dtype=torch.int32, device=DEV)
+    ops.compress_keys(kpool, ck, table, page, allpos, torch.zeros(L, dtype=torch.int32, device=DEV), ks, st)
+    sc = {"kernel_size": ks, "kernel_stride": st, "block_size": bs, "init_blocks": init, "topk": topk,
+          "window_size": window, "dense_len": dense_len}
+    positions = sorted(set([0, 1, ks - 1, ks, ks + 1, bs - 1, bs, bs + 1, window - 1, window, window + bs - 1, window + bs,
+                            max(dense_len - 1, 0), dense_len, dense_len + 1, 255, 256, 257, 300, 399, 400, L - 1]))
+    positions = [p for p in positions if 0 <= p < L]
+    n = len(positions)
+    q = rnd(n, nh, hd, seed=4, dtype=dtype)
+    lb = window // bs
+    sel_blocks = torch.full((n, nkv, topk + lb), -7, dtype=torch.int32, device=DEV)
+    sel_count = torch.full((n, nkv), -7, dtype=torch.int32, device=DEV)
+    ops.sparse_select(q.view(n, -1), ck, nh, nkv, hd, hd ** -0.5, table, page,
+                      torch.tensor(positions, dtype=torch.int32, device=DEV), torch.zeros(n, dtype=torch.int32, device=DEV),
+                      ks, st, bs, init, topk, lb, dense_len, max(positions), sel_blocks, sel_count)
+    # plain selection from the same (rounded) keys; compressed keys in the cache's own precision
+    ck_ref = plain.compressed_keys(kseq[0], ks, st).to(dtype).double()
+    for t, p in enumerate(positions):
+        want = plain.infllm_select(q[t].double().cpu(), ck_ref, p, sc, nkv)
+        for h in range(nkv):
+            c = int(sel_count[t, h])
+            if want is None:
+                assert c == -1, (p, h)
+            else:
+                assert sel_blocks[t, h, :c].tolist() == want[h], (p, h, want[h])
+
+
+def test_block_selection_ties_and_forced_blocks():
+    """All compressed keys equal: every score ties and the lowest blocks win; initial blocks count toward topk."""
+    from cpmcu_amd import ops
+    nh, nkv, hd, page, ks, st, bs = 2, 1, 16, 64, 8, 4, 16
+    L = 208
+    kpool = torch.ones(5, page, nkv * hd, device=DEV)
+    table = torch.tensor([[3, 1, 4, 0]], dtype=torch.int32, device=DEV)
+    ck = torch.zeros(5, page // st, nkv * hd, device=DEV)
+    ops.compress_keys(kpool, ck, table, page, torch.arange(L, dtype=torch.int32, device=DEV),
+                      torch.zeros(L, dtype=torch.int32, device=DEV), ks, st)
+    q = torch.ones(1, nh * hd, device=DEV)
+    for init, topk, want in ((0, 3, [0, 1, 2, 11, 12]), (2, 2, [0, 1, 11, 12]), (1, 20, list(range(13)))):
+        sb = torch.zeros(1, 1, topk + 2, dtype=torch.int32, device=DEV)
+        cnt = torch.zeros(1, 1, dtype=torch.int32, device=DEV)
+        ops.sparse_select(q, ck, nh, nkv, hd, 0.25, table, page, torch.tensor([200], dtype=torch.int32, device=DEV),
+                          torch.zeros(1, dtype=torch.int32, device=DEV), ks, st, bs, init, topk, 2, 0, 200, sb, cnt)
+        assert sb[0, 0, :int(cnt[0, 0])].tolist() == want
