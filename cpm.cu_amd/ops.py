@@ -306,7 +306,8 @@ def compress_keys(kpool: torch.Tensor, ckpool: torch.Tensor, page_table: torch.T
 def sparse_select(q: torch.Tensor, ckpool: torch.Tensor, nh: int, nkv: int, hd: int, scale: float,
                   page_table: torch.Tensor, page_size: int, positions: torch.Tensor, tok_slot: torch.Tensor,
                   kernel_size: int, kernel_stride: int, block_size: int, init_blocks: int, topk: int,
-                  window_blocks: int, dense_len: int, max_pos: int, sel_blocks: torch.Tensor, sel_count: torch.Tensor):
+                  window_blocks: int, dense_len: int, max_pos: int, sel_blocks: torch.Tensor, sel_count: torch.Tensor,
+                  force_plain: bool = False):
     """Block list per (token, kv head): sel_count -1 = dense, else the ascending blocks to attend to."""
     _need(q, "select q", shape=(None, nh * hd))
     n = q.shape[0]
@@ -321,7 +322,7 @@ def sparse_select(q: torch.Tensor, ckpool: torch.Tensor, nh: int, nkv: int, hd: 
         _p(page_table), c_int(page_table.shape[1]), c_int(page_size), _p(positions), _p(tok_slot),
         c_int(kernel_size), c_int(kernel_stride), c_int(block_size), c_int(init_blocks), c_int(topk),
         c_int(window_blocks), c_int(dense_len), c_int(max_pos), _p(sel_blocks), _p(sel_count),
-        c_int(sel_blocks.shape[2]), _stream()))
+        c_int(sel_blocks.shape[2]), c_int(1 if force_plain else 0), _stream()))
 
 
 def argmax(logits: torch.Tensor, out: torch.Tensor):

@@ -380,13 +380,14 @@ def test_compressed_keys_are_means_written_when_their_last_key_arrives(ks, st, d
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,hd", [(6, 2, 16), (32, 2, 128), (20, 1, 32)])
 @pytest.mark.parametrize("ks,st,bs,init,topk,window,dense_len", [(8, 4, 16, 1, 4, 32, 64), (32, 16, 64, 1, 3, 128, 0),
                                                               (8, 8, 32, 2, 2, 32, 100), (16, 4, 16, 0, 5, 16, 0)])
-def test_block_selection_equals_the_plain_selection(dtype, ks, st, bs, init, topk, window, dense_len):
+def test_block_selection_equals_the_plain_selection(dtype, nh, nkv, hd, ks, st, bs, init, topk, window, dense_len):
     """Positions at block edges, window edges, just past dense_len and where compressed keys become visible."""
     import plain_minicpm as plain
     from cpmcu_amd import ops
-    nh, nkv, hd, page = 6, 2, 16, 64
+    page = 64
     L = 460
     kseq, vs, kpool, vpool, table = paged_setup([L], nkv, hd, page, dtype, seed=bs + topk)
     ck = torch.zeros(kpool.shape[0], page // st, nkv * hd, dtype=dtype, device=DEV)
@@ -402,19 +403,23 @@ def test_block_selection_equals_the_plain_selection(dtype, ks, st, bs, init, top
     lb = window // bs
     sel_blocks = torch.full((n, nkv, topk + lb), -7, dtype=torch.int32, device=DEV)
     sel_count = torch.full((n, nkv), -7, dtype=torch.int32, device=DEV)
-    ops.sparse_select(q.view(n, -1), ck, nh, nkv, hd, hd ** -0.5, table, page,
-                      torch.tensor(positions, dtype=torch.int32, device=DEV), torch.zeros(n, dtype=torch.int32, device=DEV),
-                      ks, st, bs, init, topk, lb, dense_len, max(positions), sel_blocks, sel_count)
     # plain selection from the same (rounded) keys; compressed keys in the cache's own precision
     ck_ref = plain.compressed_keys(kseq[0], ks, st).to(dtype).double()
-    for t, p in enumerate(positions):
-        want = plain.infllm_select(q[t].double().cpu(), ck_ref, p, sc, nkv)
-        for h in range(nkv):
-            c = int(sel_count[t, h])
-            if want is None:
-                assert c == -1, (p, h)
-            else:
-                assert sel_blocks[t, h, :c].tolist() == want[h], (p, h, want[h])
+    for force_plain in ((False, True) if dtype == torch.bfloat16 else (True,)):     # matrix-core kernel and plain twin
+        sel_blocks.fill_(-7)
+        sel_count.fill_(-7)
+        ops.sparse_select(q.view(n, -1), ck, nh, nkv, hd, hd ** -0.5, table, page,
+                          torch.tensor(positions, dtype=torch.int32, device=DEV),
+                          torch.zeros(n, dtype=torch.int32, device=DEV),
+                          ks, st, bs, init, topk, lb, dense_len, max(positions), sel_blocks, sel_count, force_plain)
+        for t, p in enumerate(positions):
+            want = plain.infllm_select(q[t].double().cpu(), ck_ref, p, sc, nkv)
+            for h in range(nkv):
+                c = int(sel_count[t, h])
+                if want is None:
+                    assert c == -1, (p, h)
+                else:
+                    assert sel_blocks[t, h, :c].tolist() == want[h], (p, h, want[h], force_plain)
 
 
 def test_block_selection_ties_and_forced_blocks():
@@ -428,9 +433,11 @@ def test_block_selection_ties_and_forced_blocks():
     ops.compress_keys(kpool, ck, table, page, torch.arange(L, dtype=torch.int32, device=DEV),
                       torch.zeros(L, dtype=torch.int32, device=DEV), ks, st)
     q = torch.ones(1, nh * hd, device=DEV)
-    for init, topk, want in ((0, 3, [0, 1, 2, 11, 12]), (2, 2, [0, 1, 11, 12]), (1, 20, list(range(13)))):
-        sb = torch.zeros(1, 1, topk + 2, dtype=torch.int32, device=DEV)
-        cnt = torch.zeros(1, 1, dtype=torch.int32, device=DEV)
-        ops.sparse_select(q, ck, nh, nkv, hd, 0.25, table, page, torch.tensor([200], dtype=torch.int32, device=DEV),
-                          torch.zeros(1, dtype=torch.int32, device=DEV), ks, st, bs, init, topk, 2, 0, 200, sb, cnt)
-        assert sb[0, 0, :int(cnt[0, 0])].tolist() == want
+    for dtype in (torch.float32, torch.bfloat16):
+        for init, topk, want in ((0, 3, [0, 1, 2, 11, 12]), (2, 2, [0, 1, 11, 12]), (1, 20, list(range(13)))):
+            sb = torch.zeros(1, 1, topk + 2, dtype=torch.int32, device=DEV)
+            cnt = torch.zeros(1, 1, dtype=torch.int32, device=DEV)
+            ops.sparse_select(q.to(dtype), ck.to(dtype), nh, nkv, hd, 0.25, table, page,
+                              torch.tensor([200], dtype=torch.int32, device=DEV),
+                              torch.zeros(1, dtype=torch.int32, device=DEV), ks, st, bs, init, topk, 2, 0, 200, sb, cnt)
+            assert sb[0, 0, :int(cnt[0, 0])].tolist() == want, dtype
