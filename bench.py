@@ -36,6 +36,27 @@ def config_8b(layers=None):
     }
 
 
+def config_small():
+    """BASELINE.json configs[3]: the MiniCPM4-0.5B shape (tied embeddings)."""
+    import torch
+    g = torch.Generator().manual_seed(4321)
+    fac = lambda: [float(x) for x in (1.0 + 3.0 * torch.rand(32, generator=g, dtype=torch.float64))]
+    return {
+        "architectures": ["MiniCPMForCausalLM"], "model_type": "minicpm",
+        "num_hidden_layers": 24, "hidden_size": 1024, "num_attention_heads": 16, "num_key_value_heads": 2,
+        "head_dim": 64, "intermediate_size": 4096, "vocab_size": 73448, "rms_norm_eps": 1e-6, "rope_theta": 10000.0,
+        "max_position_embeddings": 32768,
+        "rope_scaling": {"rope_type": "longrope", "short_factor": fac(), "long_factor": fac(),
+                         "original_max_position_embeddings": 32768},
+        "scale_emb": 12, "dim_model_base": 256, "scale_depth": 1.4, "tie_word_embeddings": True,
+        "hidden_act": "silu", "torch_dtype": "bfloat16",
+    }
+
+
+SPARSE_32K = {"kernel_size": 32, "kernel_stride": 16, "block_size": 64, "init_blocks": 1, "topk": 64,
+              "window_size": 2048, "dense_len": 8192}
+
+
 def weight_bytes_per_step(cfg, esize):
     """Bytes of weights a decode step reads once: every layer's matrices and norms, final norm, lm_head."""
     H, I, V, L = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size, cfg.num_hidden_layers
@@ -70,6 +91,10 @@ def main():
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--hip-graph", type=int, default=1)
+    ap.add_argument("--scenario", default="headline", choices=["headline", "small_batch64", "sparse32k"],
+                    help="headline: BASELINE.json configs[2] (the default, the contract's line); small_batch64: "
+                         "configs[3], 64 unequal prompts through the generation loop; sparse32k: configs[4], "
+                         "InfLLM-v2 at 32k context")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported (no multi-GPU path exists)")
@@ -82,6 +107,9 @@ def main():
     from cpmcu_amd.weights import random_tensors
 
     dev = "cuda:0"
+    if args.scenario != "headline":
+        other_scenarios(args, dev)
+        return
     raw = config_8b(args.layers)
     cfg = MiniCPMConfig.from_dict(raw)
     esize = 2 if args.dtype == "bfloat16" else 4
@@ -169,6 +197,82 @@ def main():
             d = decode_run(b, args.context, st, max(args.warmup // 2, 3))
             pts[f"decode_b{b}"] = round(b * st / d, 2)
         rec["points"] = pts
+    print(json.dumps(rec), flush=True)
+
+
+def other_scenarios(args, dev):
+    """The two further workloads of BASELINE.json, each one JSON line of the same shape."""
+    import torch
+    from cpmcu_amd import Engine, EngineOptions, StepEntry
+    from cpmcu_amd.config import MiniCPMConfig
+    from cpmcu_amd.engine.generate import generate
+    from cpmcu_amd.weights import random_tensors
+
+    g = torch.Generator().manual_seed(11)
+    if args.scenario == "small_batch64":
+        cfg = MiniCPMConfig.from_dict(config_small())
+        lens = [int(x) for x in torch.randint(128, 2049, (64,), generator=g)]
+        new = 256
+        eng = Engine.from_tensors(cfg, random_tensors(cfg, 0, device=dev), EngineOptions(
+            dtype=args.dtype, max_tokens=sum(-(-(n + new) // 64) * 64 for n in lens), max_slots=64,
+            max_step_tokens=8192, device=dev, hip_graph=bool(args.hip_graph)))
+        prompts = [[int(t) for t in torch.randint(0, cfg.vocab_size, (n,), generator=g)] for n in lens]
+        generate(eng, prompts[:4], 8)                                   # warm-up: kernels loaded, graphs of small batches
+        outs = generate(eng, prompts, new)
+        prefill_s = max(o.prefill_time for o in outs)
+        decode_s = max(o.decode_time for o in outs)
+        n_dec = sum(len(o.tokens) - 1 for o in outs)
+        rec = {"metric": "MiniCPM4-0.5B shape, 64 unequal prompts (128..2048), 256 new tokens each: decode tok/s through "
+                         "the generation loop", "value": round(n_dec / decode_s, 1), "unit": "tokens/s", "n_gpus": 1,
+               "steps": new - 1, "warmup": 0, "ms_per_step": round(decode_s / (new - 1) * 1e3, 4),
+               "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+               "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+               "config": {"model": "MiniCPM4-0.5B shape, random weights N(0,0.02)", "layers": 24, "hidden": 1024,
+                          "heads": 16, "kv_heads": 2, "head_dim": 64, "intermediate": 4096, "vocab": 73448,
+                          "global_batch": 64, "prompt_tokens": sum(lens), "new_tokens": new, "parallelism": "1gpu",
+                          "hip_graph": bool(args.hip_graph)},
+               "prefill": {"value": round(sum(lens) / prefill_s, 1), "tokens": sum(lens), "ms": round(prefill_s * 1e3, 2)}}
+        print(json.dumps(rec), flush=True)
+        return
+    raw = config_8b(args.layers)
+    raw["sparse_config"] = dict(SPARSE_32K)
+    cfg = MiniCPMConfig.from_dict(raw)
+    n_prompt, new = 32000, 256
+    eng = Engine.from_tensors(cfg, random_tensors(cfg, 0, device=dev), EngineOptions(
+        dtype=args.dtype, max_tokens=4 * 32768, max_slots=4, max_step_tokens=2048, device=dev,
+        hip_graph=bool(args.hip_graph)))
+    rec = {"metric": "MiniCPM4-8B shape with InfLLM-v2 at 32k context: decode tok/s at batch 1 after a 32,000-token prefill",
+           "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+           "config": {"model": "MiniCPM4-8B shape + sparse_config, random weights", "layers": cfg.num_hidden_layers,
+                      "layers_full_model": 32, "kernel_size": 32, "kernel_stride": 16, "block_size": 64, "topk": 64,
+                      "window_size": 2048, "dense_len": 8192, "prompt_tokens": n_prompt, "new_tokens": new,
+                      "parallelism": "1gpu", "hip_graph": bool(args.hip_graph)}, "points": {}}
+    for batch in (1, 4):
+        slots = [eng.acquire() for _ in range(batch)]
+        ids = [[int(t) for t in torch.randint(0, cfg.vocab_size, (n_prompt + new,), generator=g)] for _ in slots]
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for sl, tok in zip(slots, ids):
+            for a in range(0, n_prompt, 2048):
+                eng.step([StepEntry(sl, tok[a:min(a + 2048, n_prompt)], [])])
+        torch.cuda.synchronize()
+        pre = time.perf_counter() - t
+        for i in range(8):
+            eng.step([StepEntry(sl, [tok[n_prompt + i]], [0]) for sl, tok in zip(slots, ids)])
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for i in range(8, new):
+            eng.step([StepEntry(sl, [tok[n_prompt + i]], [0]) for sl, tok in zip(slots, ids)])
+        torch.cuda.synchronize()
+        dec = time.perf_counter() - t
+        for sl in slots:
+            eng.release(sl)
+        if batch == 1:
+            rec.update({"value": round((new - 8) / dec, 2), "steps": new - 8, "warmup": 8,
+                        "ms_per_step": round(dec / (new - 8) * 1e3, 4),
+                        "prefill": {"value": round(n_prompt / pre, 1), "tokens": n_prompt, "ms": round(pre * 1e3, 1)}})
+        rec["points"][f"decode_b{batch}"] = round(batch * (new - 8) / dec, 2)
     print(json.dumps(rec), flush=True)
 
 
