@@ -165,7 +165,7 @@ __global__ __launch_bounds__(256) void sparse_select_kernel(const T* __restrict_
     }
 }
 
-template <int HD>
+template <int HD, int NW>
 __global__ void sparse_select_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ ckpool, PagedView pv,
                                           const int* __restrict__ positions, const int* __restrict__ tok_slot,
                                           SelectParams sp, int* __restrict__ sel_blocks, int* __restrict__ sel_count);
@@ -198,9 +198,16 @@ extern "C" const char* cpmcu_sparse_select(const void* q, const void* ckpool, in
     PagedView pv{page_table, table_width, page_size};
     if (dtype == CPMCU_BF16 && !force_plain && (hd == 16 || hd == 32 || hd == 64 || hd == 128)) {
         const size_t lds2 = sizeof(float) * ((size_t)sp.max_ck + 2 * sp.max_blocks);
-#define LAUNCH(HDv)                                                                                              \
-        sparse_select_mfma_kernel<HDv><<<grid, 256, lds2, stream>>>((const bf16_t*)q, (const bf16_t*)ckpool, pv, \
-                                                                    positions, tok_slot, sp, sel_blocks, sel_count)
+        // few tokens (decode steps): 16 wavefronts share a (token, kv head)'s compressed keys; many: 4
+#define LAUNCH(HDv)                                                                                          \
+        do {                                                                                                 \
+            if (n * nkv <= 256)                                                                              \
+                sparse_select_mfma_kernel<HDv, 16><<<grid, 1024, lds2, stream>>>(                            \
+                    (const bf16_t*)q, (const bf16_t*)ckpool, pv, positions, tok_slot, sp, sel_blocks, sel_count); \
+            else                                                                                             \
+                sparse_select_mfma_kernel<HDv, 4><<<grid, 256, lds2, stream>>>(                              \
+                    (const bf16_t*)q, (const bf16_t*)ckpool, pv, positions, tok_slot, sp, sel_blocks, sel_count); \
+        } while (0)
         if (hd == 16) LAUNCH(16);
         else if (hd == 32) LAUNCH(32);
         else if (hd == 64) LAUNCH(64);
@@ -223,8 +230,8 @@ extern "C" const char* cpmcu_sparse_select(const void* q, const void* ckpool, in
 
 // ===========================================================================
 // The same selection with the scores on the matrix cores (bf16, head size 16,
-// 32, 64 or 128).  One workgroup of 4 wavefronts per (token, kv head); tiles of
-// 16 compressed keys are dealt to the wavefronts in turn.
+// 32, 64 or 128).  One workgroup of 4 or 16 wavefronts per (token, kv head); tiles
+// of 16 compressed keys are dealt to the wavefronts in turn.
 //   S = Q . CK^T      A = the group's heads (rows) from registers, B = 16
 //                     compressed keys straight from their cache rows;
 //                     D: lane (key n, g) holds heads 4g..4g+3
@@ -237,15 +244,15 @@ extern "C" const char* cpmcu_sparse_select(const void* q, const void* ckpool, in
 typedef __bf16 sbf16x8_t __attribute__((ext_vector_type(8)));
 typedef float sfloatx4_t __attribute__((ext_vector_type(4)));
 
-template <int HD>
-__global__ __launch_bounds__(256) void sparse_select_mfma_kernel(
+template <int HD, int NW>
+__global__ __launch_bounds__(NW * 64) void sparse_select_mfma_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ ckpool, PagedView pv,
     const int* __restrict__ positions, const int* __restrict__ tok_slot, SelectParams sp,
     int* __restrict__ sel_blocks, int* __restrict__ sel_count) {
     constexpr int KSTEPS = (HD + 31) / 32;
     extern __shared__ float lds[];
-    __shared__ float stat_s[4][16][2];
-    __shared__ int wave_tot[4];
+    __shared__ float stat_s[NW][16][2];
+    __shared__ int wave_tot[NW];
     float* score = lds;
     float* pool = score + sp.max_ck;
     int* flag = (int*)(pool + sp.max_blocks);
@@ -301,7 +308,7 @@ __global__ __launch_bounds__(256) void sparse_select_mfma_kernel(
         };
         // pass 1: running max and sum per head, per lane
         float m[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY}, l[4] = {0.f, 0.f, 0.f, 0.f};
-        for (int tile = wave; tile < n_tiles; tile += 4) {
+        for (int tile = wave; tile < n_tiles; tile += NW) {
             const sfloatx4_t st = scores_of_tile(tile);
             if (tile * 16 + n < n_vis) {
 #pragma unroll
@@ -339,9 +346,9 @@ __global__ __launch_bounds__(256) void sparse_select_mfma_kernel(
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             float mm = -INFINITY;
-            for (int w = 0; w < 4; ++w) mm = fmaxf(mm, stat_s[w][4 * g + i][0]);
+            for (int w = 0; w < NW; ++w) mm = fmaxf(mm, stat_s[w][4 * g + i][0]);
             float ll = 0.f;
-            for (int w = 0; w < 4; ++w) {
+            for (int w = 0; w < NW; ++w) {
                 const float wm = stat_s[w][4 * g + i][0];
                 if (wm != -INFINITY) ll += stat_s[w][4 * g + i][1] * exp2f(wm - mm);
             }
@@ -350,7 +357,7 @@ __global__ __launch_bounds__(256) void sparse_select_mfma_kernel(
             invL[i] = (ht * 16 + 4 * g + i < G && ll > 0.f) ? 1.0f / ll : 0.f;
         }
         // pass 2: normalised scores summed over the heads of the group
-        for (int tile = wave; tile < n_tiles; tile += 4) {
+        for (int tile = wave; tile < n_tiles; tile += NW) {
             const sfloatx4_t st = scores_of_tile(tile);
             float v = 0.f;
 #pragma unroll
@@ -391,10 +398,10 @@ __global__ __launch_bounds__(256) void sparse_select_mfma_kernel(
         flag[b] = f;
     }
     __syncthreads();
-    // ascending list: a prefix count over the flags, 256 blocks a round
+    // ascending list: a prefix count over the flags, one block a thread a round
     int* dst = sel_blocks + out_idx * sp.max_sel;
     int base = 0;
-    for (int b0 = 0; b0 <= q_block; b0 += 256) {
+    for (int b0 = 0; b0 <= q_block; b0 += NW * 64) {
         const int b = b0 + tid;
         const int f = (b <= q_block) ? flag[b] : 0;
         const unsigned long long mask = __builtin_amdgcn_ballot_w64(f != 0);
@@ -404,7 +411,7 @@ __global__ __launch_bounds__(256) void sparse_select_mfma_kernel(
         int off = base;
         for (int w = 0; w < wave; ++w) off += wave_tot[w];
         if (f && off + before < sp.max_sel) dst[off + before] = b;
-        base += wave_tot[0] + wave_tot[1] + wave_tot[2] + wave_tot[3];
+        for (int w = 0; w < NW; ++w) base += wave_tot[w];
         __syncthreads();
     }
     if (tid == 0) sel_count[out_idx] = min(base, sp.max_sel);
