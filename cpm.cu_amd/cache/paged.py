@@ -121,6 +121,7 @@ class SequenceCache:
             for e in entries:
                 self.entry_group[e] = len(self.groups)
             self.groups.append(g)
+        self._has_window = any(g.needs.window is not None for g in self.groups)
         self.free_slots: List[int] = list(range(max_slots - 1, -1, -1))
         self.live: Dict[int, int] = {}        # slot -> tokens held
         self._views: Dict[int, CacheView] = {}
@@ -204,6 +205,15 @@ class SequenceCache:
                 g.dirty.add(slot)
         self.live[slot] = new
         return old
+
+    def extend_one(self, slot: int) -> int:
+        """extend(slot, 1) for the decode loop: nothing but the length changes while the token fits the
+        slot's last page and no group drops pages."""
+        old = self.live[slot]
+        if old % self.page_size and not self._has_window:
+            self.live[slot] = old + 1
+            return old
+        return self.extend(slot, 1)
 
     def sync(self):
         """Copy the page-table rows that changed to the device (before kernels read them)."""

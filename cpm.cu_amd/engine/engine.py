@@ -181,6 +181,11 @@ class Engine:
         """Run the entries' tokens; float32 logits [wanted, vocab] in the order of entries and of ``want``
         (None if nothing is wanted)."""
         entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
+        if entries and len(entries) <= self.max_step_tokens and all(len(e.tokens) == 1 for e in entries):
+            with torch.cuda.device(self.device):
+                out = self._step_single_tokens(entries)
+            self.steps_run += 1
+            return out
         self._validate(entries)
         row_of: Dict[Tuple[int, int], List[int]] = {}
         n_rows = 0
@@ -194,6 +199,99 @@ class Engine:
                 self._forward(entries, chunk, row_of, result)
         self.steps_run += 1
         return result
+
+    def _step_single_tokens(self, entries) -> Optional[torch.Tensor]:
+        """The step of a decode loop: every sequence brings one token.  The same checks and the same forward
+        pass as the general path, with the bookkeeping done on whole arrays."""
+        cache = self.cache
+        B = len(entries)
+        slots = [e.slot for e in entries]
+        tok = np.fromiter((e.tokens[0] for e in entries), dtype=np.int64, count=B)
+        if len(set(slots)) != B:
+            dup = next(s for s in slots if slots.count(s) > 1)
+            raise StepError(f"slot {dup} occurs twice in one step")
+        live = cache.live
+        for s in slots:
+            if s not in live:
+                raise StepError(f"slot {s} is not held by a live sequence")
+        if tok.min() < 0 or tok.max() >= self.vocab_size:
+            bad = int(tok[(tok < 0) | (tok >= self.vocab_size)][0])
+            raise StepError(f"slot {slots[int(np.where(tok == bad)[0][0])]}: token id {bad} is outside the vocabulary "
+                            f"[0, {self.vocab_size})")
+        want_rows: List[int] = []
+        for i, e in enumerate(entries):
+            for w in e.want:
+                if int(w) != 0:
+                    raise StepError(f"slot {e.slot}: wanted place {w} is outside the 1 tokens of this step")
+                want_rows.append(i)
+        pages = 0
+        for s in slots:
+            have = live[s]
+            if have + 1 > self.max_seq_len:
+                raise StepError(f"slot {s}: {have} cached + 1 new tokens exceed the longest sequence this engine "
+                                f"holds ({self.max_seq_len})")
+            pages += have % cache.page_size == 0
+        if pages > cache.free_page_count():
+            raise StepError(f"the cache is full: this step needs {pages} more pages of {cache.page_size} tokens, "
+                            f"{cache.free_page_count()} are free (max_tokens={self.options.max_tokens})")
+        pos = np.fromiter((cache.extend_one(s) for s in slots), dtype=np.int32, count=B)
+        cache.sync()
+        sl = np.asarray(slots, dtype=np.int32)
+        graph = bool(self.options.hip_graph)
+        rows = np.arange(B, dtype=np.int32) if graph else np.asarray(want_rows, dtype=np.int32)
+        host = np.concatenate([tok.astype(np.int32), pos, sl, np.arange(B + 1, dtype=np.int32), sl, pos + 1, rows])
+        logits = self._run(host, B, B, [1] * B, int(pos.max()), True, graph, int(rows.size))
+        if not want_rows:
+            return None
+        if graph and want_rows != list(range(B)):
+            return logits.index_select(0, torch.tensor(want_rows, dtype=torch.long).to(self.device, non_blocking=True))
+        return logits.clone()
+
+    def _run(self, host: np.ndarray, n: int, B: int, q_lens: List[int], max_pos: int, single: bool, graph: bool,
+             R: int) -> Optional[torch.Tensor]:
+        """Upload one forward pass's metadata (tokens, positions, token slots, sequence starts, sequence slots,
+        sequence lengths, wanted rows) and run it, eagerly or from a captured graph.  Returns the logits of the
+        wanted rows (a view of engine scratch)."""
+        if graph:
+            # a captured step sizes its launches for the largest position of a whole range of steps, so that
+            # one capture serves all of them
+            bound = 256
+            while bound < max_pos + 1:
+                bound *= 2
+            max_pos = min(bound, self.max_seq_len) - 1
+        key = (B, max_pos)
+        entry = self._graphs.get(key) if graph else None
+        if entry is not None and entry[3] != self.workspace.generation:
+            self._graphs.clear()            # scratch buffers moved: what was captured points at freed memory
+            entry = None
+        if graph:
+            meta = entry[1] if entry is not None else torch.zeros(host.size, dtype=torch.int32, device=self.device)
+        else:
+            if host.size > self._meta.numel():
+                self._meta = torch.zeros(host.size * 2, dtype=torch.int32, device=self.device)
+            meta = self._meta
+        self._upload(host, meta)
+        if entry is not None:
+            entry[0].replay()
+            return entry[2]
+        o1, o2, o3 = n, 2 * n, 3 * n
+        o4 = o3 + B + 1
+        o5 = o4 + B
+        o6 = o5 + B
+        ctx = StepContext(
+            n_tokens=n, n_seqs=B, token_ids=meta[0:o1], positions=meta[o1:o2], tok_slot=meta[o2:o3],
+            cu_q=meta[o3:o4], seq_slot=meta[o4:o5], seq_len=meta[o5:o6], q_lens=q_lens,
+            kv_lens=[int(x) for x in host[o5:o6]], max_pos=max_pos, single_token=single,
+            ws=self.workspace, cache=self.cache, logit_rows=meta[o6:o6 + R] if R else None)
+        logits = self.model.forward(ctx)
+        if graph:
+            # the eager run above did this step's work and sized the scratch buffers; recording the same
+            # launches executes nothing and serves the following steps of this batch size
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                captured = self.model.forward(ctx)
+            self._graphs[key] = (g, meta, captured, self.workspace.generation)
+        return logits
 
     def _forward(self, entries, chunk, row_of, result):
         cache = self.cache
@@ -229,52 +327,9 @@ class Engine:
                         dest.append(r)
             o += q
         cache.sync()
-        max_pos = int(pos.max())
-        if graph:
-            # a captured step computes the logits of all its rows, and sizes its launches for the largest
-            # position of a whole range of steps, so that one capture serves all of them
-            bound = 256
-            while bound < max_pos + 1:
-                bound *= 2
-            max_pos = min(bound, self.max_seq_len) - 1
-            want_rows = np.arange(B, dtype=np.int32)
-        else:
-            want_rows = np.asarray(rows, dtype=np.int32)
-        R = int(want_rows.size)
+        want_rows = np.arange(B, dtype=np.int32) if graph else np.asarray(rows, dtype=np.int32)
         host = np.concatenate([tok, pos, tslot, cu, sslot, slen, want_rows])
-        key = (B, max_pos)
-        entry = self._graphs.get(key) if graph else None
-        if entry is not None and entry[3] != self.workspace.generation:
-            self._graphs.clear()            # scratch buffers moved: what was captured points at freed memory
-            entry = None
-        if graph:
-            meta = entry[1] if entry is not None else torch.zeros(host.size, dtype=torch.int32, device=self.device)
-        else:
-            if host.size > self._meta.numel():
-                self._meta = torch.zeros(host.size * 2, dtype=torch.int32, device=self.device)
-            meta = self._meta
-        self._upload(host, meta)
-        if entry is not None:
-            entry[0].replay()
-            logits = entry[2]
-        else:
-            o1, o2, o3 = n, 2 * n, 3 * n
-            o4 = o3 + B + 1
-            o5 = o4 + B
-            o6 = o5 + B
-            ctx = StepContext(
-                n_tokens=n, n_seqs=B, token_ids=meta[0:o1], positions=meta[o1:o2], tok_slot=meta[o2:o3],
-                cu_q=meta[o3:o4], seq_slot=meta[o4:o5], seq_len=meta[o5:o6], q_lens=q_lens,
-                kv_lens=[int(x) for x in slen], max_pos=max_pos, single_token=single,
-                ws=self.workspace, cache=cache, logit_rows=meta[o6:o6 + R] if R else None)
-            logits = self.model.forward(ctx)
-            if graph:
-                # the eager run above did this step's work and sized the scratch buffers; recording the same
-                # launches executes nothing and serves the following steps of this batch size
-                g = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(g):
-                    captured = self.model.forward(ctx)
-                self._graphs[key] = (g, meta, captured, self.workspace.generation)
+        logits = self._run(host, n, B, q_lens, int(pos.max()), single, graph, int(want_rows.size))
         if rows:
             dest_t = torch.tensor([dest, rows], dtype=torch.long).to(self.device, non_blocking=True)
             if graph:
