@@ -100,8 +100,7 @@ class LLM:
             import os
             total = torch.cuda.get_device_properties(torch.device(self.device)).total_memory
             weight_bytes = sum(os.path.getsize(f) for f in checkpoint_files(self.path))
-            if self.dtype == "float32":
-                weight_bytes *= 2
+            weight_bytes *= 2          # float32: upcast weights; bfloat16: the second copy in the decode layout
             model = self.arch.build(self.config, sparse=self.apply_sparse)
             esize = 4 if self.dtype == "float32" else 2
             per_token = sum(sum(s.width / s.every for _, s in n.streams) for n in model.cache_needs()) * esize
