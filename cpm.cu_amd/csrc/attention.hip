@@ -442,8 +442,8 @@ extern "C" const char* cpmcu_attention_mfma(const void* q, void* out, float* par
 // row, and a tile is skipped for chunks that lie behind all of its rows.
 // `tiles` holds, per wavefront, the first packed token and the number of tokens.
 // ===========================================================================
-template <int HD, int R>
-__global__ __launch_bounds__(64) void attention_prefill_mfma_kernel(
+template <int HD, int R, int NW>
+__global__ __launch_bounds__(NW * 64) void attention_prefill_mfma_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ kpool,
     const bf16_t* __restrict__ vtpool, PagedView pv, const int* __restrict__ tiles,
     const int* __restrict__ positions, const int* __restrict__ tok_slot, int nh, int nkv, float scale_log2e,
@@ -452,7 +452,7 @@ __global__ __launch_bounds__(64) void attention_prefill_mfma_kernel(
     constexpr int DT = HD / 16;
     const int tile_id = gridDim.x - 1 - blockIdx.x;      // later tiles of a prompt see more keys: start them first
     const int kvh = blockIdx.y % nkv, ht = blockIdx.y / nkv;
-    const int lane = threadIdx.x, n = lane & 15, g = lane >> 4;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
     const int G = nh / nkv;
     const int t0 = tiles[2 * tile_id], n_tok = tiles[2 * tile_id + 1];
     const int slot = tok_slot[t0];
@@ -517,19 +517,20 @@ __global__ __launch_bounds__(64) void attention_prefill_mfma_kernel(
     };
     // one buffer each for keys and values: the next chunk's keys are asked for as soon as the last tile's
     // scores are issued, its values as soon as the last tile's P.V is, so both arrive behind other work
+    // with NW wavefronts a workgroup the chunks are dealt to them in turn and merged at the end
     abf16x8_t kf[2][KSTEPS], vf[DT];
-    {
-        const int page = ptab[0];
-        load_k(page, 0, kf);
-        load_v(page, 0, vf);
+    if (wave < total_chunks) {
+        const int page = ptab[(wave * 32) / pv.page_size];
+        load_k(page, (wave * 32) % pv.page_size, kf);
+        load_v(page, (wave * 32) % pv.page_size, vf);
     }
-    for (int c = 0; c < total_chunks; ++c) {
+    for (int c = wave; c < total_chunks; c += NW) {
         const int key0 = c * 32;
-        const bool more = c + 1 < total_chunks;
+        const bool more = c + NW < total_chunks;
         int pagen = 0, pon = 0;
         if (more) {
-            pagen = ptab[(key0 + 32) / pv.page_size];
-            pon = (key0 + 32) % pv.page_size;
+            pagen = ptab[(key0 + 32 * NW) / pv.page_size];
+            pon = (key0 + 32 * NW) % pv.page_size;
         }
 #pragma unroll
         for (int r = 0; r < R; ++r) {
@@ -594,6 +595,47 @@ __global__ __launch_bounds__(64) void attention_prefill_mfma_kernel(
         }
         if (more) load_v(pagen, pon, vf);
     }
+    if (NW > 1) {
+        // wavefronts 1.. hand their running results to wavefront 0, one after the other through one buffer
+        __shared__ float ml_s[R][16][2];
+        __shared__ float acc_s[R * DT * 4 * 64];
+        for (int w = 1; w < NW; ++w) {
+            __syncthreads();
+            if (wave == w) {
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    if (g == 0) {
+                        ml_s[r][n][0] = m[r];
+                        ml_s[r][n][1] = l[r];
+                    }
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) acc_s[((r * DT + dt) * 4 + i) * 64 + lane] = acc[r][dt][i];
+                }
+            }
+            __syncthreads();
+            if (wave == 0) {
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const float om = ml_s[r][n][0], ol = ml_s[r][n][1];
+                    if (ol > 0.f) {
+                        const float m_new = fmaxf(m[r], om);
+                        const float sa = l[r] > 0.f ? fast_exp2(m[r] - m_new) : 0.f;
+                        const float sb = fast_exp2(om - m_new);
+                        l[r] = l[r] * sa + ol * sb;
+                        m[r] = m_new;
+#pragma unroll
+                        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                            for (int i = 0; i < 4; ++i)
+                                acc[r][dt][i] = acc[r][dt][i] * sa + acc_s[((r * DT + dt) * 4 + i) * 64 + lane] * sb;
+                    }
+                }
+            }
+        }
+        if (wave != 0) return;
+    }
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         if (!row_ok[r]) continue;
@@ -615,7 +657,7 @@ extern "C" int cpmcu_attention_prefill_tokens_per_wave(int nh, int nkv, int tile
 
 // tiles: int32 [n_tiles, 2] = (first packed token, tokens) with tokens <= cpmcu_attention_prefill_tokens_per_wave
 extern "C" const char* cpmcu_attention_prefill_mfma(const void* q, void* out, int n_tiles, const int* tiles,
-                                                    int tiles_per_wave, int nh,
+                                                    int tiles_per_wave, int waves_per_group, int nh,
                                                     int nkv, int hd, float scale, const void* kpool,
                                                     const void* vtpool, const int* page_table, int table_width,
                                                     int page_size, const int* positions, const int* tok_slot,
@@ -633,15 +675,17 @@ extern "C" const char* cpmcu_attention_prefill_mfma(const void* q, void* out, in
     dim3 grid(n_tiles, nkv * HT);
     const float sl = scale * 1.4426950408889634f;
     CPMCU_REQUIRE(tiles_per_wave == 2 || tiles_per_wave == 4, "attention_prefill: %d tiles a wavefront (2 or 4 are built)", tiles_per_wave);
-#define LAUNCH(HDv, Rv)                                                                                          \
-    attention_prefill_mfma_kernel<HDv, Rv><<<grid, 64, 0, stream>>>((const bf16_t*)q, (bf16_t*)out,              \
-                                                                    (const bf16_t*)kpool, (const bf16_t*)vtpool, \
-                                                                    pv, tiles, positions, tok_slot, nh, nkv, sl, \
-                                                                    rpt, tpt)
-#define BY_R(HDv)                                \
-    do {                                         \
-        if (tiles_per_wave == 4) LAUNCH(HDv, 4); \
-        else LAUNCH(HDv, 2);                     \
+    CPMCU_REQUIRE(waves_per_group == 1 || waves_per_group == 2, "attention_prefill: %d wavefronts a workgroup (1 or 2 are built)", waves_per_group);
+#define LAUNCH(HDv, Rv, NWv)                                                                                     \
+    attention_prefill_mfma_kernel<HDv, Rv, NWv><<<grid, NWv * 64, 0, stream>>>(                                  \
+        (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kpool, (const bf16_t*)vtpool, pv, tiles, positions,       \
+        tok_slot, nh, nkv, sl, rpt, tpt)
+#define BY_R(HDv)                                                               \
+    do {                                                                        \
+        if (tiles_per_wave == 4 && waves_per_group == 2) LAUNCH(HDv, 4, 2);     \
+        else if (tiles_per_wave == 4) LAUNCH(HDv, 4, 1);                        \
+        else if (waves_per_group == 2) LAUNCH(HDv, 2, 2);                       \
+        else LAUNCH(HDv, 2, 1);                                                 \
     } while (0)
     if (hd == 16) BY_R(16);
     else if (hd == 32) BY_R(32);

@@ -235,18 +235,21 @@ def attention_prefill_tokens_per_wave(nh: int, nkv: int, tiles_per_wave: int = 4
     return int(lib.cpmcu_attention_prefill_tokens_per_wave(c_int(nh), c_int(nkv), c_int(tiles_per_wave)))
 
 
-def attention_prefill_tiles_per_wave(n_tokens: int, nh: int, nkv: int, hd: int) -> int:
-    """4 tiles of 16 rows a wavefront halve the cache traffic of 2 and run long prompts faster; a short
-    prompt has too few wavefronts for the 256 CUs with 4 (measured on the MI355X at head size 128: 2,048
-    tokens 150 us with 2 against 192 us with 4; 8,192 tokens 1.89 ms against 1.38 ms)."""
+def attention_prefill_shape(n_tokens: int, nh: int, nkv: int, hd: int):
+    """(tiles a wavefront, wavefronts a workgroup) for the prompt kernel.  4 tiles of 16 rows a wavefront
+    halve the cache traffic of 2; when a prompt is too short to give every SIMD of the 256 CUs a wavefront of
+    its own twice over, two wavefronts share each group of tiles, taking the chunks of keys in turn, which also
+    evens out the causal triangle (measured on the MI355X at head size 128, 2,048 tokens: 128 us against 189 us
+    with one wavefront and 148 us with 2 tiles; at 8,192 tokens one wavefront is best, 1.36 ms)."""
     per4 = attention_prefill_tokens_per_wave(nh, nkv, 4)
     waves4 = -(-n_tokens // per4) * nkv * -(-(nh // nkv) // 16)
-    return 4 if waves4 >= 2048 else 2
+    return 4, (2 if waves4 < 2048 else 1)
 
 
 def attention_prefill_mfma(q: torch.Tensor, out: torch.Tensor, tiles: torch.Tensor, nh: int, nkv: int, hd: int,
                            scale: float, kpool: torch.Tensor, vpool: torch.Tensor, page_table: torch.Tensor,
-                           page_size: int, positions: torch.Tensor, tok_slot: torch.Tensor, tiles_per_wave: int = 4):
+                           page_size: int, positions: torch.Tensor, tok_slot: torch.Tensor, tiles_per_wave: int = 4,
+                           waves_per_group: int = 1):
     """Dense causal bf16 attention for prompts: tiles int32 [T, 2] = (first packed token, tokens), each a run of
     consecutive tokens of one sequence, at most attention_prefill_tokens_per_wave(nh, nkv, tiles_per_wave) long."""
     _need(q, "attention q", torch.bfloat16, (None, nh * hd))
@@ -259,7 +262,8 @@ def attention_prefill_mfma(q: torch.Tensor, out: torch.Tensor, tiles: torch.Tens
     _need(positions, "attention positions", torch.int32, (n,))
     _need(tok_slot, "attention token slots", torch.int32, (n,))
     _check(_fn("attention", "cpmcu_attention_prefill_mfma")(
-        _p(q), _p(out), c_int(tiles.shape[0]), _p(tiles), c_int(tiles_per_wave), c_int(nh), c_int(nkv), c_int(hd),
+        _p(q), _p(out), c_int(tiles.shape[0]), _p(tiles), c_int(tiles_per_wave), c_int(waves_per_group), c_int(nh),
+        c_int(nkv), c_int(hd),
         c_float(scale),
         _p(kpool), _p(vpool), _p(page_table), c_int(page_table.shape[1]), c_int(page_size), _p(positions),
         _p(tok_slot), _stream()))
@@ -449,14 +453,14 @@ def attention(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, c
               sel_blocks=None, sel_count=None, block_size=0):
     """Attention of the step's queries over the cache, with the kernel that suits the step."""
     if sel_count is None and not ctx.single_token and attention_mfma_ok(q, hd, page_size):
-        r = attention_prefill_tiles_per_wave(q.shape[0], nh, nkv, hd)
+        r, nw = attention_prefill_shape(q.shape[0], nh, nkv, hd)
         tpw = attention_prefill_tokens_per_wave(nh, nkv, r)
         key = ("prefill_tiles", tpw)
         tiles = ctx.extras.get(key)
         if tiles is None:
             tiles = ctx.extras[key] = prefill_tiles(ctx.q_lens, tpw, q.device)
         attention_prefill_mfma(q, out, tiles, nh, nkv, hd, scale, kpool, vpool, page_table, page_size,
-                               ctx.positions, ctx.tok_slot, r)
+                               ctx.positions, ctx.tok_slot, r, nw)
         return
     if attention_mfma_ok(q, hd, page_size, block_size if sel_count is not None else 0):
         n = q.shape[0]

@@ -233,12 +233,12 @@ def test_attention_over_scrambled_pages(nh, nkv, hd, dtype):
                                splits, po, pm, waves_per_group=nw)
             assert float((out.double().cpu().view(n, nh, hd) - ref).abs().max()) <= tol, f"splits={splits} waves={nw}"
         # the prompt kernel: runs of consecutive tokens of one sequence share a wavefront
-        for r in (2, 4):
+        for r, nw in ((2, 1), (4, 1), (2, 2), (4, 2)):
             tpw = ops.attention_prefill_tokens_per_wave(nh, nkv, r)
             tiles = ops.prefill_tiles([40, 1, 1], tpw, DEV)
             out.fill_(float("nan"))
             ops.attention_prefill_mfma(q.view(n, -1), out, tiles, nh, nkv, hd, scale, kpool, vpool, table, page, pos_t,
-                                       slot_t, r)
+                                       slot_t, r, nw)
             assert float((out.double().cpu().view(n, nh, hd) - ref).abs().max()) <= tol, "prompt kernel"
     elif dtype == torch.bfloat16:
         assert not ops.attention_mfma_ok(q.view(n, -1), hd, page)
@@ -264,15 +264,15 @@ def test_prompt_attention_from_position_zero_and_continued(nh, nkv, hd):
     ref = attention_reference(q.double().cpu(), ks, vs, positions, seq_of, nh, scale)
     pos_t = torch.tensor(positions, dtype=torch.int32, device=DEV)
     slot_t = torch.tensor(seq_of, dtype=torch.int32, device=DEV)
-    for r in (2, 4):
+    for r, nw in ((2, 1), (4, 1), (2, 2), (4, 2)):
         tiles = ops.prefill_tiles(q_lens, ops.attention_prefill_tokens_per_wave(nh, nkv, r), DEV)
         out = torch.full((n, nh * hd), float("nan"), dtype=dtype, device=DEV)
         ops.attention_prefill_mfma(q.view(n, -1), out, tiles, nh, nkv, hd, scale, kpool, vpool, table, page, pos_t,
-                                   slot_t, r)
+                                   slot_t, r, nw)
         # the output is rounded to bf16 (8 significant bits): allow its half ulp at the size of each token's values
         err = (out.double().cpu().view(n, nh, hd) - ref).abs().amax(dim=(1, 2))
         bad = (err > 2 ** -7 * ref.abs().amax(dim=(1, 2)).clamp(min=1.0)).nonzero().flatten()
-        assert bad.numel() == 0, f"first wrong token {int(bad[0])} (position {positions[int(bad[0])]}), {r} tiles a wave"
+        assert bad.numel() == 0, f"first wrong token {int(bad[0])} (position {positions[int(bad[0])]}), {r} tiles, {nw} waves"
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
