@@ -246,9 +246,12 @@ __global__ void rope_store_kernel(const IT* __restrict__ qkv, long width, int np
                                   T* __restrict__ q_out, int nh, int nkv, int hd, const int* __restrict__ positions,
                                   const int* __restrict__ tok_slot, const float* __restrict__ inv_freq, float mscale,
                                   T* __restrict__ kpool, T* __restrict__ vpool, PagedView pv, int write_kv) {
-    // one block per (token, head): heads [0, nh) are queries, then nkv key heads, then nkv value heads
+    // 64 threads per (token, head): heads [0, nh) are queries, then nkv key heads, then nkv value heads;
+    // a block holds blockDim.x / 64 heads of one token
     const long t = blockIdx.x;
-    const int head = blockIdx.y;
+    const int head = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (head >= nh + (write_kv ? 2 * nkv : 0)) return;
     const int half = hd / 2;
     const int pos = positions[t];
     const IT* row = qkv + t * width + (long)head * hd;
@@ -262,7 +265,7 @@ __global__ void rope_store_kernel(const IT* __restrict__ qkv, long width, int np
     if (head < nh + nkv) {
         T* dst = head < nh ? q_out + (t * nh + head) * (long)hd
                            : kpool + kv_row * (long)nkv * hd + (long)(head - nh) * hd;
-        for (int c = threadIdx.x; c < half; c += blockDim.x) {
+        for (int c = lane; c < half; c += 64) {
             float cs = 1.f, sn = 0.f;
             if (inv_freq) {
                 const float ang = (float)pos * inv_freq[c];
@@ -279,7 +282,7 @@ __global__ void rope_store_kernel(const IT* __restrict__ qkv, long width, int np
         const long page = kv_row / pv.page_size;
         const int in_page = (int)(kv_row - page * pv.page_size);
         T* dst = vpool + (page * nkv + (head - nh - nkv)) * (long)hd * pv.page_size + in_page;
-        for (int d = threadIdx.x; d < hd; d += blockDim.x) dst[(long)d * pv.page_size] = from_f32<T>(load(d));
+        for (int d = lane; d < hd; d += 64) dst[(long)d * pv.page_size] = from_f32<T>(load(d));
     }
 }
 
@@ -297,9 +300,12 @@ extern "C" const char* cpmcu_rope_store(const void* qkv, long row_width, int in_
                   "rope_store: a row of %ld elements cannot hold %d query%s heads of %d", row_width, nh,
                   write_kv ? " and key/value" : "", hd);
     PagedView pv{page_table, table_width, page_size};
-    const int block = hd >= 128 ? 64 : (hd / 2 > 32 ? 64 : 32);
-    CPMCU_REQUIRE(nh + 2 * nkv <= 65535, "rope_store: %d heads exceed the launch grid", nh + 2 * nkv);
-    dim3 grid(n, nh + (write_kv ? 2 * nkv : 0));
+    // few tokens (decode steps): a block a head, for more blocks; many: 4 heads a block
+    const int heads = nh + (write_kv ? 2 * nkv : 0);
+    const int hpb = n >= 64 ? 4 : 1;
+    const int block = 64 * hpb;
+    CPMCU_REQUIRE(heads <= 65535, "rope_store: %d heads exceed the launch grid", heads);
+    dim3 grid(n, (heads + hpb - 1) / hpb);
 #define LAUNCH(IT, T)                                                                                          \
     rope_store_kernel<IT, T><<<grid, block, 0, stream>>>((const IT*)qkv, row_width, nparts, part_stride, (T*)q_out, nh, nkv, \
                                                       hd, positions, tok_slot, inv_freq, mscale, (T*)kpool,   \
