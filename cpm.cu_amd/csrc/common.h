@@ -63,13 +63,10 @@ __device__ inline float block_sum(float v, float* red) {
     __syncthreads();
     if (lane == 0) red[w] = v;
     __syncthreads();
-    if (threadIdx.x == 0) {
-        float t = 0.f;
-        for (int i = 0; i < nw; ++i) t += red[i];
-        red[16] = t;
-    }
-    __syncthreads();
-    return red[16];
+    // every thread adds the wave sums in the same order
+    float t = 0.f;
+    for (int i = 0; i < nw; ++i) t += red[i];
+    return t;
 }
 __device__ inline float block_max(float v, float* red) {
     const int lane = threadIdx.x & (CPMCU_WAVE - 1), w = threadIdx.x / CPMCU_WAVE;
@@ -78,13 +75,9 @@ __device__ inline float block_max(float v, float* red) {
     __syncthreads();
     if (lane == 0) red[w] = v;
     __syncthreads();
-    if (threadIdx.x == 0) {
-        float t = red[0];
-        for (int i = 1; i < nw; ++i) t = fmaxf(t, red[i]);
-        red[16] = t;
-    }
-    __syncthreads();
-    return red[16];
+    float t = red[0];
+    for (int i = 1; i < nw; ++i) t = fmaxf(t, red[i]);
+    return t;
 }
 
 // ---- error convention ----

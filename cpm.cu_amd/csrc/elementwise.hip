@@ -97,8 +97,8 @@ __global__ __launch_bounds__(1024) void add_rms_norm_vec4_kernel(float* __restri
     const long r = rows ? rows[r_out] : r_out;
     float* xr = x + r * H;
     const int H4 = H / 4;
-    float ss = 0.f;
-    for (int c = threadIdx.x; c < H4; c += blockDim.x) {
+    OT* o = out + r_out * H;
+    auto summed = [&](int c) {
         float4 v = *(const float4*)(xr + 4 * c);
         if (branch) {
             float4 b = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -107,28 +107,40 @@ __global__ __launch_bounds__(1024) void add_rms_norm_vec4_kernel(float* __restri
                 b.x += t.x; b.y += t.y; b.z += t.z; b.w += t.w;
             }
             v.x += bscale * b.x; v.y += bscale * b.y; v.z += bscale * b.z; v.w += bscale * b.w;
-            if (!rows) *(float4*)(xr + 4 * c) = v;
         }
-        ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
-    }
-    ss = block_sum(ss, red);
-    const float rs = 1.0f / sqrtf(ss / (float)H + eps);
-    OT* o = out + r_out * H;
-    for (int c = threadIdx.x; c < H4; c += blockDim.x) {
-        float4 v = *(const float4*)(xr + 4 * c);
-        if (branch && rows) {
-            float4 b = make_float4(0.f, 0.f, 0.f, 0.f);
-            for (int p = 0; p < nparts; ++p) {
-                const float4 t = load4(branch + p * part_stride + r * H + 4 * c);
-                b.x += t.x; b.y += t.y; b.z += t.z; b.w += t.w;
-            }
-            v.x += bscale * b.x; v.y += bscale * b.y; v.z += bscale * b.z; v.w += bscale * b.w;
-        }
+        return v;
+    };
+    auto emit = [&](int c, float4 v, float rs) {
         const float4 wv = *(const float4*)(w + 4 * c);
         o[4 * c + 0] = from_f32<OT>(v.x * rs * wv.x);
         o[4 * c + 1] = from_f32<OT>(v.y * rs * wv.y);
         o[4 * c + 2] = from_f32<OT>(v.z * rs * wv.z);
         o[4 * c + 3] = from_f32<OT>(v.w * rs * wv.w);
+    };
+    if (H4 <= (int)blockDim.x) {
+        // the whole row fits the block: each thread keeps its 4 columns in registers between the two phases
+        const int c = threadIdx.x;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (c < H4) {
+            v = summed(c);
+            if (branch && !rows) *(float4*)(xr + 4 * c) = v;
+        }
+        const float ss = block_sum(v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w, red);
+        if (c < H4) emit(c, v, 1.0f / sqrtf(ss / (float)H + eps));
+        return;
+    }
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < H4; c += blockDim.x) {
+        const float4 v = summed(c);
+        if (branch && !rows) *(float4*)(xr + 4 * c) = v;
+        ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+    }
+    ss = block_sum(ss, red);
+    const float rs = 1.0f / sqrtf(ss / (float)H + eps);
+    for (int c = threadIdx.x; c < H4; c += blockDim.x) {
+        // x holds the sum already unless only chosen rows are normed (then it is formed again)
+        const float4 v = (branch && rows) ? summed(c) : *(const float4*)(xr + 4 * c);
+        emit(c, v, rs);
     }
 }
 
