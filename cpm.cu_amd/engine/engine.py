@@ -177,15 +177,24 @@ class Engine:
         if cur:
             yield cur
 
-    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    accepts_device_tokens = True
+
+    def step(self, entries: Sequence[StepEntry], device_tokens: Optional[torch.Tensor] = None
+             ) -> Optional[torch.Tensor]:
         """Run the entries' tokens; float32 logits [wanted, vocab] in the order of entries and of ``want``
-        (None if nothing is wanted)."""
+        (None if nothing is wanted).  ``device_tokens`` (int32 [entries], on the GPU; single-token steps only)
+        replaces the entries' token ids: a decode loop can feed what it sampled without reading it back."""
         entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
         if entries and len(entries) <= self.max_step_tokens and all(len(e.tokens) == 1 for e in entries):
+            if device_tokens is not None and (device_tokens.dtype != torch.int32 or device_tokens.device != self.device
+                                              or tuple(device_tokens.shape) != (len(entries),)):
+                raise StepError(f"device_tokens must be int32 [{len(entries)}] on {self.device}")
             with torch.cuda.device(self.device):
-                out = self._step_single_tokens(entries)
+                out = self._step_single_tokens(entries, device_tokens)
             self.steps_run += 1
             return out
+        if device_tokens is not None:
+            raise StepError("device_tokens serve steps in which every sequence brings exactly one token")
         self._validate(entries)
         row_of: Dict[Tuple[int, int], List[int]] = {}
         n_rows = 0
@@ -200,7 +209,7 @@ class Engine:
         self.steps_run += 1
         return result
 
-    def _step_single_tokens(self, entries) -> Optional[torch.Tensor]:
+    def _step_single_tokens(self, entries, device_tokens=None) -> Optional[torch.Tensor]:
         """The step of a decode loop: every sequence brings one token.  The same checks and the same forward
         pass as the general path, with the bookkeeping done on whole arrays."""
         cache = self.cache
@@ -214,7 +223,7 @@ class Engine:
         for s in slots:
             if s not in live:
                 raise StepError(f"slot {s} is not held by a live sequence")
-        if tok.min() < 0 or tok.max() >= self.vocab_size:
+        if device_tokens is None and (tok.min() < 0 or tok.max() >= self.vocab_size):
             bad = int(tok[(tok < 0) | (tok >= self.vocab_size)][0])
             raise StepError(f"slot {slots[int(np.where(tok == bad)[0][0])]}: token id {bad} is outside the vocabulary "
                             f"[0, {self.vocab_size})")
@@ -240,7 +249,7 @@ class Engine:
         graph = bool(self.options.hip_graph)
         rows = np.arange(B, dtype=np.int32) if graph else np.asarray(want_rows, dtype=np.int32)
         host = np.concatenate([tok.astype(np.int32), pos, sl, np.arange(B + 1, dtype=np.int32), sl, pos + 1, rows])
-        logits = self._run(host, B, B, [1] * B, int(pos.max()), True, graph, int(rows.size))
+        logits = self._run(host, B, B, [1] * B, int(pos.max()), True, graph, int(rows.size), device_tokens)
         if not want_rows:
             return None
         if graph and want_rows != list(range(B)):
@@ -248,7 +257,7 @@ class Engine:
         return logits.clone()
 
     def _run(self, host: np.ndarray, n: int, B: int, q_lens: List[int], max_pos: int, single: bool, graph: bool,
-             R: int) -> Optional[torch.Tensor]:
+             R: int, device_tokens: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Upload one forward pass's metadata (tokens, positions, token slots, sequence starts, sequence slots,
         sequence lengths, wanted rows) and run it, eagerly or from a captured graph.  Returns the logits of the
         wanted rows (a view of engine scratch)."""
@@ -271,6 +280,8 @@ class Engine:
                 self._meta = torch.zeros(host.size * 2, dtype=torch.int32, device=self.device)
             meta = self._meta
         self._upload(host, meta)
+        if device_tokens is not None:
+            meta[:n].copy_(device_tokens)
         if entry is not None:
             entry[0].replay()
             return entry[2]

@@ -77,8 +77,9 @@ def generate(engine: Engine, prompts: Sequence[Sequence[int]], max_new_tokens: i
     batches = plan_batches([len(p) for p in prompts], max_new_tokens, max_batch, engine.options.max_tokens,
                            engine.cache.page_size, engine.max_seq_len)
     results: List[Optional[Completion]] = [None] * len(prompts)
+    run = _run_batch_overlapped if getattr(engine, "accepts_device_tokens", False) else _run_batch
     for batch in batches:
-        _run_batch(engine, prompts, batch, max_new_tokens, stop, sampler, results, on_token, on_prefill)
+        run(engine, prompts, batch, max_new_tokens, stop, sampler, results, on_token, on_prefill)
     return results  # type: ignore[return-value]
 
 
@@ -123,6 +124,83 @@ def _run_batch(engine, prompts, batch, max_new_tokens, stop, sampler, results, o
             active = [i for i, _ in nxt]
             logits = engine.step([StepEntry(slots[i], [t], [0]) for i, t in nxt])
             tokens = sampler.sample(logits, active, [len(out[i]) for i in active]).tolist()
+    finally:
+        for s in slots.values():
+            engine.release(s)
+
+
+def _run_batch_overlapped(engine, prompts, batch, max_new_tokens, stop, sampler, results, on_token, on_prefill):
+    """The same loop with the host one step behind the GPU: the tokens a step samples stay on the device and
+    feed the next step directly, while the host reads the previous step's tokens and decides who has ended.
+    A sequence that ends on a stop token has then already been fed once more; that step's token is dropped
+    (its cache rows die with the slot).  Sequences that end by length are known beforehand and are not fed."""
+    slots = {i: engine.acquire() for i in batch}
+    out: Dict[int, List[int]] = {i: [] for i in batch}
+    n_gen: Dict[int, int] = {}
+    finished = set()
+    staging = [torch.empty(len(batch), dtype=torch.int32).pin_memory() for _ in range(2)]
+    try:
+        _sync(engine)
+        t0 = time.time()
+        if on_prefill:
+            on_prefill("begin", {"total_tokens": sum(len(prompts[i]) for i in batch)})
+        logits = engine.step([StepEntry(slots[i], list(prompts[i]), [len(prompts[i]) - 1]) for i in batch])
+        first = sampler.sample(logits, batch, [0] * len(batch))
+        tokens = first.tolist()
+        prefill_time = time.time() - t0
+        if on_prefill:
+            on_prefill("finish", {"total_time": prefill_time})
+        t1 = time.time()
+
+        def resolve(ids, toks):
+            for i, t in zip(ids, toks):
+                if i in finished:
+                    continue
+                out[i].append(t)
+                if on_token:
+                    on_token(i, t)
+                reason = "stop" if t in stop else ("length" if len(out[i]) >= max_new_tokens else None)
+                if reason:
+                    finished.add(i)
+                    results[i] = Completion(out[i], reason, prefill_time, time.time() - t1)
+                    engine.release(slots.pop(i))
+
+        for i in batch:
+            n_gen[i] = 1
+        resolve(batch, tokens)
+        active = [i for i in batch if i not in finished]
+        feed_host: Optional[List[int]] = [out[i][-1] for i in active]
+        feed_dev = None
+        inflight = None
+        turn = 0
+        while active or inflight is not None:
+            launched = None
+            if active:
+                entries = [StepEntry(slots[i], [feed_host[k] if feed_host is not None else 0], [0])
+                           for k, i in enumerate(active)]
+                logits = engine.step(entries, device_tokens=feed_dev)
+                sampled = sampler.sample(logits, active, [n_gen[i] for i in active])
+                for i in active:
+                    n_gen[i] += 1
+                host = staging[turn][:len(active)]
+                turn ^= 1
+                host.copy_(sampled, non_blocking=True)
+                ev = torch.cuda.Event()
+                ev.record()
+                launched = (list(active), sampled, host, ev)
+            if inflight is not None:
+                ids, _, host, ev = inflight
+                ev.synchronize()
+                resolve(ids, host.tolist())
+            inflight = launched
+            active, feed_host, feed_dev = [], None, None
+            if inflight is not None:
+                ids, sampled = inflight[0], inflight[1]
+                keep = [k for k, i in enumerate(ids) if i not in finished and n_gen[i] < max_new_tokens]
+                active = [ids[k] for k in keep]
+                if active:
+                    feed_dev = sampled if len(keep) == len(ids) else sampled.index_select(
+                        0, torch.tensor(keep, dtype=torch.long).to(sampled.device, non_blocking=True))
     finally:
         for s in slots.values():
             engine.release(s)

@@ -204,3 +204,30 @@ def test_captured_decode_steps_equal_eager_ones(model_dirs, references, name, dt
     got = schedules.tail(eng, {"d": reqs["d"]}, 40)
     check(got, {"d": refs["d"]}, dtype, "graph tail")
     eng.cache.check()
+
+
+@pytest.mark.parametrize("temperature", [0.0, 0.8])
+def test_overlapped_generation_loop_equals_the_plain_loop(model_dirs, references, temperature):
+    """The loop that keeps sampled tokens on the device and runs the host one step behind gives the same
+    completions as the simple loop: stop tokens in the middle of a batch, unequal lengths, two batches."""
+    from cpmcu_amd.engine import generate as gen
+    from cpmcu_amd.sampling import Sampler
+    cfg, w, reqs, _ = references["B"]
+    eng = engine_for(model_dirs, "B", "float32", hip_graph=True)
+    prompts = [reqs["a"][:20], reqs["b"][:75], reqs["c"][:3], reqs["d"][:40], reqs["e"][:9]]
+
+    def run(fn, stop):
+        results = [None] * len(prompts)
+        for batch in ([0, 1, 2], [3, 4]):
+            fn(eng, prompts, batch, 12, set(stop), Sampler(temperature, seed=5), results, None, None)
+        eng.cache.check()
+        assert not eng.cache.live
+        return [(c.tokens, c.finish_reason) for c in results]
+
+    free = run(gen._run_batch, [])
+    assert run(gen._run_batch_overlapped, []) == free
+    # stop on tokens that occur in the middle of some completions
+    stops = [free[0][0][4], free[3][0][7]]
+    plain_loop = run(gen._run_batch, stops)
+    assert any(r == "stop" for _, r in plain_loop) and any(r == "length" for _, r in plain_loop)
+    assert run(gen._run_batch_overlapped, stops) == plain_loop
