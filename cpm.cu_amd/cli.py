@@ -196,6 +196,10 @@ def run_generation(args):
 
 
 def main(argv=None):
+    # a fatal signal prints the Python stack of every thread (the reference installs handlers that print a
+    # native backtrace, src/signal_handler.cu:7-124)
+    import faulthandler
+    faulthandler.enable()
     try:
         run_generation(parse_cli_args(argv))
     except (ValueError, FileNotFoundError) as e:

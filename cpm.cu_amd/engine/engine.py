@@ -79,6 +79,7 @@ class Engine:
         self._meta = torch.zeros(cap, dtype=torch.int32, device=self.device)
         self.vocab_size = model.vocab_size
         self.steps_run = 0
+        self.perf = None                       # utils.perf.PerfTimers; while enabled, steps run eagerly (no graph)
         self._graphs: Dict[Tuple[int, int], tuple] = {}
         self._stage = [torch.empty(cap, dtype=torch.int32).pin_memory() for _ in range(4)]
         self._stage_ev: List[Optional[torch.cuda.Event]] = [None] * 4
@@ -261,6 +262,8 @@ class Engine:
         """Upload one forward pass's metadata (tokens, positions, token slots, sequence starts, sequence slots,
         sequence lengths, wanted rows) and run it, eagerly or from a captured graph.  Returns the logits of the
         wanted rows (a view of engine scratch)."""
+        perf_on = self.perf is not None and self.perf.enabled
+        graph = graph and not perf_on
         if graph:
             # a captured step sizes its launches for the largest position of a whole range of steps, so that
             # one capture serves all of them
@@ -293,7 +296,8 @@ class Engine:
             n_tokens=n, n_seqs=B, token_ids=meta[0:o1], positions=meta[o1:o2], tok_slot=meta[o2:o3],
             cu_q=meta[o3:o4], seq_slot=meta[o4:o5], seq_len=meta[o5:o6], q_lens=q_lens,
             kv_lens=[int(x) for x in host[o5:o6]], max_pos=max_pos, single_token=single,
-            ws=self.workspace, cache=self.cache, logit_rows=meta[o6:o6 + R] if R else None)
+            ws=self.workspace, cache=self.cache, logit_rows=meta[o6:o6 + R] if R else None,
+            perf=self.perf if perf_on else None)
         logits = self.model.forward(ctx)
         if graph:
             # the eager run above did this step's work and sized the scratch buffers; recording the same

@@ -124,6 +124,7 @@ class LLM:
         raw = read_config_json(self.path)
         # the engine reads config.json itself; sparse overrides are handed over through the typed config
         self.engine = Engine.from_dir(self.path, opts, config=self.config)
+        self.engine.perf = self.perf
         return self
 
     def _need_engine(self) -> Engine:

@@ -104,6 +104,7 @@ class StepContext:
     cache: Optional[SequenceCache]
     logit_rows: Optional[torch.Tensor] = None     # int32 [R]: packed token rows whose logits are wanted
     extras: Dict[str, object] = field(default_factory=dict)   # what kernels derive from the batch once a step
+    perf: Optional[object] = None                 # label-keyed timers (utils.perf.PerfTimers) when switched on
 
 
 @dataclass

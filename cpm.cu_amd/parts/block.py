@@ -28,6 +28,18 @@ class PreNormBlock(Block):
         return [self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward]
 
     def forward(self, stream: ResidualStream, ctx: StepContext, cache: Optional[CacheView], writes_cache: bool = True):
+        if ctx.perf is not None and ctx.perf.enabled:
+            # the reference's timer labels distinguish prefill from decode and attention from feed-forward
+            # (src/model/minicpm4/minicpm4_layer.cuh:46-83)
+            phase = "decode" if ctx.single_token else "prefill"
+            with ctx.perf.gpu(f"{phase}_attn"):
+                h = self.mixer_norm.forward(stream.x, stream.pending, stream.pending_scale, ctx, tag="block.h")
+                a = self.mixer.forward(h, ctx, cache, writes_cache)
+            with ctx.perf.gpu(f"{phase}_ffn"):
+                h = self.ff_norm.forward(stream.x, a, self.residual_scale, ctx, tag="block.h")
+                stream.pending = self.feed_forward.forward(h, ctx)
+            stream.pending_scale = self.residual_scale
+            return
         h = self.mixer_norm.forward(stream.x, stream.pending, stream.pending_scale, ctx, tag="block.h")
         a = self.mixer.forward(h, ctx, cache, writes_cache)
         h = self.ff_norm.forward(stream.x, a, self.residual_scale, ctx, tag="block.h")

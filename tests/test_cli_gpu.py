@@ -25,8 +25,9 @@ def test_cli_generates_from_token_ids(model_dirs, tmp_path):
     ids = tmp_path / "ids.txt"
     ids.write_text("\n".join(" ".join(map(str, p)) for p in prompts) + "\n")
     p = run_cli("--model-path", model_dirs["A"], "--dtype", "float32", "--prompt-ids", str(ids), "--num-generate", "5",
-                "--ignore-eos", "true", "--max-tokens", "512", "--use_stream", "false")
+                "--ignore-eos", "true", "--max-tokens", "512", "--use_stream", "false", "--perf")
     assert p.returncode == 0, p.stderr[-1500:]
+    assert "prefill_attn" in p.stdout and "decode_ffn" in p.stdout and "GPU memory" in p.stdout      # the timer summary
     lines = [l for l in p.stdout.splitlines() if l.startswith("[")]
     want = [plain.greedy(cfg, w, pr, 5) for pr in prompts]
     assert [[int(t) for t in l.split(") ")[1].split()] for l in lines] == want
