@@ -281,12 +281,14 @@ def prefill_tiles(q_lens: Sequence[int], tokens_per_wave: int, device) -> torch.
 
 
 def attention_splits(n_tokens: int, nkv: int, group: int, max_keys: int) -> int:
-    """Shares of a token's keys for steps of few tokens: about 512 workgroups of 4 wavefronts fill the 256
-    CUs; a share should still hold 512 keys (4 chunks of 32 for each wavefront)."""
+    """Shares of a token's keys for steps of few tokens.  Measured on the MI355X (head size 128, 2 kv heads,
+    workgroups of 4 wavefronts, graph replay, attention + merge): 8 sequences at 4,096 keys 60/36/24/17/18/25 us
+    for 1/2/4/8/16/32 shares; 64 sequences 68/46/50/51/59 us; 8 sequences at 32,768 keys 124/68/50/60 us for
+    4/8/16/32.  So: about 256 workgroups in all, and a share of at least 512 keys."""
     if n_tokens > 256:
         return 1
     groups = n_tokens * nkv * -(-group // 16)
-    return max(1, min(512 // max(groups, 1), max_keys // 512, 64))
+    return max(1, min(256 // max(groups, 1), max_keys // 512, 64))
 
 
 def compress_keys(kpool: torch.Tensor, ckpool: torch.Tensor, page_table: torch.Tensor, page_size: int,
