@@ -74,7 +74,7 @@ def create_cli_parser() -> argparse.ArgumentParser:
                    help="File of token ids: one prompt a line, ids separated by blanks or commas (no tokenizer needed)")
     p.add_argument("--prompt-lens", "--prompt_lens", type=str, default=None,
                    help="Comma-separated lengths of random prompts, e.g. 5,11,17 (ids uniform from --seed)")
-    p.add_argument("--batch", type=int, default=None, help="Most sequences that run together (default: all that fit)")
+    p.add_argument("--batch", "--max-slots", "--max_slots", dest="batch", type=int, default=None, help="Most sequences that run together (default: all that fit)")
 
     g = parser.add_argument_group("Generation Configuration")
     _flag(g, "--use-stream", "--use_stream", default=True, help="Use stream generation (default: True)")

@@ -27,6 +27,7 @@ __global__ __launch_bounds__(64) void attention_paged_kernel(
     __syncthreads();
     const long kv_stride = (long)nkv * hd;
     const int nd = (hd + 63) / 64;
+    const int vt = value_tile(pv.page_size);
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, l = 0.f;
 
@@ -68,12 +69,12 @@ __global__ __launch_bounds__(64) void attention_paged_kernel(
             for (int jj = 0; jj < cnt; ++jj) {
                 const float pj = __shfl(p, jj, 64);
                 const int rj = __shfl(row, jj, 64);
-                // values are transposed inside a page: [page][kv head][d][token of the page]
+                // values are transposed in tiles of tokens inside a page (value_index)
                 const int pg = rj / pv.page_size;
-                const T* vr = vpool + ((long)pg * kv_stride + (long)g * hd) * pv.page_size + (rj - pg * pv.page_size);
+                const T* vr = vpool + value_index(pg, rj - pg * pv.page_size, g, 0, nkv, hd, pv.page_size);
                 for (int i = 0; i < nd; ++i) {
                     const int d = lane + 64 * i;
-                    if (d < hd) acc[i] += pj * to_f32(vr[(long)d * pv.page_size]);
+                    if (d < hd) acc[i] += pj * to_f32(vr[(long)d * vt]);
                 }
             }
         }
@@ -125,7 +126,7 @@ extern "C" const char* cpmcu_attention_plain(const void* q, void* out, int dtype
 //                      B = Q^T held in registers for the whole kernel
 //   P^T = exp2(S^T*c - m) in float, per head (a D column), running max/sum
 //   O^T += V^T . P^T   A = V^T: 16 d x 32 keys, one 16-byte load a lane because
-//                      values are stored transposed inside a page
+//                      values are stored transposed in tiles of 32 tokens inside a page
 // The two key tiles of a chunk take keys {8g..8g+3} and {8g+4..8g+7} of every
 // group of 8 so that a lane's 8 probabilities are 8 consecutive keys, the order
 // the V^T vector has.  With 4 wavefronts a workgroup (decode steps) the wavefronts take
@@ -143,18 +144,36 @@ typedef float afloatx4_t __attribute__((ext_vector_type(4)));
 // normal range come out as 0, which is what a probability that small contributes anyway
 __device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-template <int HD, int NW>
-__global__ __launch_bounds__(NW * 64) void attention_mfma_kernel(
+template <int HD, int NW, int TW>
+__global__ __launch_bounds__(NW * TW * 64) void attention_mfma_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, float* __restrict__ part_o, float2* __restrict__ part_ml,
     const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vtpool, PagedView pv,
     const int* __restrict__ positions, const int* __restrict__ tok_slot, int nh, int nkv, float scale_log2e,
-    const int* __restrict__ sel_blocks, const int* __restrict__ sel_count, int max_sel, int block_size, int n_splits) {
+    const int* __restrict__ sel_blocks, const int* __restrict__ sel_count, int max_sel, int block_size, int n_splits,
+    int xcd_major, int n_tokens, int last_blocks_first) {
+    static_assert(NW == 1 || TW == 1, "either the wavefronts of a workgroup share a token or each has its own");
     constexpr int KSTEPS = (HD + 31) / 32;
     constexpr int DT = HD / 16;
-    const int t = blockIdx.x;
-    const int kvh = blockIdx.y % nkv, ht = blockIdx.y / nkv;
+    int t = blockIdx.x, by = blockIdx.y;
+    if (xcd_major) {
+        // Workgroups are dealt to the 8 XCDs in turn.  For prompts, give each XCD one run of consecutive
+        // tokens of one kv head: neighbours read nearly the same keys, so they meet in that XCD's L2.
+        const int total = gridDim.x * gridDim.y, per = total / 8;
+        const int lin = blockIdx.y * gridDim.x + blockIdx.x;
+        const int logical = lin < per * 8 ? (lin % 8) * per + lin / 8 : lin;
+        t = logical % gridDim.x;
+        by = logical / gridDim.x;
+    }
+    const int kvh = by % nkv, ht = by / nkv;
     const int split = blockIdx.z;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
+    // TW > 1: the wavefronts of a workgroup take neighbouring tokens, which visit mostly the same keys at the
+    // same time and so meet in the CU's L1
+    const int wave = TW > 1 ? 0 : threadIdx.x >> 6;
+    if (TW > 1) {
+        t = t * TW + (threadIdx.x >> 6);
+        if (t >= n_tokens) return;
+    }
+    const int lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
     const int G = nh / nkv;
     const int head = kvh * G + ht * 16 + n;            // the head this lane's D column belongs to
     const bool head_ok = ht * 16 + n < G;
@@ -173,13 +192,15 @@ __global__ __launch_bounds__(NW * 64) void attention_mfma_kernel(
     // which chunks of 32 keys are this workgroup's; its wavefronts take them in turn
     const int* sel = nullptr;
     int total_chunks = pos / 32 + 1;
-    int cpb = 1;
+    int cpb = 1, rot = 0;
     if (sel_count) {
         const int cnt = sel_count[(long)t * nkv + kvh];
         if (cnt >= 0) {
             sel = sel_blocks + ((long)t * nkv + kvh) * max_sel;
             cpb = block_size / 32;
             total_chunks = cnt * cpb;
+            // the list's last blocks (the window, which neighbouring tokens share) are visited first
+            rot = max(cnt - last_blocks_first, 0) * cpb;
         }
     }
     const int per_split = (total_chunks + n_splits - 1) / n_splits;
@@ -191,7 +212,12 @@ __global__ __launch_bounds__(NW * 64) void attention_mfma_kernel(
     float m = -INFINITY, l = 0.f;
     const long kv_width = (long)nkv * HD;
 
-    auto chunk_key0 = [&](int c) { return sel ? sel[c / cpb] * block_size + (c % cpb) * 32 : c * 32; };
+    auto chunk_key0 = [&](int c) {
+        if (!sel) return c * 32;
+        c += rot;
+        if (c >= total_chunks) c -= total_chunks;
+        return sel[c / cpb] * block_size + (c % cpb) * 32;
+    };
     // key slot r of tile u is key0 + r + 4*(r/4) + 4u
     auto load_k = [&](int page, int po, abf16x8_t (&kf)[2][KSTEPS]) {
 #pragma unroll
@@ -207,12 +233,26 @@ __global__ __launch_bounds__(NW * 64) void attention_mfma_kernel(
         }
     };
 
-    int c = c0 + wave;
+    // Where the wavefront's chunks lie is looked up for 64 chunks at a time, one chunk a lane (its first key and
+    // its page), and read back lane by lane: the loads of keys and values then wait for no address lookup.
+    int key0_v = 0, page_v = 0, kbase = 0;
+    auto lookup = [&](int kb) {
+        const int cj = c0 + wave + (kb + lane) * NW;
+        int k0 = 0, pg = 0;
+        if (cj < c1) {
+            k0 = chunk_key0(cj);
+            pg = ptab[k0 / pv.page_size];
+        }
+        key0_v = k0;
+        page_v = pg;
+    };
+    int c = c0 + wave, k = 0;
     abf16x8_t kf[2][KSTEPS];
     int key0 = 0, page = 0, po = 0;
     if (c < c1) {
-        key0 = chunk_key0(c);
-        page = ptab[key0 / pv.page_size];
+        lookup(0);
+        key0 = __builtin_amdgcn_readlane(key0_v, 0);
+        page = __builtin_amdgcn_readlane(page_v, 0);
         po = key0 % pv.page_size;
         load_k(page, po, kf);
     }
@@ -220,16 +260,21 @@ __global__ __launch_bounds__(NW * 64) void attention_mfma_kernel(
         // this chunk's values and the next chunk's keys are asked for before this chunk's arithmetic
         abf16x8_t vf[DT];
         {
-            const bf16_t* vp = vtpool + (((long)page * nkv + kvh) * HD + n) * pv.page_size + po + g * 8;
+            const bf16_t* vp = vtpool + value_index(page, po, kvh, n, nkv, HD, pv.page_size) + g * 8;
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const abf16x8_t*)(vp + (long)dt * 16 * pv.page_size);
+            for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const abf16x8_t*)(vp + dt * 16 * 32);
         }
         const int cn = c + NW;
+        ++k;
         abf16x8_t kn[2][KSTEPS];
         int key0n = 0, pagen = 0, pon = 0;
         if (cn < c1) {
-            key0n = chunk_key0(cn);
-            pagen = ptab[key0n / pv.page_size];
+            if (k - kbase == 64) {
+                kbase = k;
+                lookup(kbase);
+            }
+            key0n = __builtin_amdgcn_readlane(key0_v, k - kbase);
+            pagen = __builtin_amdgcn_readlane(page_v, k - kbase);
             pon = key0n % pv.page_size;
             load_k(pagen, pon, kn);
         }
@@ -388,7 +433,7 @@ extern "C" const char* cpmcu_attention_mfma(const void* q, void* out, float* par
                                             const int* page_table, int table_width, int page_size,
                                             const int* positions, const int* tok_slot, const int* sel_blocks,
                                             const int* sel_count, int max_sel, int block_size, int n_splits,
-                                            int waves_per_group, hipStream_t stream) {
+                                            int waves_per_group, int last_blocks_first, hipStream_t stream) {
     CPMCU_REQUIRE(n > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_mfma: bad shape n=%d heads=%d kv_heads=%d", n, nh, nkv);
     CPMCU_REQUIRE(hd == 16 || hd == 32 || hd == 64 || hd == 128,
                   "attention_mfma: head_dim %d has no matrix-core kernel (16, 32, 64, 128 have; the plain kernel takes the rest)", hd);
@@ -401,19 +446,24 @@ extern "C" const char* cpmcu_attention_mfma(const void* q, void* out, float* par
     const int HT = (G + 15) / 16;
     CPMCU_REQUIRE((long)nkv * HT <= 65535, "attention_mfma: too many head tiles");
     PagedView pv{page_table, table_width, page_size};
-    dim3 grid(n, nkv * HT, n_splits);
     const float sl = scale * 1.4426950408889634f;
-    // few tokens (decode steps): 4 wavefronts share a workgroup's keys; many tokens (prompts): one each
+    // few tokens (decode steps): 4 wavefronts share a workgroup's keys; many tokens (prompts): a wavefront a
+    // token, 4 neighbouring tokens a workgroup
     const int nw = waves_per_group > 0 ? waves_per_group : (n <= 256 ? 4 : 1);
     CPMCU_REQUIRE(nw == 1 || nw == 4, "attention_mfma: %d wavefronts a workgroup (1 or 4 are built)", nw);
-#define LAUNCH(HDv, NWv)                                                                                           \
-    attention_mfma_kernel<HDv, NWv><<<grid, NWv * 64, 0, stream>>>(                                               \
+    const int tw = nw == 1 && n_splits == 1 && n >= 64 ? 4 : 1;
+    const int xcd_major = tw > 1 ? 1 : 0;
+    dim3 grid((n + tw - 1) / tw, nkv * HT, n_splits);
+#define LAUNCH(HDv, NWv, TWv)                                                                                      \
+    attention_mfma_kernel<HDv, NWv, TWv><<<grid, NWv * TWv * 64, 0, stream>>>(                                    \
         (const bf16_t*)q, (bf16_t*)out, part_o, (float2*)part_ml, (const bf16_t*)kpool, (const bf16_t*)vtpool, pv, \
-        positions, tok_slot, nh, nkv, sl, sel_blocks, sel_count, max_sel, block_size, n_splits)
-#define BY_NW(HDv)                 \
-    do {                           \
-        if (nw == 4) LAUNCH(HDv, 4); \
-        else LAUNCH(HDv, 1);       \
+        positions, tok_slot, nh, nkv, sl, sel_blocks, sel_count, max_sel, block_size, n_splits, xcd_major, n,      \
+        last_blocks_first)
+#define BY_NW(HDv)                            \
+    do {                                      \
+        if (nw == 4) LAUNCH(HDv, 4, 1);       \
+        else if (tw == 4) LAUNCH(HDv, 1, 4);  \
+        else LAUNCH(HDv, 1, 1);               \
     } while (0)
     if (hd == 16) BY_NW(16);
     else if (hd == 32) BY_NW(32);
@@ -512,9 +562,9 @@ __global__ __launch_bounds__(NW * 64) void attention_prefill_mfma_kernel(
         }
     };
     auto load_v = [&](int page, int po, abf16x8_t (&vf)[DT]) {
-        const bf16_t* vp = vtpool + (((long)page * nkv + kvh) * HD + n) * pv.page_size + po + g * 8;
+        const bf16_t* vp = vtpool + value_index(page, po, kvh, n, nkv, HD, pv.page_size) + g * 8;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const abf16x8_t*)(vp + (long)dt * 16 * pv.page_size);
+        for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const abf16x8_t*)(vp + dt * 16 * 32);
     };
     // one buffer each for keys and values: the next chunk's keys are asked for as soon as the last tile's
     // scores are issued, its values as soon as the last tile's P.V is, so both arrive behind other work

@@ -111,3 +111,12 @@ __device__ inline long paged_row(const PagedView& pv, int slot, int pos) {
     const int page = pv.page_table[(long)slot * pv.table_width + pos / pv.page_size];
     return (long)page * pv.page_size + pos % pv.page_size;
 }
+
+// Values are kept transposed in tiles of value_tile() tokens inside a page,
+// [page][kv head][tile][d][token of the tile], so that attention reads, for one d, the values of consecutive
+// keys as one vector and a chunk of 32 keys is one contiguous piece of memory.
+__host__ __device__ inline int value_tile(int page_size) { return page_size % 32 == 0 ? 32 : page_size; }
+__device__ inline long value_index(long page, int in_page, int kvh, int d, int nkv, int hd, int page_size) {
+    const int vt = value_tile(page_size);
+    return (((page * nkv + kvh) * (page_size / vt) + in_page / vt) * hd + d) * vt + in_page % vt;
+}

@@ -251,7 +251,7 @@ extern "C" const char* cpmcu_silu_mul(const void* gu, void* out, int dtype, int 
 // (a, b) = (x[c], x[c+hd/2]) -> (a cos - b sin, a sin + b cos), cos and sin
 // times `mscale` (reference: src/model/rotary.cuh:7-34; cache rows
 // src/model/attn.cuh:14-21).  inv_freq null: no rotation.  Keys lie [token][kv head][d];
-// values lie transposed inside their page, [page][kv head][d][token of the page].
+// values lie transposed in tiles of tokens inside their page (value_index).
 // ---------------------------------------------------------------------------
 template <typename IT, typename T>
 __global__ void rope_store_kernel(const IT* __restrict__ qkv, long width, int nparts, long part_stride,
@@ -289,12 +289,12 @@ __global__ void rope_store_kernel(const IT* __restrict__ qkv, long width, int np
             dst[c + half] = from_f32<T>(a * sn + b * cs);
         }
     } else {
-        // values are kept transposed inside a page, [page][kv head][d][token of the page], so that
-        // attention reads, for one d, the values of consecutive keys as one vector
+        // values are kept transposed in tiles of tokens inside a page (value_index)
         const long page = kv_row / pv.page_size;
         const int in_page = (int)(kv_row - page * pv.page_size);
-        T* dst = vpool + (page * nkv + (head - nh - nkv)) * (long)hd * pv.page_size + in_page;
-        for (int d = lane; d < hd; d += 64) dst[(long)d * pv.page_size] = from_f32<T>(load(d));
+        const int vt = value_tile(pv.page_size);
+        T* dst = vpool + value_index(page, in_page, head - nh - nkv, 0, nkv, hd, pv.page_size);
+        for (int d = lane; d < hd; d += 64) dst[(long)d * vt] = from_f32<T>(load(d));
     }
 }
 

@@ -202,10 +202,12 @@ def attention_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hd: in
                    positions: torch.Tensor, tok_slot: torch.Tensor, n_splits: int = 1,
                    part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None,
                    sel_blocks: Optional[torch.Tensor] = None, sel_count: Optional[torch.Tensor] = None,
-                   block_size: int = 0, waves_per_group: int = 0):
+                   block_size: int = 0, waves_per_group: int = 0, last_blocks_first: int = 0):
     """bf16 attention on the matrix cores (head_dim 16, 32, 64 or 128; pages and key blocks multiples of 32).
     With n_splits > 1 every token's keys are shared among n_splits wavefronts and merged afterwards;
-    part_o float32 [n, nh, n_splits, hd] and part_ml float32 [n, nh, n_splits, 2] are its scratch."""
+    part_o float32 [n, nh, n_splits, hd] and part_ml float32 [n, nh, n_splits, 2] are its scratch.
+    last_blocks_first: that many blocks at the end of every block list (the window that neighbouring tokens
+    share) are visited before the others; it changes the order of the sums only."""
     _need(q, "attention q", torch.bfloat16, (None, nh * hd))
     n = q.shape[0]
     _need(out, "attention out", torch.bfloat16, (n, nh * hd))
@@ -226,7 +228,7 @@ def attention_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hd: in
         _p(q), _p(out), _p(part_o), _p(part_ml), c_int(n), c_int(nh), c_int(nkv), c_int(hd), c_float(scale),
         _p(kpool), _p(vpool), _p(page_table), c_int(page_table.shape[1]), c_int(page_size), _p(positions),
         _p(tok_slot), _p(sel_blocks), _p(sel_count), c_int(max_sel), c_int(block_size), c_int(n_splits),
-        c_int(waves_per_group), _stream()))
+        c_int(waves_per_group), c_int(last_blocks_first), _stream()))
 
 
 def attention_prefill_tokens_per_wave(nh: int, nkv: int, tiles_per_wave: int = 4) -> int:
@@ -452,7 +454,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, alpha: float = 1
 
 
 def attention(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, ctx,
-              sel_blocks=None, sel_count=None, block_size=0):
+              sel_blocks=None, sel_count=None, block_size=0, window_blocks=0):
     """Attention of the step's queries over the cache, with the kernel that suits the step."""
     if sel_count is None and not ctx.single_token and attention_mfma_ok(q, hd, page_size):
         r, nw = attention_prefill_shape(q.shape[0], nh, nkv, hd)
@@ -475,7 +477,7 @@ def attention(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, c
             part_o = ctx.ws.get("attn.part_o", (n, nh, splits, hd), torch.float32)
             part_ml = ctx.ws.get("attn.part_ml", (n, nh, splits, 2), torch.float32)
         attention_mfma(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, ctx.positions, ctx.tok_slot,
-                       splits, part_o, part_ml, sel_blocks, sel_count, block_size)
+                       splits, part_o, part_ml, sel_blocks, sel_count, block_size, last_blocks_first=window_blocks)
         return
     attention_plain(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, ctx.positions, ctx.tok_slot,
                     sel_blocks, sel_count, block_size)

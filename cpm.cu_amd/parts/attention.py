@@ -72,9 +72,9 @@ class GQAAttention(Mixer):
 
     def attend(self, q, ctx: StepContext, cache: CacheView, sel=None) -> torch.Tensor:
         out = ctx.ws.get("attn.out", tuple(q.shape), q.dtype)
-        sel_blocks, sel_count, bs = sel if sel is not None else (None, None, 0)
+        sel_blocks, sel_count, bs, window_blocks = sel if sel is not None else (None, None, 0, 0)
         ops.attention(q, out, self.nh, self.nkv, self.hd, self.scale, cache.streams["k"], cache.streams["v"],
-                      cache.page_table, cache.page_size, ctx, sel_blocks, sel_count, bs)
+                      cache.page_table, cache.page_size, ctx, sel_blocks, sel_count, bs, window_blocks)
         return out
 
     def forward(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool = True) -> torch.Tensor:
@@ -116,6 +116,6 @@ class InfLLMv2Attention(GQAAttention):
                               cache.page_size, ctx.positions, ctx.tok_slot, self.ks, self.st, self.bs,
                               self.init_blocks, self.topk, self.window_blocks, self.dense_len, ctx.max_pos,
                               sel_blocks, sel_count)
-            sel = (sel_blocks, sel_count, self.bs)
+            sel = (sel_blocks, sel_count, self.bs, self.window_blocks)
         a = self.attend(q, ctx, cache, sel)
         return self.o.forward(a, ctx, "attn.o", out_dtype=torch.float32, partials=True)

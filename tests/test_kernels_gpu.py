@@ -159,6 +159,14 @@ def test_silu_mul(dtype, I):
 
 
 # ---------------------------------------------------------------------------- attention over the paged cache
+def value_tiles(full):
+    """[page tokens, kv heads, d] -> the cache's layout of values, [kv head][tile][d][token of the tile], with
+    tiles of 32 tokens when the page is a multiple of 32 and of the whole page otherwise."""
+    page, nkv, hd = full.shape
+    t = 32 if page % 32 == 0 else page
+    return full.view(page // t, t, nkv, hd).permute(2, 0, 3, 1).contiguous()
+
+
 def paged_setup(lens, nkv, hd, page, dtype, seed=0, scramble=True):
     """Sequences of the given lengths in a paged cache whose pages are handed out in a scrambled order.
     Returns keys/values per sequence (float64) and the pools/page table as the kernels want them."""
@@ -168,7 +176,7 @@ def paged_setup(lens, nkv, hd, page, dtype, seed=0, scramble=True):
     perm = torch.randperm(total, generator=g).tolist() if scramble else list(range(total))
     table = torch.zeros(len(lens), max(n_pages_seq), dtype=torch.int32)
     kpool = torch.zeros(total, page, nkv * hd, dtype=dtype)
-    vpool = torch.zeros(total, page, nkv * hd, dtype=dtype)            # [page][kv head][d][token]: same bytes
+    vpool = torch.zeros(total, page, nkv * hd, dtype=dtype)            # [page][kv head][tile][d][token of the tile]: same bytes
     ks, vs = [], []
     it = iter(perm)
     for s, L in enumerate(lens):
@@ -181,8 +189,9 @@ def paged_setup(lens, nkv, hd, page, dtype, seed=0, scramble=True):
             table[s, pn] = pg
             a, b = pn * page, min((pn + 1) * page, L)
             kpool[pg, :b - a] = k[a:b].reshape(b - a, nkv * hd)
-            vt = vpool[pg].view(nkv, hd, page)
-            vt[:, :, :b - a] = v[a:b].permute(1, 2, 0)
+            full = torch.zeros(page, nkv, hd, dtype=dtype)
+            full[:b - a] = v[a:b]
+            vpool[pg] = value_tiles(full).reshape(page, nkv * hd)
     return ks, vs, kpool.to(DEV), vpool.to(DEV), table.to(DEV)
 
 
@@ -354,6 +363,43 @@ def test_attention_with_block_lists(bs, dtype):
             ops.attention_mfma(q.view(n, -1), out, nh, nkv, hd, hd ** -0.5, kpool, vpool, table, page, pos_t, slot_t,
                                splits, po, pm, sel_blocks.to(DEV), sel_count.to(DEV), bs, waves_per_group=nw)
             assert float((out.double().cpu().view(n, nh, hd) - ref).abs().max()) <= tol
+
+
+@pytest.mark.parametrize("first", [0, 2, 100])
+def test_block_lists_of_a_prompt_chunk_in_any_visiting_order(first):
+    """Steps of many tokens give each wavefront of a workgroup a token of its own and may visit the last blocks
+    of every list first: neither changes which keys count."""
+    from cpmcu_amd import ops
+    nh, nkv, hd, page, bs = 6, 2, 32, 64, 32
+    L = 400
+    ks, vs, kpool, vpool, table = paged_setup([L], nkv, hd, page, torch.bfloat16, seed=11)
+    positions = list(range(329, 400))                 # 71 tokens: the last workgroup is not full
+    n = len(positions)
+    q = rnd(n, nh, hd, seed=4, dtype=torch.bfloat16)
+    max_sel = 7
+    sel_blocks = torch.zeros(n, nkv, max_sel, dtype=torch.int32)
+    sel_count = torch.zeros(n, nkv, dtype=torch.int32)
+    allowed = torch.zeros(n, nkv, L, dtype=torch.bool)
+    g = torch.Generator().manual_seed(5)
+    for t, p in enumerate(positions):
+        for h in range(nkv):
+            if t % 17 == 3 and h == 0:
+                sel_count[t, h] = -1
+                allowed[t, h] = True
+                continue
+            own = p // bs
+            blocks = sorted(set(torch.randperm(own - 1, generator=g)[:4].tolist() + [own - 1, own]))
+            sel_count[t, h] = len(blocks)
+            sel_blocks[t, h, :len(blocks)] = torch.tensor(blocks, dtype=torch.int32)
+            for b in blocks:
+                allowed[t, h, b * bs:(b + 1) * bs] = True
+    ref = attention_reference(q.double().cpu(), ks, vs, positions, [0] * n, nh, hd ** -0.5, allowed)
+    pos_t = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    slot_t = torch.zeros(n, dtype=torch.int32, device=DEV)
+    out = torch.empty(n, nh * hd, dtype=torch.bfloat16, device=DEV)
+    ops.attention_mfma(q.view(n, -1), out, nh, nkv, hd, hd ** -0.5, kpool, vpool, table, page, pos_t, slot_t,
+                       1, None, None, sel_blocks.to(DEV), sel_count.to(DEV), bs, last_blocks_first=first)
+    assert float((out.double().cpu().view(n, nh, hd) - ref).abs().max()) <= 2 ** -7
 
 
 # ---------------------------------------------------------------------------- InfLLM-v2 kernels
