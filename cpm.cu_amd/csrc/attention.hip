@@ -25,9 +25,7 @@ __global__ __launch_bounds__(64) void attention_paged_kernel(
     const T* qrow = q + ((long)t * nh + h) * hd;
     for (int d = lane; d < hd; d += 64) qs[d] = to_f32(qrow[d]);
     __syncthreads();
-    const long kv_stride = (long)nkv * hd;
     const int nd = (hd + 63) / 64;
-    const int vt = value_tile(pv.page_size);
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, l = 0.f;
 
@@ -53,9 +51,10 @@ __global__ __launch_bounds__(64) void attention_paged_kernel(
             float s = -INFINITY;
             if (valid) {
                 row = (int)paged_row(pv, slot, j);
-                const T* kr = kpool + (long)row * kv_stride + (long)g * hd;
+                const int pg = row / pv.page_size;
+                const T* kr = kpool + key_index(pg, row - pg * pv.page_size, g, nkv, hd, pv.page_size);
                 float dot = 0.f;
-                for (int d = 0; d < hd; ++d) dot += qs[d] * to_f32(kr[d]);
+                for (int d = 0; d < hd; ++d) dot += qs[d] * to_f32(kr[key_d_offset(d)]);
                 s = dot * scale;
             }
             const float m_new = fmaxf(m, wave_max(s));
@@ -69,12 +68,11 @@ __global__ __launch_bounds__(64) void attention_paged_kernel(
             for (int jj = 0; jj < cnt; ++jj) {
                 const float pj = __shfl(p, jj, 64);
                 const int rj = __shfl(row, jj, 64);
-                // values are transposed in tiles of tokens inside a page (value_index)
                 const int pg = rj / pv.page_size;
-                const T* vr = vpool + value_index(pg, rj - pg * pv.page_size, g, 0, nkv, hd, pv.page_size);
+                const T* vr = vpool + value_index(pg, rj - pg * pv.page_size, g, nkv, hd, pv.page_size);
                 for (int i = 0; i < nd; ++i) {
                     const int d = lane + 64 * i;
-                    if (d < hd) acc[i] += pj * to_f32(vr[(long)d * vt]);
+                    if (d < hd) acc[i] += pj * to_f32(vr[value_d_offset(d)]);
                 }
             }
         }
@@ -125,8 +123,9 @@ extern "C" const char* cpmcu_attention_plain(const void* q, void* out, int dtype
 //   S^T = K . Q^T      A = 16 keys x head_dim straight from the cache rows,
 //                      B = Q^T held in registers for the whole kernel
 //   P^T = exp2(S^T*c - m) in float, per head (a D column), running max/sum
-//   O^T += V^T . P^T   A = V^T: 16 d x 32 keys, one 16-byte load a lane because
-//                      values are stored transposed in tiles of 32 tokens inside a page
+//   O^T += V^T . P^T   A = V^T: 16 d x 32 keys, one 16-byte load a lane
+// Keys and values lie in their pages in the order of these operands (key_index, value_index), so every
+// operand load of a wavefront is one contiguous KiB.
 // The two key tiles of a chunk take keys {8g..8g+3} and {8g+4..8g+7} of every
 // group of 8 so that a lane's 8 probabilities are 8 consecutive keys, the order
 // the V^T vector has.  With 4 wavefronts a workgroup (decode steps) the wavefronts take
@@ -210,7 +209,6 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_mfma_kernel(
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc[dt] = afloatx4_t{0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, l = 0.f;
-    const long kv_width = (long)nkv * HD;
 
     auto chunk_key0 = [&](int c) {
         if (!sel) return c * 32;
@@ -218,16 +216,15 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_mfma_kernel(
         if (c >= total_chunks) c -= total_chunks;
         return sel[c / cpb] * block_size + (c % cpb) * 32;
     };
-    // key slot r of tile u is key0 + r + 4*(r/4) + 4u
+    // key slot r of tile u is key key0 + r + 4*(r/4) + 4u; a tile lies [d / 8][slot][d % 8] in the page
     auto load_k = [&](int page, int po, abf16x8_t (&kf)[2][KSTEPS]) {
+        const bf16_t* kp = kpool + key_index(page, po, kvh, nkv, HD, pv.page_size) + (g * 16 + n) * 8;
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            const long krow = (long)page * pv.page_size + po + n + 4 * (n >> 2) + 4 * u;
-            const bf16_t* kp = kpool + krow * kv_width + (long)kvh * HD + g * 8;
 #pragma unroll
             for (int ks = 0; ks < KSTEPS; ++ks) {
                 abf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
-                if (ks * 32 + g * 8 < HD) v = *(const abf16x8_t*)(kp + ks * 32);
+                if (ks * 32 + g * 8 < HD) v = *(const abf16x8_t*)(kp + (u * (HD / 8) + ks * 4) * 128);
                 kf[u][ks] = v;
             }
         }
@@ -260,9 +257,9 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_mfma_kernel(
         // this chunk's values and the next chunk's keys are asked for before this chunk's arithmetic
         abf16x8_t vf[DT];
         {
-            const bf16_t* vp = vtpool + value_index(page, po, kvh, n, nkv, HD, pv.page_size) + g * 8;
+            const bf16_t* vp = vtpool + value_index(page, po, kvh, nkv, HD, pv.page_size) + (g * 16 + n) * 8;
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const abf16x8_t*)(vp + dt * 16 * 32);
+            for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const abf16x8_t*)(vp + dt * 512);
         }
         const int cn = c + NW;
         ++k;
@@ -547,24 +544,22 @@ __global__ __launch_bounds__(NW * 64) void attention_prefill_mfma_kernel(
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) acc[r][dt] = afloatx4_t{0.f, 0.f, 0.f, 0.f};
     }
-    const long kv_width = (long)nkv * HD;
     auto load_k = [&](int page, int po, abf16x8_t (&kf)[2][KSTEPS]) {
+        const bf16_t* kp = kpool + key_index(page, po, kvh, nkv, HD, pv.page_size) + (g * 16 + n) * 8;
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            const long krow = (long)page * pv.page_size + po + n + 4 * (n >> 2) + 4 * u;
-            const bf16_t* kp = kpool + krow * kv_width + (long)kvh * HD + g * 8;
 #pragma unroll
             for (int ks = 0; ks < KSTEPS; ++ks) {
                 abf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
-                if (ks * 32 + g * 8 < HD) v = *(const abf16x8_t*)(kp + ks * 32);
+                if (ks * 32 + g * 8 < HD) v = *(const abf16x8_t*)(kp + (u * (HD / 8) + ks * 4) * 128);
                 kf[u][ks] = v;
             }
         }
     };
     auto load_v = [&](int page, int po, abf16x8_t (&vf)[DT]) {
-        const bf16_t* vp = vtpool + value_index(page, po, kvh, n, nkv, HD, pv.page_size) + g * 8;
+        const bf16_t* vp = vtpool + value_index(page, po, kvh, nkv, HD, pv.page_size) + (g * 16 + n) * 8;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const abf16x8_t*)(vp + dt * 16 * 32);
+        for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const abf16x8_t*)(vp + dt * 512);
     };
     // one buffer each for keys and values: the next chunk's keys are asked for as soon as the last tile's
     // scores are issued, its values as soon as the last tile's P.V is, so both arrive behind other work

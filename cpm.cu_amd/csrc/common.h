@@ -112,11 +112,28 @@ __device__ inline long paged_row(const PagedView& pv, int slot, int pos) {
     return (long)page * pv.page_size + pos % pv.page_size;
 }
 
-// Values are kept transposed in tiles of value_tile() tokens inside a page,
-// [page][kv head][tile][d][token of the tile], so that attention reads, for one d, the values of consecutive
-// keys as one vector and a chunk of 32 keys is one contiguous piece of memory.
-__host__ __device__ inline int value_tile(int page_size) { return page_size % 32 == 0 ? 32 : page_size; }
-__device__ inline long value_index(long page, int in_page, int kvh, int d, int nkv, int hd, int page_size) {
-    const int vt = value_tile(page_size);
-    return (((page * nkv + kvh) * (page_size / vt) + in_page / vt) * hd + d) * vt + in_page % vt;
+// Keys and values of a page lie in the order in which the matrix cores take them, so that a wavefront's
+// operand load is one contiguous KiB (loads of 16 bytes a lane that are scattered over rows keep the
+// address unit busy four times as long).  A page holds a multiple of 32 tokens; per kv head and chunk of 32:
+//   keys:   two tiles of 16 key slots (token 8a + 4u + i of the chunk is slot 4a + i of tile u; a lane's 8
+//           scores of a chunk are then 8 consecutive keys), a tile is [d / 8][slot][d % 8]
+//   values: [d / 16][token / 8][d % 16][token % 8], the transposed operand of P.V
+// key_index / value_index give the element of (token of the page, d = 0); *_d_offset adds d.
+__host__ __device__ inline long key_index(long page, int in_page, int kvh, int nkv, int hd, int page_size) {
+    const int c = in_page >> 5, t32 = in_page & 31;
+    const int u = (t32 >> 2) & 1, slot = ((t32 >> 3) << 2) | (t32 & 3);
+    return ((((page * nkv + kvh) * (page_size >> 5) + c) * 2 + u) * (hd >> 3)) * 128 + slot * 8;
 }
+__host__ __device__ inline int key_d_offset(int d) { return (d >> 3) * 128 + (d & 7); }
+__host__ __device__ inline long value_index(long page, int in_page, int kvh, int nkv, int hd, int page_size) {
+    const int c = in_page >> 5, t32 = in_page & 31;
+    return (((page * nkv + kvh) * (page_size >> 5) + c) * (hd >> 4) * 4 + (t32 >> 3)) * 128 + (t32 & 7);
+}
+__host__ __device__ inline int value_d_offset(int d) { return (d >> 4) * 512 + (d & 15) * 8; }
+// Compressed keys (one row for every `stride` tokens, rows_per_page rows a page) lie per kv head as
+// [d / 8][row of the page][d % 8]: neighbouring lanes of a matrix-core operand load, which hold neighbouring
+// rows, then read neighbouring 16 bytes.
+__host__ __device__ inline long ck_index(long page, int row_in_page, int kvh, int nkv, int hd, int rows_per_page) {
+    return ((page * nkv + kvh) * (hd >> 3) * rows_per_page + row_in_page) * 8;
+}
+__host__ __device__ inline int ck_d_offset(int d, int rows_per_page) { return (d >> 3) * rows_per_page * 8 + (d & 7); }

@@ -250,8 +250,8 @@ extern "C" const char* cpmcu_silu_mul(const void* gu, void* out, int dtype, int 
 // to `q_out` (row stride nh*hd).  theta = pos * inv_freq[c];
 // (a, b) = (x[c], x[c+hd/2]) -> (a cos - b sin, a sin + b cos), cos and sin
 // times `mscale` (reference: src/model/rotary.cuh:7-34; cache rows
-// src/model/attn.cuh:14-21).  inv_freq null: no rotation.  Keys lie [token][kv head][d];
-// values lie transposed in tiles of tokens inside their page (value_index).
+// src/model/attn.cuh:14-21).  inv_freq null: no rotation.  In the cache,
+// keys and values lie in their page in the matrix cores' operand order (key_index, value_index).
 // ---------------------------------------------------------------------------
 template <typename IT, typename T>
 __global__ void rope_store_kernel(const IT* __restrict__ qkv, long width, int nparts, long part_stride,
@@ -275,8 +275,16 @@ __global__ void rope_store_kernel(const IT* __restrict__ qkv, long width, int np
     long kv_row = 0;
     if (head >= nh) kv_row = paged_row(pv, tok_slot[t], pos);
     if (head < nh + nkv) {
-        T* dst = head < nh ? q_out + (t * nh + head) * (long)hd
-                           : kpool + kv_row * (long)nkv * hd + (long)(head - nh) * hd;
+        // queries go out as plain rows; keys into their page in the matrix cores' order (key_index)
+        const bool is_q = head < nh;
+        T* dst = q_out;
+        if (is_q) {
+            dst = q_out + (t * nh + head) * (long)hd;
+        } else {
+            const long page = kv_row / pv.page_size;
+            dst = kpool + key_index(page, (int)(kv_row - page * pv.page_size), head - nh, nkv, hd, pv.page_size);
+        }
+        auto at = [&](int d) { return is_q ? d : key_d_offset(d); };
         for (int c = lane; c < half; c += 64) {
             float cs = 1.f, sn = 0.f;
             if (inv_freq) {
@@ -285,16 +293,14 @@ __global__ void rope_store_kernel(const IT* __restrict__ qkv, long width, int np
                 sn = sinf(ang) * mscale;
             }
             const float a = load(c), b = load(c + half);
-            dst[c] = from_f32<T>(a * cs - b * sn);
-            dst[c + half] = from_f32<T>(a * sn + b * cs);
+            dst[at(c)] = from_f32<T>(a * cs - b * sn);
+            dst[at(c + half)] = from_f32<T>(a * sn + b * cs);
         }
     } else {
-        // values are kept transposed in tiles of tokens inside a page (value_index)
+        // values go into their page transposed, in the matrix cores' order (value_index)
         const long page = kv_row / pv.page_size;
-        const int in_page = (int)(kv_row - page * pv.page_size);
-        const int vt = value_tile(pv.page_size);
-        T* dst = vpool + value_index(page, in_page, head - nh - nkv, 0, nkv, hd, pv.page_size);
-        for (int d = lane; d < hd; d += 64) dst[(long)d * vt] = from_f32<T>(load(d));
+        T* dst = vpool + value_index(page, (int)(kv_row - page * pv.page_size), head - nh - nkv, nkv, hd, pv.page_size);
+        for (int d = lane; d < hd; d += 64) dst[value_d_offset(d)] = from_f32<T>(load(d));
     }
 }
 
@@ -307,6 +313,9 @@ extern "C" const char* cpmcu_rope_store(const void* qkv, long row_width, int in_
                   "rope_store: bad shape n=%d heads=%d kv_heads=%d head_dim=%d (head_dim must be even)", n, nh, nkv, hd);
     CPMCU_REQUIRE(!write_kv || (kpool && vpool && page_table && table_width > 0 && page_size > 0),
                   "rope_store: cache pointers missing");
+    CPMCU_REQUIRE(!write_kv || (page_size % 32 == 0 && hd % 16 == 0),
+                  "rope_store: the cache takes pages of a multiple of 32 tokens and head sizes in steps of 16 "
+                  "(page %d, head_dim %d)", page_size, hd);
     CPMCU_REQUIRE(nparts >= 1, "rope_store: nparts=%d", nparts);
     CPMCU_REQUIRE(row_width >= (long)(nh + (write_kv ? 2 * nkv : 0)) * hd,
                   "rope_store: a row of %ld elements cannot hold %d query%s heads of %d", row_width, nh,

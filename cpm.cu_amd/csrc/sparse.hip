@@ -20,8 +20,9 @@
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ void compress_keys_kernel(const T* __restrict__ kpool, T* __restrict__ ckpool, PagedView pv,
-                                     const int* __restrict__ positions, const int* __restrict__ tok_slot, int width,
-                                     int ks, int st) {
+                                     const int* __restrict__ positions, const int* __restrict__ tok_slot, int nkv,
+                                     int hd, int ks, int st) {
+    const int width = nkv * hd;
     const int t = blockIdx.x;
     const int p = positions[t];
     if (p + 1 < ks || (p + 1 - ks) % st != 0) return;
@@ -29,29 +30,37 @@ __global__ void compress_keys_kernel(const T* __restrict__ kpool, T* __restrict_
     const int slot = tok_slot[t];
     const int first = st * j;
     const int page = pv.page_table[(long)slot * pv.table_width + first / pv.page_size];
-    const long ck_row = (long)page * (pv.page_size / st) + (first % pv.page_size) / st;
+    const int rpp = pv.page_size / st;
     for (int e = threadIdx.x; e < width; e += blockDim.x) {
         float s = 0.f;
-        for (int r = 0; r < ks; ++r) s += to_f32(kpool[paged_row(pv, slot, first + r) * width + e]);
-        ckpool[ck_row * width + e] = from_f32<T>(s / (float)ks);
+        const int kvh = e / hd, d = e - kvh * hd;
+        for (int r = 0; r < ks; ++r) {
+            const long row = paged_row(pv, slot, first + r);
+            const long pg = row / pv.page_size;
+            s += to_f32(kpool[key_index(pg, (int)(row - pg * pv.page_size), kvh, nkv, hd, pv.page_size) + key_d_offset(d)]);
+        }
+        ckpool[ck_index(page, (first % pv.page_size) / st, kvh, nkv, hd, rpp) + ck_d_offset(d, rpp)] = from_f32<T>(s / (float)ks);
     }
 }
 
-extern "C" const char* cpmcu_compress_keys(const void* kpool, void* ckpool, int dtype, int n, int width,
+extern "C" const char* cpmcu_compress_keys(const void* kpool, void* ckpool, int dtype, int n, int nkv, int hd,
                                            const int* page_table, int table_width, int page_size,
                                            const int* positions, const int* tok_slot, int ks, int st,
                                            hipStream_t stream) {
-    CPMCU_REQUIRE(n > 0 && width > 0, "compress_keys: empty shape");
+    CPMCU_REQUIRE(n > 0 && nkv > 0 && hd > 0, "compress_keys: empty shape");
+    CPMCU_REQUIRE(page_size % 32 == 0 && hd % 16 == 0,
+                  "compress_keys: the cache takes pages of a multiple of 32 tokens and head sizes in steps of 16 "
+                  "(page %d, head_dim %d)", page_size, hd);
     CPMCU_REQUIRE(st > 0 && ks >= st && page_size % st == 0,
                   "compress_keys: kernel_stride %d must divide the cache page of %d tokens (kernel_size %d)", st,
                   page_size, ks);
     PagedView pv{page_table, table_width, page_size};
     if (dtype == CPMCU_F32)
         compress_keys_kernel<float><<<n, 128, 0, stream>>>((const float*)kpool, (float*)ckpool, pv, positions,
-                                                           tok_slot, width, ks, st);
+                                                           tok_slot, nkv, hd, ks, st);
     else if (dtype == CPMCU_BF16)
         compress_keys_kernel<bf16_t><<<n, 128, 0, stream>>>((const bf16_t*)kpool, (bf16_t*)ckpool, pv, positions,
-                                                            tok_slot, width, ks, st);
+                                                            tok_slot, nkv, hd, ks, st);
     else
         CPMCU_FAIL("compress_keys: unknown dtype %d", dtype);
     CPMCU_LAUNCH_CHECK("compress_keys");
@@ -95,7 +104,6 @@ __global__ __launch_bounds__(256) void sparse_select_kernel(const T* __restrict_
     const int q_block = p / sp.bs;
     const int n_cand = max(q_block - sp.window_blocks + 1, 0);
     const int rows_per_page = pv.page_size / sp.st;
-    const long width = (long)sp.nkv * sp.hd;
 
     for (int j = tid; j < n_vis; j += blockDim.x) score[j] = 0.f;
     for (int hh = 0; hh < G; ++hh) {
@@ -107,9 +115,9 @@ __global__ __launch_bounds__(256) void sparse_select_kernel(const T* __restrict_
         for (int j = tid; j < n_vis; j += blockDim.x) {
             const int first = sp.st * j;
             const int page = pv.page_table[(long)slot * pv.table_width + first / pv.page_size];
-            const T* ck = ckpool + ((long)page * rows_per_page + (first % pv.page_size) / sp.st) * width + (long)g * sp.hd;
+            const T* ck = ckpool + ck_index(page, (first % pv.page_size) / sp.st, g, sp.nkv, sp.hd, rows_per_page);
             float dot = 0.f;
-            for (int d = 0; d < sp.hd; ++d) dot += qs[d] * to_f32(ck[d]);
+            for (int d = 0; d < sp.hd; ++d) dot += qs[d] * to_f32(ck[ck_d_offset(d, rows_per_page)]);
             const float s = dot * sp.scale;
             tmp[j] = s;
             mx = fmaxf(mx, s);
@@ -177,6 +185,7 @@ extern "C" const char* cpmcu_sparse_select(const void* q, const void* ckpool, in
                                            int max_pos, int* sel_blocks, int* sel_count, int max_sel,
                                            int force_plain, hipStream_t stream) {
     CPMCU_REQUIRE(n > 0 && nh > 0 && nkv > 0 && hd > 0 && nh % nkv == 0, "sparse_select: bad shape");
+    CPMCU_REQUIRE(hd % 8 == 0, "sparse_select: compressed keys lie in pieces of 8 elements; head_dim %d is no multiple", hd);
     CPMCU_REQUIRE(st > 0 && ks >= st && bs % st == 0 && page_size % st == 0,
                   "sparse_select: kernel_stride %d must divide block_size %d and the cache page of %d tokens", st, bs,
                   page_size);
@@ -272,7 +281,6 @@ __global__ __launch_bounds__(NW * 64) void sparse_select_mfma_kernel(
     const int q_block = p / sp.bs;
     const int n_cand = max(q_block - sp.window_blocks + 1, 0);
     const int rows_per_page = pv.page_size / sp.st;
-    const long width = (long)sp.nkv * HD;
     const float scale_log2e = sp.scale * 1.4426950408889634f;
     const int n_tiles = (n_vis + 15) / 16;
 
@@ -295,13 +303,13 @@ __global__ __launch_bounds__(NW * 64) void sparse_select_mfma_kernel(
             const int j = min(tile * 16 + n, n_vis - 1);
             const int first = sp.st * j;
             const int page = ptab[first / pv.page_size];
-            const bf16_t* ck = ckpool + ((long)page * rows_per_page + (first % pv.page_size) / sp.st) * width +
-                               (long)kvh * HD + g * 8;
+            const bf16_t* ck = ckpool + ck_index(page, (first % pv.page_size) / sp.st, kvh, sp.nkv, HD, rows_per_page) +
+                               g * rows_per_page * 8;
             sfloatx4_t st = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ks = 0; ks < KSTEPS; ++ks) {
                 sbf16x8_t b = {0, 0, 0, 0, 0, 0, 0, 0};
-                if (ks * 32 + g * 8 < HD) b = *(const sbf16x8_t*)(ck + ks * 32);
+                if (ks * 32 + g * 8 < HD) b = *(const sbf16x8_t*)(ck + ks * 4 * rows_per_page * 8);
                 st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ks], b, st, 0, 0, 0);
             }
             return st;                      // st[i]: head 4g+i (of this head tile) x key tile*16+n

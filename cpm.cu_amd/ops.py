@@ -293,11 +293,14 @@ def attention_splits(n_tokens: int, nkv: int, group: int, max_keys: int) -> int:
     return max(1, min(256 // max(groups, 1), max_keys // 512, 64))
 
 
-def compress_keys(kpool: torch.Tensor, ckpool: torch.Tensor, page_table: torch.Tensor, page_size: int,
+def compress_keys(kpool: torch.Tensor, ckpool: torch.Tensor, nkv: int, page_table: torch.Tensor, page_size: int,
                   positions: torch.Tensor, tok_slot: torch.Tensor, kernel_size: int, kernel_stride: int):
-    """Write the compressed keys (means of kernel_size keys, every kernel_stride) that the step's tokens complete."""
+    """Write the compressed keys (means of kernel_size keys, every kernel_stride) that the step's tokens complete.
+    The keys lie in their pages as rope_store writes them; a compressed key is a plain row [kv head][d]."""
     _need(kpool, "compress key pool", shape=(None, page_size, None))
     width = kpool.shape[2]
+    if nkv <= 0 or width % nkv:
+        raise KernelError(f"compress_keys: rows of {width} elements do not hold {nkv} kv heads")
     if kernel_stride <= 0 or page_size % kernel_stride:
         raise KernelError(f"compress_keys: kernel_stride {kernel_stride} must divide the cache page of {page_size} tokens")
     _need(ckpool, "compressed key pool", kpool.dtype, (kpool.shape[0], page_size // kernel_stride, width))
@@ -305,8 +308,8 @@ def compress_keys(kpool: torch.Tensor, ckpool: torch.Tensor, page_table: torch.T
     _need(positions, "compress positions", torch.int32, (None,))
     n = positions.shape[0]
     _need(tok_slot, "compress token slots", torch.int32, (n,))
-    _check(_fn("sparse", "cpmcu_compress_keys")(_p(kpool), _p(ckpool), c_int(_code(kpool)), c_int(n), c_int(width),
-                                                _p(page_table), c_int(page_table.shape[1]), c_int(page_size),
+    _check(_fn("sparse", "cpmcu_compress_keys")(_p(kpool), _p(ckpool), c_int(_code(kpool)), c_int(n), c_int(nkv),
+                                                c_int(width // nkv), _p(page_table), c_int(page_table.shape[1]), c_int(page_size),
                                                 _p(positions), _p(tok_slot), c_int(kernel_size), c_int(kernel_stride),
                                                 _stream()))
 

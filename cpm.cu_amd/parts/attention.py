@@ -104,7 +104,7 @@ class InfLLMv2Attention(GQAAttention):
     def forward(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool = True) -> torch.Tensor:
         q = self.project_and_store(h, ctx, cache, writes_cache)
         if writes_cache:
-            ops.compress_keys(cache.streams["k"], cache.streams["ck"], cache.page_table, cache.page_size,
+            ops.compress_keys(cache.streams["k"], cache.streams["ck"], self.nkv, cache.page_table, cache.page_size,
                               ctx.positions, ctx.tok_slot, self.ks, self.st)
         sel = None
         if ctx.max_pos + 1 > self.dense_len:

@@ -159,12 +159,29 @@ def test_silu_mul(dtype, I):
 
 
 # ---------------------------------------------------------------------------- attention over the paged cache
-def value_tiles(full):
-    """[page tokens, kv heads, d] -> the cache's layout of values, [kv head][tile][d][token of the tile], with
-    tiles of 32 tokens when the page is a multiple of 32 and of the whole page otherwise."""
+def key_tiles(full):
+    """[page tokens, kv heads, d] -> the cache's layout of keys: per kv head and chunk of 32 tokens two tiles of
+    16 key slots (token 8a + 4u + i of the chunk is slot 4a + i of tile u), a tile [d / 8][slot][d % 8]."""
     page, nkv, hd = full.shape
-    t = 32 if page % 32 == 0 else page
-    return full.view(page // t, t, nkv, hd).permute(2, 0, 3, 1).contiguous()
+    x = full.view(page // 32, 4, 2, 4, nkv, hd // 8, 8)          # chunk, a, u, i, kv head, d / 8, d % 8
+    return x.permute(4, 0, 2, 5, 1, 3, 6).contiguous()            # kv head, chunk, u, d / 8, a, i, d % 8
+
+
+def key_elements(in_page, kvh, nkv, hd, page):
+    """Where the hd elements of one key lie inside its page (flat indices), by the same rule as key_tiles."""
+    c, t32 = divmod(in_page, 32)
+    a_, r = divmod(t32, 8)
+    u, i = divmod(r, 4)
+    d = torch.arange(hd)
+    return ((((kvh * (page // 32) + c) * 2 + u) * (hd // 8) + d // 8) * 16 + a_ * 4 + i) * 8 + d % 8
+
+
+def value_tiles(full):
+    """[page tokens, kv heads, d] -> the cache's layout of values: per kv head and chunk of 32 tokens
+    [d / 16][token / 8][d % 16][token % 8]."""
+    page, nkv, hd = full.shape
+    x = full.view(page // 32, 4, 8, nkv, hd // 16, 16)           # chunk, token / 8, token % 8, kv head, d / 16, d % 16
+    return x.permute(3, 0, 4, 1, 5, 2).contiguous()
 
 
 def paged_setup(lens, nkv, hd, page, dtype, seed=0, scramble=True):
@@ -176,7 +193,7 @@ def paged_setup(lens, nkv, hd, page, dtype, seed=0, scramble=True):
     perm = torch.randperm(total, generator=g).tolist() if scramble else list(range(total))
     table = torch.zeros(len(lens), max(n_pages_seq), dtype=torch.int32)
     kpool = torch.zeros(total, page, nkv * hd, dtype=dtype)
-    vpool = torch.zeros(total, page, nkv * hd, dtype=dtype)            # [page][kv head][tile][d][token of the tile]: same bytes
+    vpool = torch.zeros(total, page, nkv * hd, dtype=dtype)            # both in the matrix cores' operand order: same bytes
     ks, vs = [], []
     it = iter(perm)
     for s, L in enumerate(lens):
@@ -188,7 +205,9 @@ def paged_setup(lens, nkv, hd, page, dtype, seed=0, scramble=True):
             pg = next(it)
             table[s, pn] = pg
             a, b = pn * page, min((pn + 1) * page, L)
-            kpool[pg, :b - a] = k[a:b].reshape(b - a, nkv * hd)
+            full = torch.zeros(page, nkv, hd, dtype=dtype)
+            full[:b - a] = k[a:b]
+            kpool[pg] = key_tiles(full).reshape(page, nkv * hd)
             full = torch.zeros(page, nkv, hd, dtype=dtype)
             full[:b - a] = v[a:b]
             vpool[pg] = value_tiles(full).reshape(page, nkv * hd)
@@ -297,9 +316,12 @@ def test_attention_finds_one_far_key_among_hundreds(dtype):
         q = torch.zeros(1, nh, hd, dtype=torch.float64)
         q[0, :, 5] = 40.0
         pg, off = int(table[0, far // page]), far % page
-        saved = kpool[pg, off].clone()
-        kpool[pg, off] = 0
-        kpool[pg, off, 5] = 40.0
+        where = key_elements(off, 0, nkv, hd, page).to(DEV)
+        flat = kpool[pg].view(-1)
+        saved = flat[where].clone()
+        one = torch.zeros(hd, dtype=dtype, device=DEV)
+        one[5] = 40.0
+        flat[where] = one
         pos_t = torch.tensor([L - 1], dtype=torch.int32, device=DEV)
         slot_t = torch.zeros(1, dtype=torch.int32, device=DEV)
         qd = q.to(dtype).to(DEV).view(1, -1)
@@ -316,7 +338,7 @@ def test_attention_finds_one_far_key_among_hundreds(dtype):
                 outs.append(out.clone())
         for o in outs:
             assert float((o.double().cpu().view(nh, hd) - vs[0][far, 0]).abs().max()) < 1e-2, far
-        kpool[pg, off] = saved
+        flat[where] = saved
 
 
 @pytest.mark.parametrize("bs", [16, 32, 64])
@@ -416,11 +438,13 @@ def test_compressed_keys_are_means_written_when_their_last_key_arrives(ks, st, d
     for a0, b0, a1, b1 in ((0, 100, 0, 20), (100, 150, 20, 37)):
         positions = list(range(a0, b0)) + list(range(a1, b1))
         slots = [0] * (b0 - a0) + [1] * (b1 - a1)
-        ops.compress_keys(kpool, ck, table, page, torch.tensor(positions, dtype=torch.int32, device=DEV),
+        ops.compress_keys(kpool, ck, nkv, table, page, torch.tensor(positions, dtype=torch.int32, device=DEV),
                           torch.tensor(slots, dtype=torch.int32, device=DEV), ks, st)
     for s, L in enumerate(lens):
         ref = F.avg_pool1d(kseq[s].reshape(L, -1).T[None], ks, st)[0].T        # [n_ck, nkv*hd]
-        got = torch.stack([ck[int(table[s, (st * j) // page]), ((st * j) % page) // st] for j in range(ref.shape[0])])
+        # a page of compressed keys lies [kv head][d / 8][row][d % 8]
+        got = torch.stack([ck[int(table[s, (st * j) // page])].view(nkv, hd // 8, page // st, 8)
+                           [:, :, ((st * j) % page) // st].reshape(nkv * hd) for j in range(ref.shape[0])])
         tol = 1e-6 if dtype == torch.float32 else 2 ** -8
         assert float((got.double().cpu() - ref).abs().max()) <= tol * float(ref.abs().max() + 1)
 
@@ -438,7 +462,7 @@ def test_block_selection_equals_the_plain_selection(dtype, nh, nkv, hd, ks, st, 
     kseq, vs, kpool, vpool, table = paged_setup([L], nkv, hd, page, dtype, seed=bs + topk)
     ck = torch.zeros(kpool.shape[0], page // st, nkv * hd, dtype=dtype, device=DEV)
     allpos = torch.arange(L, dtype=torch.int32, device=DEV)
-    ops.compress_keys(kpool, ck, table, page, allpos, torch.zeros(L, dtype=torch.int32, device=DEV), ks, st)
+    ops.compress_keys(kpool, ck, nkv, table, page, allpos, torch.zeros(L, dtype=torch.int32, device=DEV), ks, st)
     sc = {"kernel_size": ks, "kernel_stride": st, "block_size": bs, "init_blocks": init, "topk": topk,
           "window_size": window, "dense_len": dense_len}
     positions = sorted(set([0, 1, ks - 1, ks, ks + 1, bs - 1, bs, bs + 1, window - 1, window, window + bs - 1, window + bs,
@@ -476,7 +500,7 @@ def test_block_selection_ties_and_forced_blocks():
     kpool = torch.ones(5, page, nkv * hd, device=DEV)
     table = torch.tensor([[3, 1, 4, 0]], dtype=torch.int32, device=DEV)
     ck = torch.zeros(5, page // st, nkv * hd, device=DEV)
-    ops.compress_keys(kpool, ck, table, page, torch.arange(L, dtype=torch.int32, device=DEV),
+    ops.compress_keys(kpool, ck, nkv, table, page, torch.arange(L, dtype=torch.int32, device=DEV),
                       torch.zeros(L, dtype=torch.int32, device=DEV), ks, st)
     q = torch.ones(1, nh * hd, device=DEV)
     for dtype in (torch.float32, torch.bfloat16):
