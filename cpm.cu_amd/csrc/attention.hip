@@ -51,8 +51,7 @@ __global__ __launch_bounds__(64) void attention_paged_kernel(
             float s = -INFINITY;
             if (valid) {
                 row = (int)paged_row(pv, slot, j);
-                const int pg = row / pv.page_size;
-                const T* kr = kpool + key_index(pg, row - pg * pv.page_size, g, nkv, hd, pv.page_size);
+                const T* kr = kpool + key_index(row, g, nkv, hd);
                 float dot = 0.f;
                 for (int d = 0; d < hd; ++d) dot += qs[d] * to_f32(kr[key_d_offset(d)]);
                 s = dot * scale;
@@ -68,8 +67,7 @@ __global__ __launch_bounds__(64) void attention_paged_kernel(
             for (int jj = 0; jj < cnt; ++jj) {
                 const float pj = __shfl(p, jj, 64);
                 const int rj = __shfl(row, jj, 64);
-                const int pg = rj / pv.page_size;
-                const T* vr = vpool + value_index(pg, rj - pg * pv.page_size, g, nkv, hd, pv.page_size);
+                const T* vr = vpool + value_index(rj, g, nkv, hd);
                 for (int i = 0; i < nd; ++i) {
                     const int d = lane + 64 * i;
                     if (d < hd) acc[i] += pj * to_f32(vr[value_d_offset(d)]);
@@ -177,7 +175,6 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_mfma_kernel(
     const int head = kvh * G + ht * 16 + n;            // the head this lane's D column belongs to
     const bool head_ok = ht * 16 + n < G;
     const int pos = positions[t], slot = tok_slot[t];
-    const int* ptab = pv.page_table + (long)slot * pv.table_width;
 
     abf16x8_t qf[KSTEPS];
 #pragma unroll
@@ -216,9 +213,28 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_mfma_kernel(
         if (c >= total_chunks) c -= total_chunks;
         return sel[c / cpb] * block_size + (c % cpb) * 32;
     };
-    // key slot r of tile u is key key0 + r + 4*(r/4) + 4u; a tile lies [d / 8][slot][d % 8] in the page
-    auto load_k = [&](int page, int po, abf16x8_t (&kf)[2][KSTEPS]) {
-        const bf16_t* kp = kpool + key_index(page, po, kvh, nkv, HD, pv.page_size) + (g * 16 + n) * 8;
+    // Where the wavefront's chunks lie is looked up for 64 chunks at a time, one chunk a lane (its first key and
+    // its physical chunk of the pool), and read back lane by lane: the loads of keys and values then wait for
+    // no address lookup, and the loop holds no division.
+    int key0_v = 0, pchunk_v = 0, kbase = 0;
+    auto lookup = [&](int kb) {
+        const int cj = c0 + wave + (kb + lane) * NW;
+        int k0 = 0, pc = 0;
+        if (cj < c1) {
+            k0 = chunk_key0(cj);
+            pc = (int)(paged_row(pv, slot, k0) >> 5);
+        }
+        key0_v = k0;
+        pchunk_v = pc;
+    };
+    const long chunk_elems = 32L * HD;
+    const int lane_off = (g * 16 + n) * 8;
+    const bf16_t* kbase_p = kpool + (long)kvh * chunk_elems + lane_off;
+    const bf16_t* vbase_p = vtpool + (long)kvh * chunk_elems + lane_off;
+    const long chunk_stride = (long)nkv * chunk_elems;
+    // key slot r of tile u is key key0 + r + 4*(r/4) + 4u; a tile lies [d / 8][slot][d % 8]
+    auto load_k = [&](int pchunk, abf16x8_t (&kf)[2][KSTEPS]) {
+        const bf16_t* kp = kbase_p + pchunk * chunk_stride;
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
 #pragma unroll
@@ -229,54 +245,39 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_mfma_kernel(
             }
         }
     };
-
-    // Where the wavefront's chunks lie is looked up for 64 chunks at a time, one chunk a lane (its first key and
-    // its page), and read back lane by lane: the loads of keys and values then wait for no address lookup.
-    int key0_v = 0, page_v = 0, kbase = 0;
-    auto lookup = [&](int kb) {
-        const int cj = c0 + wave + (kb + lane) * NW;
-        int k0 = 0, pg = 0;
-        if (cj < c1) {
-            k0 = chunk_key0(cj);
-            pg = ptab[k0 / pv.page_size];
-        }
-        key0_v = k0;
-        page_v = pg;
+    auto load_v = [&](int pchunk, abf16x8_t (&vf)[DT]) {
+        const bf16_t* vp = vbase_p + pchunk * chunk_stride;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const abf16x8_t*)(vp + dt * 512);
     };
+    // One buffer each for keys and values: the next chunk's keys are asked for as soon as this chunk's scores
+    // are issued, its values as soon as this chunk's P.V is, so both arrive behind the other half of the work
+    // (and behind the other wavefronts of the SIMD).
     int c = c0 + wave, k = 0;
-    abf16x8_t kf[2][KSTEPS];
-    int key0 = 0, page = 0, po = 0;
+    abf16x8_t kf[2][KSTEPS], vf[DT];
+    int key0 = 0;
     if (c < c1) {
         lookup(0);
         key0 = __builtin_amdgcn_readlane(key0_v, 0);
-        page = __builtin_amdgcn_readlane(page_v, 0);
-        po = key0 % pv.page_size;
-        load_k(page, po, kf);
+        const int pchunk = __builtin_amdgcn_readlane(pchunk_v, 0);
+        load_k(pchunk, kf);
+        load_v(pchunk, vf);
     }
     while (c < c1) {
-        // this chunk's values and the next chunk's keys are asked for before this chunk's arithmetic
-        abf16x8_t vf[DT];
-        {
-            const bf16_t* vp = vtpool + value_index(page, po, kvh, nkv, HD, pv.page_size) + (g * 16 + n) * 8;
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const abf16x8_t*)(vp + dt * 512);
-        }
         const int cn = c + NW;
         ++k;
-        abf16x8_t kn[2][KSTEPS];
-        int key0n = 0, pagen = 0, pon = 0;
+        int key0n = 0, pchunkn = 0;
         if (cn < c1) {
             if (k - kbase == 64) {
                 kbase = k;
                 lookup(kbase);
             }
             key0n = __builtin_amdgcn_readlane(key0_v, k - kbase);
-            pagen = __builtin_amdgcn_readlane(page_v, k - kbase);
-            pon = key0n % pv.page_size;
-            load_k(pagen, pon, kn);
+            pchunkn = __builtin_amdgcn_readlane(pchunk_v, k - kbase);
         }
-        if (key0 <= pos) {
-            afloatx4_t st[2];
+        const bool live = key0 <= pos;           // a listed block may reach beyond the token's own position
+        afloatx4_t st[2];
+        if (live) {
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
                 st[u] = afloatx4_t{0.f, 0.f, 0.f, 0.f};
@@ -284,27 +285,32 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_mfma_kernel(
                 for (int ks = 0; ks < KSTEPS; ++ks)
                     st[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][ks], qf[ks], st[u], 0, 0, 0);
             }
-            // lane (head n, g): st[u][i] is key key0 + 8g + 4u + i
+        }
+        if (cn < c1) load_k(pchunkn, kf);
+        if (live) {
+            // lane (head n, g): st[u][i] is key key0 + 8g + 4u + i; only the chunk that holds the token's own
+            // position needs the causal mask
             float sc[8];
-            float mx = -INFINITY;
 #pragma unroll
             for (int u = 0; u < 2; ++u)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int key = key0 + 8 * g + 4 * u + i;
-                    const float v = key <= pos ? st[u][i] * scale_log2e : -INFINITY;
-                    sc[u * 4 + i] = v;
-                    mx = fmaxf(mx, v);
-                }
+                for (int i = 0; i < 4; ++i) sc[u * 4 + i] = st[u][i];
+            if (key0 + 31 > pos) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (key0 + 8 * g + j > pos) sc[j] = -INFINITY;
+            }
+            float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
             mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            const float m_new = fmaxf(m, mx);
+            // m is kept in units of the exponent: scores times scale*log2(e)
+            const float m_new = fmaxf(m, mx * scale_log2e);
             const float corr = fast_exp2(m - m_new);
             float rs = 0.f;
             abf16x8_t pb;
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                const float p = fast_exp2(sc[j] - m_new);
+                const float p = fast_exp2(__builtin_fmaf(sc[j], scale_log2e, -m_new));
                 rs += p;
                 pb[j] = (__bf16)p;
             }
@@ -324,14 +330,9 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_mfma_kernel(
             for (int dt = 0; dt < DT; ++dt)
                 acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pb, acc[dt], 0, 0, 0);
         }
+        if (cn < c1) load_v(pchunkn, vf);
         c = cn;
         key0 = key0n;
-        page = pagen;
-        po = pon;
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-#pragma unroll
-            for (int ks = 0; ks < KSTEPS; ++ks) kf[u][ks] = kn[u][ks];
     }
 
     if (NW > 1) {
@@ -545,7 +546,7 @@ __global__ __launch_bounds__(NW * 64) void attention_prefill_mfma_kernel(
         for (int dt = 0; dt < DT; ++dt) acc[r][dt] = afloatx4_t{0.f, 0.f, 0.f, 0.f};
     }
     auto load_k = [&](int page, int po, abf16x8_t (&kf)[2][KSTEPS]) {
-        const bf16_t* kp = kpool + key_index(page, po, kvh, nkv, HD, pv.page_size) + (g * 16 + n) * 8;
+        const bf16_t* kp = kpool + chunk_base((long)page * pv.page_size + po, kvh, nkv, HD) + (g * 16 + n) * 8;
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
 #pragma unroll
@@ -557,7 +558,7 @@ __global__ __launch_bounds__(NW * 64) void attention_prefill_mfma_kernel(
         }
     };
     auto load_v = [&](int page, int po, abf16x8_t (&vf)[DT]) {
-        const bf16_t* vp = vtpool + value_index(page, po, kvh, nkv, HD, pv.page_size) + (g * 16 + n) * 8;
+        const bf16_t* vp = vtpool + chunk_base((long)page * pv.page_size + po, kvh, nkv, HD) + (g * 16 + n) * 8;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const abf16x8_t*)(vp + dt * 512);
     };

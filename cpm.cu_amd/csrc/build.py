@@ -40,6 +40,18 @@ HIPCC_FLAGS = [
 ]
 
 
+# extra flags of single libraries
+#   attention: matrix-core results stay in ordinary vector registers; with the accumulation registers the
+#   compiler moves the running output there and back around every rescale
+MODULE_FLAGS: Dict[str, List[str]] = {
+    "attention": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+}
+
+
+def _flags(module: str) -> List[str]:
+    return HIPCC_FLAGS + MODULE_FLAGS.get(module, [])
+
+
 class BuildError(RuntimeError):
     pass
 
@@ -53,7 +65,7 @@ def _hipcc() -> str:
 
 def _digest(module: str) -> str:
     h = hashlib.sha256()
-    h.update(" ".join(HIPCC_FLAGS).encode())
+    h.update(" ".join(_flags(module)).encode())
     for name in HEADERS + MODULES[module]:
         with open(os.path.join(HERE, name), "rb") as f:
             h.update(name.encode())
@@ -87,7 +99,7 @@ def build(module: str, verbose: bool = True) -> str:
     """Compile one library now, whether or not a current one exists."""
     out = lib_path(module)
     tmp = f"{out}.{os.getpid()}.tmp"
-    cmd = [_hipcc()] + HIPCC_FLAGS + ["-I", HERE, "-o", tmp] + [os.path.join(HERE, s) for s in MODULES[module]]
+    cmd = [_hipcc()] + _flags(module) + ["-I", HERE, "-o", tmp] + [os.path.join(HERE, s) for s in MODULES[module]]
     t0 = time.time()
     if verbose:
         print(f"[cpmcu_amd] compiling {module} ({', '.join(MODULES[module])}) for {ARCH} ...", file=sys.stderr, flush=True)

@@ -114,22 +114,27 @@ __device__ inline long paged_row(const PagedView& pv, int slot, int pos) {
 
 // Keys and values of a page lie in the order in which the matrix cores take them, so that a wavefront's
 // operand load is one contiguous KiB (loads of 16 bytes a lane that are scattered over rows keep the
-// address unit busy four times as long).  A page holds a multiple of 32 tokens; per kv head and chunk of 32:
+// address unit busy four times as long).  A page holds a multiple of 32 tokens; per chunk of 32 tokens
+// and kv head (the chunk comes first: physical chunk number = physical token row / 32):
 //   keys:   two tiles of 16 key slots (token 8a + 4u + i of the chunk is slot 4a + i of tile u; a lane's 8
 //           scores of a chunk are then 8 consecutive keys), a tile is [d / 8][slot][d % 8]
 //   values: [d / 16][token / 8][d % 16][token % 8], the transposed operand of P.V
-// key_index / value_index give the element of (token of the page, d = 0); *_d_offset adds d.
-__host__ __device__ inline long key_index(long page, int in_page, int kvh, int nkv, int hd, int page_size) {
-    const int c = in_page >> 5, t32 = in_page & 31;
+// key_index / value_index give the element of (token row, d = 0); *_d_offset adds d.
+__host__ __device__ inline long chunk_base(long row, int kvh, int nkv, int hd) {
+    return ((row >> 5) * nkv + kvh) * (32L * hd);
+}
+__host__ __device__ inline long key_index(long row, int kvh, int nkv, int hd) {
+    const int t32 = (int)(row & 31);
     const int u = (t32 >> 2) & 1, slot = ((t32 >> 3) << 2) | (t32 & 3);
-    return ((((page * nkv + kvh) * (page_size >> 5) + c) * 2 + u) * (hd >> 3)) * 128 + slot * 8;
+    return chunk_base(row, kvh, nkv, hd) + (u * (hd >> 3) * 16 + slot) * 8;
 }
 __host__ __device__ inline int key_d_offset(int d) { return (d >> 3) * 128 + (d & 7); }
-__host__ __device__ inline long value_index(long page, int in_page, int kvh, int nkv, int hd, int page_size) {
-    const int c = in_page >> 5, t32 = in_page & 31;
-    return (((page * nkv + kvh) * (page_size >> 5) + c) * (hd >> 4) * 4 + (t32 >> 3)) * 128 + (t32 & 7);
+__host__ __device__ inline long value_index(long row, int kvh, int nkv, int hd) {
+    const int t32 = (int)(row & 31);
+    return chunk_base(row, kvh, nkv, hd) + (t32 >> 3) * 128 + (t32 & 7);
 }
 __host__ __device__ inline int value_d_offset(int d) { return (d >> 4) * 512 + (d & 15) * 8; }
+
 // Compressed keys (one row for every `stride` tokens, rows_per_page rows a page) lie per kv head as
 // [d / 8][row of the page][d % 8]: neighbouring lanes of a matrix-core operand load, which hold neighbouring
 // rows, then read neighbouring 16 bytes.

@@ -281,8 +281,7 @@ __global__ void rope_store_kernel(const IT* __restrict__ qkv, long width, int np
         if (is_q) {
             dst = q_out + (t * nh + head) * (long)hd;
         } else {
-            const long page = kv_row / pv.page_size;
-            dst = kpool + key_index(page, (int)(kv_row - page * pv.page_size), head - nh, nkv, hd, pv.page_size);
+            dst = kpool + key_index(kv_row, head - nh, nkv, hd);
         }
         auto at = [&](int d) { return is_q ? d : key_d_offset(d); };
         for (int c = lane; c < half; c += 64) {
@@ -298,8 +297,7 @@ __global__ void rope_store_kernel(const IT* __restrict__ qkv, long width, int np
         }
     } else {
         // values go into their page transposed, in the matrix cores' order (value_index)
-        const long page = kv_row / pv.page_size;
-        T* dst = vpool + value_index(page, (int)(kv_row - page * pv.page_size), head - nh - nkv, nkv, hd, pv.page_size);
+        T* dst = vpool + value_index(kv_row, head - nh - nkv, nkv, hd);
         for (int d = lane; d < hd; d += 64) dst[value_d_offset(d)] = from_f32<T>(load(d));
     }
 }

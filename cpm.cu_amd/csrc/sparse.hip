@@ -35,9 +35,7 @@ __global__ void compress_keys_kernel(const T* __restrict__ kpool, T* __restrict_
         float s = 0.f;
         const int kvh = e / hd, d = e - kvh * hd;
         for (int r = 0; r < ks; ++r) {
-            const long row = paged_row(pv, slot, first + r);
-            const long pg = row / pv.page_size;
-            s += to_f32(kpool[key_index(pg, (int)(row - pg * pv.page_size), kvh, nkv, hd, pv.page_size) + key_d_offset(d)]);
+            s += to_f32(kpool[key_index(paged_row(pv, slot, first + r), kvh, nkv, hd) + key_d_offset(d)]);
         }
         ckpool[ck_index(page, (first % pv.page_size) / st, kvh, nkv, hd, rpp) + ck_d_offset(d, rpp)] = from_f32<T>(s / (float)ks);
     }

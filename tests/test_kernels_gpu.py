@@ -160,11 +160,11 @@ def test_silu_mul(dtype, I):
 
 # ---------------------------------------------------------------------------- attention over the paged cache
 def key_tiles(full):
-    """[page tokens, kv heads, d] -> the cache's layout of keys: per kv head and chunk of 32 tokens two tiles of
+    """[page tokens, kv heads, d] -> the cache's layout of keys: per chunk of 32 tokens and kv head two tiles of
     16 key slots (token 8a + 4u + i of the chunk is slot 4a + i of tile u), a tile [d / 8][slot][d % 8]."""
     page, nkv, hd = full.shape
     x = full.view(page // 32, 4, 2, 4, nkv, hd // 8, 8)          # chunk, a, u, i, kv head, d / 8, d % 8
-    return x.permute(4, 0, 2, 5, 1, 3, 6).contiguous()            # kv head, chunk, u, d / 8, a, i, d % 8
+    return x.permute(0, 4, 2, 5, 1, 3, 6).contiguous()            # chunk, kv head, u, d / 8, a, i, d % 8
 
 
 def key_elements(in_page, kvh, nkv, hd, page):
@@ -173,15 +173,15 @@ def key_elements(in_page, kvh, nkv, hd, page):
     a_, r = divmod(t32, 8)
     u, i = divmod(r, 4)
     d = torch.arange(hd)
-    return ((((kvh * (page // 32) + c) * 2 + u) * (hd // 8) + d // 8) * 16 + a_ * 4 + i) * 8 + d % 8
+    return ((((c * nkv + kvh) * 2 + u) * (hd // 8) + d // 8) * 16 + a_ * 4 + i) * 8 + d % 8
 
 
 def value_tiles(full):
-    """[page tokens, kv heads, d] -> the cache's layout of values: per kv head and chunk of 32 tokens
+    """[page tokens, kv heads, d] -> the cache's layout of values: per chunk of 32 tokens and kv head
     [d / 16][token / 8][d % 16][token % 8]."""
     page, nkv, hd = full.shape
     x = full.view(page // 32, 4, 8, nkv, hd // 16, 16)           # chunk, token / 8, token % 8, kv head, d / 16, d % 16
-    return x.permute(3, 0, 4, 1, 5, 2).contiguous()
+    return x.permute(0, 3, 4, 1, 5, 2).contiguous()
 
 
 def paged_setup(lens, nkv, hd, page, dtype, seed=0, scramble=True):
