@@ -165,9 +165,11 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_mfma_kernel(
     const int split = blockIdx.z;
     // TW > 1: the wavefronts of a workgroup take neighbouring tokens, which visit mostly the same keys at the
     // same time and so meet in the CU's L1
-    const int wave = TW > 1 ? 0 : threadIdx.x >> 6;
+    // (the wavefront's number is the same in all its lanes: saying so keeps what follows from it in scalar registers)
+    const int wave_id = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int wave = TW > 1 ? 0 : wave_id;
     if (TW > 1) {
-        t = t * TW + (threadIdx.x >> 6);
+        t = t * TW + wave_id;
         if (t >= n_tokens) return;
     }
     const int lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
@@ -214,14 +216,14 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_mfma_kernel(
         return sel[c / cpb] * block_size + (c % cpb) * 32;
     };
     // Where the wavefront's chunks lie is looked up for 64 chunks at a time, one chunk a lane (its first key and
-    // its physical chunk of the pool), and read back lane by lane: the loads of keys and values then wait for
-    // no address lookup, and the loop holds no division.
-    int key0_v = 0, pchunk_v = 0, kbase = 0;
-    auto lookup = [&](int kb) {
-        const int cj = c0 + wave + (kb + lane) * NW;
+    // its physical chunk of the pool), a batch ahead, and read back lane by lane: the loads of keys and values
+    // then wait for no address lookup, and the loop holds no division.
+    const int n_mine = c1 > c0 + wave ? (c1 - c0 - wave + NW - 1) / NW : 0;      // chunks of this wavefront
+    auto lookup = [&](int kb, int& key0_v, int& pchunk_v) {
+        const int kj = kb + lane;
         int k0 = 0, pc = 0;
-        if (cj < c1) {
-            k0 = chunk_key0(cj);
+        if (kj < n_mine) {
+            k0 = chunk_key0(c0 + wave + kj * NW);
             pc = (int)(paged_row(pv, slot, k0) >> 5);
         }
         key0_v = k0;
@@ -252,87 +254,83 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_mfma_kernel(
     };
     // One buffer each for keys and values: the next chunk's keys are asked for as soon as this chunk's scores
     // are issued, its values as soon as this chunk's P.V is, so both arrive behind the other half of the work
-    // (and behind the other wavefronts of the SIMD).
-    int c = c0 + wave, k = 0;
-    abf16x8_t kf[2][KSTEPS], vf[DT];
-    int key0 = 0;
-    if (c < c1) {
-        lookup(0);
-        key0 = __builtin_amdgcn_readlane(key0_v, 0);
-        const int pchunk = __builtin_amdgcn_readlane(pchunk_v, 0);
+    // (and behind the other wavefronts of the SIMD).  The loads stand outside every branch (the last chunk
+    // asks for itself once more) so that the waits for them are counted exactly.
+    if (n_mine > 0) {
+        abf16x8_t kf[2][KSTEPS], vf[DT];
+        int key0_c, pchunk_c, key0_x, pchunk_x;
+        lookup(0, key0_c, pchunk_c);
+        int key0 = __builtin_amdgcn_readlane(key0_c, 0);
+        int pchunk = __builtin_amdgcn_readlane(pchunk_c, 0);
         load_k(pchunk, kf);
         load_v(pchunk, vf);
-    }
-    while (c < c1) {
-        const int cn = c + NW;
-        ++k;
-        int key0n = 0, pchunkn = 0;
-        if (cn < c1) {
-            if (k - kbase == 64) {
-                kbase = k;
-                lookup(kbase);
-            }
-            key0n = __builtin_amdgcn_readlane(key0_v, k - kbase);
-            pchunkn = __builtin_amdgcn_readlane(pchunk_v, k - kbase);
-        }
-        const bool live = key0 <= pos;           // a listed block may reach beyond the token's own position
-        afloatx4_t st[2];
-        if (live) {
+        for (int kb = 0; kb < n_mine; kb += 64) {
+            lookup(kb + 64, key0_x, pchunk_x);
+            const int lim = min(64, n_mine - kb);
+            for (int i = 0; i < lim; ++i) {
+                int key0n = i < 63 ? __builtin_amdgcn_readlane(key0_c, (i + 1) & 63) : __builtin_amdgcn_readlane(key0_x, 0);
+                int pchunkn = i < 63 ? __builtin_amdgcn_readlane(pchunk_c, (i + 1) & 63)
+                                     : __builtin_amdgcn_readlane(pchunk_x, 0);
+                if (kb + i + 1 >= n_mine) {
+                    key0n = key0;
+                    pchunkn = pchunk;
+                }
+                afloatx4_t st[2];
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                st[u] = afloatx4_t{0.f, 0.f, 0.f, 0.f};
+                for (int u = 0; u < 2; ++u) {
+                    st[u] = afloatx4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int ks = 0; ks < KSTEPS; ++ks)
-                    st[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][ks], qf[ks], st[u], 0, 0, 0);
-            }
-        }
-        if (cn < c1) load_k(pchunkn, kf);
-        if (live) {
-            // lane (head n, g): st[u][i] is key key0 + 8g + 4u + i; only the chunk that holds the token's own
-            // position needs the causal mask
-            float sc[8];
+                    for (int ks = 0; ks < KSTEPS; ++ks)
+                        st[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][ks], qf[ks], st[u], 0, 0, 0);
+                }
+                load_k(pchunkn, kf);
+                // lane (head n, g): st[u][i] is key key0 + 8g + 4u + i; only a chunk that reaches beyond the
+                // token's own position needs the causal mask (a listed block may even lie wholly beyond it)
+                if (key0 + 31 > pos) {
 #pragma unroll
-            for (int u = 0; u < 2; ++u)
+                    for (int u = 0; u < 2; ++u)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) sc[u * 4 + i] = st[u][i];
-            if (key0 + 31 > pos) {
+                        for (int e = 0; e < 4; ++e)
+                            if (key0 + 8 * g + 4 * u + e > pos) st[u][e] = -INFINITY;
+                }
+                float mx = fmaxf(fmaxf(fmaxf(st[0][0], st[0][1]), fmaxf(st[0][2], st[0][3])),
+                                 fmaxf(fmaxf(st[1][0], st[1][1]), fmaxf(st[1][2], st[1][3])));
+                mx = rows_max(mx);
+                // m is kept in units of the exponent: scores times scale*log2(e)
+                const float m_new = fmaxf(m, mx * scale_log2e);
+                const float m_ref = m_new == -INFINITY ? 0.f : m_new;      // nothing seen yet: all weights 0
+                const float corr = fast_exp2(m - m_ref);
+                float rs = 0.f;
+                abf16x8_t pb;
 #pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    if (key0 + 8 * g + j > pos) sc[j] = -INFINITY;
-            }
-            float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
-            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            // m is kept in units of the exponent: scores times scale*log2(e)
-            const float m_new = fmaxf(m, mx * scale_log2e);
-            const float corr = fast_exp2(m - m_new);
-            float rs = 0.f;
-            abf16x8_t pb;
+                for (int u = 0; u < 2; ++u)
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const float p = fast_exp2(__builtin_fmaf(sc[j], scale_log2e, -m_new));
-                rs += p;
-                pb[j] = (__bf16)p;
-            }
-            rs += __shfl_xor(rs, 16, 64);
-            rs += __shfl_xor(rs, 32, 64);
-            l = l * corr + rs;
-            // the accumulators are rescaled only when some row's maximum moved (rare after the first chunks)
-            if (__builtin_amdgcn_ballot_w64(m_new != m) != 0) {
+                    for (int e = 0; e < 4; ++e) {
+                        const float p = fast_exp2(__builtin_fmaf(st[u][e], scale_log2e, -m_ref));
+                        rs += p;
+                        pb[u * 4 + e] = (__bf16)p;
+                    }
+                rs = rows_sum(rs);
+                l = l * corr + rs;
+                // the accumulators are rescaled only when some row's maximum moved (rare after the first chunks)
+                if (__builtin_amdgcn_ballot_w64(m_new != m) != 0) {
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[dt][e] *= corr;
+                }
+                m = m_new;
+                // O^T += V^T . P^T ; A operand: lane (d row n, g) holds V^T[d][key0 + 8g .. +8]
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) acc[dt][i] *= corr;
+                    acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pb, acc[dt], 0, 0, 0);
+                load_v(pchunkn, vf);
+                key0 = key0n;
+                pchunk = pchunkn;
             }
-            m = m_new;
-            // O^T += V^T . P^T ; A operand: lane (d row n, g) holds V^T[d][key0 + 8g .. +8]
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-                acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pb, acc[dt], 0, 0, 0);
+            key0_c = key0_x;
+            pchunk_c = pchunk_x;
         }
-        if (cn < c1) load_v(pchunkn, vf);
-        c = cn;
-        key0 = key0n;
     }
 
     if (NW > 1) {

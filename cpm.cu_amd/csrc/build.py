@@ -41,10 +41,11 @@ HIPCC_FLAGS = [
 
 
 # extra flags of single libraries
-#   attention: matrix-core results stay in ordinary vector registers; with the accumulation registers the
-#   compiler moves the running output there and back around every rescale
+#   attention: matrix-core results stay in ordinary vector registers (with the accumulation registers the
+#   compiler moves the running output there and back around every rescale); no score is ever NaN, which
+#   spares a canonicalising instruction before every max
 MODULE_FLAGS: Dict[str, List[str]] = {
-    "attention": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "attention": ["-mllvm", "-amdgpu-mfma-vgpr-form", "-fno-honor-nans"],
 }
 
 

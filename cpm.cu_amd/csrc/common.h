@@ -53,6 +53,22 @@ __device__ inline float wave_max(float v) {
     for (int o = CPMCU_WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, CPMCU_WAVE));
     return v;
 }
+// Max / sum over the four rows of 16 lanes of a wavefront (lanes that differ in bits 4 and 5 only); every
+// lane gets the result.  gfx950's row swaps exchange rows between two registers inside the vector unit:
+// swapping a value with itself leaves (row 0, row 0, row 2, row 2) and (row 1, row 1, row 3, row 3).
+typedef unsigned cpmcu_u32x2_t __attribute__((ext_vector_type(2)));
+__device__ inline float rows_max(float v) {
+    cpmcu_u32x2_t r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ inline float rows_sum(float v) {
+    cpmcu_u32x2_t r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
 // Sum over a block of up to 1024 threads; every thread gets the result.
 // `red` is LDS for 17 floats.  The order of the additions is fixed, so the
 // result does not depend on timing.
