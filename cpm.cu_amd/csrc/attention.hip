@@ -397,9 +397,9 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_mfma_kernel(
 // out[token][head][:] = sum_s 2^(m_s - m) o_s / sum_s 2^(m_s - m) l_s   (splits without keys have l = 0)
 __global__ void attention_combine_kernel(const float* __restrict__ part_o, const float2* __restrict__ part_ml,
                                          bf16_t* __restrict__ out, int hd, int n_splits) {
+    __shared__ float wgt[64];
     const long row = blockIdx.x;             // token * nh + head
     const float2* ml = part_ml + row * n_splits;
-    // every thread forms the shares' weights itself (at most 64 shares): no LDS, no barrier
     float m = -INFINITY;
     for (int s = 0; s < n_splits; ++s) {
         const float2 v = ml[s];
@@ -408,18 +408,17 @@ __global__ void attention_combine_kernel(const float* __restrict__ part_o, const
     float denom = 0.f;
     for (int s = 0; s < n_splits; ++s) {
         const float2 v = ml[s];
-        if (v.y > 0.f) denom += exp2f(v.x - m) * v.y;
+        const float wv = v.y > 0.f ? exp2f(v.x - m) : 0.f;
+        denom += wv * v.y;
+        if (threadIdx.x == 0) wgt[s] = wv;
     }
+    __syncthreads();
     const float inv = 1.0f / denom;
     const float* po = part_o + row * n_splits * hd;
     for (int d = threadIdx.x; d < hd; d += blockDim.x) {
         float a = 0.f;
 #pragma unroll 8
-        for (int s = 0; s < n_splits; ++s) {
-            const float2 v = ml[s];
-            const float wv = v.y > 0.f ? exp2f(v.x - m) : 0.f;
-            a += wv * po[(long)s * hd + d];
-        }
+        for (int s = 0; s < n_splits; ++s) a += wgt[s] * po[(long)s * hd + d];
         out[row * hd + d] = f32_to_bf16(a * inv);
     }
 }
