@@ -498,7 +498,9 @@ __global__ __launch_bounds__(NW * 64) void attention_prefill_mfma_kernel(
     constexpr int DT = HD / 16;
     const int tile_id = gridDim.x - 1 - blockIdx.x;      // later tiles of a prompt see more keys: start them first
     const int kvh = blockIdx.y % nkv, ht = blockIdx.y / nkv;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
+    // (the wavefront's number is the same in all its lanes: saying so keeps what follows from it in scalar registers)
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
     const int G = nh / nkv;
     const int t0 = tiles[2 * tile_id], n_tok = tiles[2 * tile_id + 1];
     const int slot = tok_slot[t0];
@@ -542,8 +544,12 @@ __global__ __launch_bounds__(NW * 64) void attention_prefill_mfma_kernel(
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) acc[r][dt] = afloatx4_t{0.f, 0.f, 0.f, 0.f};
     }
-    auto load_k = [&](int page, int po, abf16x8_t (&kf)[2][KSTEPS]) {
-        const bf16_t* kp = kpool + chunk_base((long)page * pv.page_size + po, kvh, nkv, HD) + (g * 16 + n) * 8;
+    const long chunk_elems = 32L * HD;
+    const bf16_t* kbase_p = kpool + (long)kvh * chunk_elems + (g * 16 + n) * 8;
+    const bf16_t* vbase_p = vtpool + (long)kvh * chunk_elems + (g * 16 + n) * 8;
+    const long chunk_stride = (long)nkv * chunk_elems;
+    auto load_k = [&](int pchunk, abf16x8_t (&kf)[2][KSTEPS]) {
+        const bf16_t* kp = kbase_p + pchunk * chunk_stride;
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
 #pragma unroll
@@ -554,28 +560,36 @@ __global__ __launch_bounds__(NW * 64) void attention_prefill_mfma_kernel(
             }
         }
     };
-    auto load_v = [&](int page, int po, abf16x8_t (&vf)[DT]) {
-        const bf16_t* vp = vtpool + chunk_base((long)page * pv.page_size + po, kvh, nkv, HD) + (g * 16 + n) * 8;
+    auto load_v = [&](int pchunk, abf16x8_t (&vf)[DT]) {
+        const bf16_t* vp = vbase_p + pchunk * chunk_stride;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) vf[dt] = *(const abf16x8_t*)(vp + dt * 512);
+    };
+    // the wavefront's chunks in turn: page number and chunk inside the page advance without a division
+    const int cpp = pv.page_size / 32;
+    int pg_i = wave / cpp, in_pg = wave % cpp;
+    auto next_pchunk = [&]() {
+        in_pg += NW;
+        while (in_pg >= cpp) {
+            in_pg -= cpp;
+            ++pg_i;
+        }
+        return ptab[pg_i] * cpp + in_pg;
     };
     // one buffer each for keys and values: the next chunk's keys are asked for as soon as the last tile's
     // scores are issued, its values as soon as the last tile's P.V is, so both arrive behind other work
     // with NW wavefronts a workgroup the chunks are dealt to them in turn and merged at the end
     abf16x8_t kf[2][KSTEPS], vf[DT];
     if (wave < total_chunks) {
-        const int page = ptab[(wave * 32) / pv.page_size];
-        load_k(page, (wave * 32) % pv.page_size, kf);
-        load_v(page, (wave * 32) % pv.page_size, vf);
+        const int pchunk = ptab[pg_i] * cpp + in_pg;
+        load_k(pchunk, kf);
+        load_v(pchunk, vf);
     }
     for (int c = wave; c < total_chunks; c += NW) {
         const int key0 = c * 32;
         const bool more = c + NW < total_chunks;
-        int pagen = 0, pon = 0;
-        if (more) {
-            pagen = ptab[(key0 + 32 * NW) / pv.page_size];
-            pon = (key0 + 32 * NW) % pv.page_size;
-        }
+        int pchunkn = 0;
+        if (more) pchunkn = next_pchunk();
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const bool active = r < n_tiles_used && key0 <= tile_last_pos[r];
@@ -589,7 +603,7 @@ __global__ __launch_bounds__(NW * 64) void attention_prefill_mfma_kernel(
                         st[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][ks], qf[r][ks], st[u], 0, 0, 0);
                 }
             }
-            if (r == R - 1 && more) load_k(pagen, pon, kf);      // the last tile's scores are issued: keys are free
+            if (r == R - 1 && more) load_k(pchunkn, kf);      // the last tile's scores are issued: keys are free
             if (active) {
                 // raw scores; only a chunk that reaches past a row's position needs the causal mask
                 float sc[8];
@@ -606,8 +620,7 @@ __global__ __launch_bounds__(NW * 64) void attention_prefill_mfma_kernel(
                 }
                 float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
                                  fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
-                mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                mx = rows_max(mx);
                 // running maximum in units of scaled scores (scale > 0); a row whose position lies before
                 // this chunk sees none of its keys: nothing changes for it
                 const float m_new = fmaxf(m[r], mx * scale_log2e);
@@ -621,8 +634,7 @@ __global__ __launch_bounds__(NW * 64) void attention_prefill_mfma_kernel(
                     rs += p;
                     pb[j] = (__bf16)p;
                 }
-                rs += __shfl_xor(rs, 16, 64);
-                rs += __shfl_xor(rs, 32, 64);
+                rs = rows_sum(rs);
                 l[r] = l[r] * corr + rs;
                 // the accumulators are rescaled only when some row's maximum moved (rare after the first chunks)
                 if (__builtin_amdgcn_ballot_w64(m_new != m[r]) != 0) {
@@ -637,7 +649,7 @@ __global__ __launch_bounds__(NW * 64) void attention_prefill_mfma_kernel(
                     acc[r][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pb, acc[r][dt], 0, 0, 0);
             }
         }
-        if (more) load_v(pagen, pon, vf);
+        if (more) load_v(pchunkn, vf);
     }
     if (NW > 1) {
         // wavefronts 1.. hand their running results to wavefront 0, one after the other through one buffer
@@ -719,15 +731,18 @@ extern "C" const char* cpmcu_attention_prefill_mfma(const void* q, void* out, in
     dim3 grid(n_tiles, nkv * HT);
     const float sl = scale * 1.4426950408889634f;
     CPMCU_REQUIRE(tiles_per_wave == 2 || tiles_per_wave == 4, "attention_prefill: %d tiles a wavefront (2 or 4 are built)", tiles_per_wave);
-    CPMCU_REQUIRE(waves_per_group == 1 || waves_per_group == 2, "attention_prefill: %d wavefronts a workgroup (1 or 2 are built)", waves_per_group);
+    CPMCU_REQUIRE(waves_per_group == 1 || waves_per_group == 2 || waves_per_group == 4,
+                  "attention_prefill: %d wavefronts a workgroup (1, 2 or 4 are built)", waves_per_group);
 #define LAUNCH(HDv, Rv, NWv)                                                                                     \
     attention_prefill_mfma_kernel<HDv, Rv, NWv><<<grid, NWv * 64, 0, stream>>>(                                  \
         (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kpool, (const bf16_t*)vtpool, pv, tiles, positions,       \
         tok_slot, nh, nkv, sl, rpt, tpt)
 #define BY_R(HDv)                                                               \
     do {                                                                        \
-        if (tiles_per_wave == 4 && waves_per_group == 2) LAUNCH(HDv, 4, 2);     \
+        if (tiles_per_wave == 4 && waves_per_group == 4) LAUNCH(HDv, 4, 4);     \
+        else if (tiles_per_wave == 4 && waves_per_group == 2) LAUNCH(HDv, 4, 2); \
         else if (tiles_per_wave == 4) LAUNCH(HDv, 4, 1);                        \
+        else if (waves_per_group == 4) LAUNCH(HDv, 2, 4);                       \
         else if (waves_per_group == 2) LAUNCH(HDv, 2, 2);                       \
         else LAUNCH(HDv, 2, 1);                                                 \
     } while (0)

@@ -238,14 +238,15 @@ def attention_prefill_tokens_per_wave(nh: int, nkv: int, tiles_per_wave: int = 4
 
 
 def attention_prefill_shape(n_tokens: int, nh: int, nkv: int, hd: int):
-    """(tiles a wavefront, wavefronts a workgroup) for the prompt kernel.  4 tiles of 16 rows a wavefront
-    halve the cache traffic of 2; when a prompt is too short to give every SIMD of the 256 CUs a wavefront of
-    its own twice over, two wavefronts share each group of tiles, taking the chunks of keys in turn, which also
-    evens out the causal triangle (measured on the MI355X at head size 128, 2,048 tokens: 128 us against 189 us
-    with one wavefront and 148 us with 2 tiles; at 8,192 tokens one wavefront is best, 1.36 ms)."""
-    per4 = attention_prefill_tokens_per_wave(nh, nkv, 4)
-    waves4 = -(-n_tokens // per4) * nkv * -(-(nh // nkv) // 16)
-    return 4, (2 if waves4 < 2048 else 1)
+    """(tiles a wavefront, wavefronts a workgroup) for the prompt kernel.  Measured on the MI355X at head size
+    128, 32 heads in 2 groups, one prompt of 512 / 2,048 / 8,192 / 32,768 tokens, in us:
+      2 tiles, 1 / 2 / 4 wavefronts:  25 / 20 / 19    95 / 75 / 90    894 / 819 / 835   11.3 / 11.6 / 11.8 ms
+      4 tiles, 1 / 2 / 4 wavefronts:  37 / 26 / 24   123 / 86 / 116   888 / 904 / 1058  13.7 / 13.4 / 14.1 ms
+    Two tiles of 16 rows a wavefront leave room for two wavefronts a SIMD; wavefronts that share a group of
+    tiles take the chunks of keys in turn, which evens out the causal triangle of short prompts."""
+    if n_tokens <= 1024:
+        return 2, 4
+    return 2, (2 if n_tokens < 16384 else 1)
 
 
 def attention_prefill_mfma(q: torch.Tensor, out: torch.Tensor, tiles: torch.Tensor, nh: int, nkv: int, hd: int,

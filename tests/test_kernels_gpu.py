@@ -261,7 +261,7 @@ def test_attention_over_scrambled_pages(nh, nkv, hd, dtype):
                                splits, po, pm, waves_per_group=nw)
             assert float((out.double().cpu().view(n, nh, hd) - ref).abs().max()) <= tol, f"splits={splits} waves={nw}"
         # the prompt kernel: runs of consecutive tokens of one sequence share a wavefront
-        for r, nw in ((2, 1), (4, 1), (2, 2), (4, 2)):
+        for r, nw in ((2, 1), (4, 1), (2, 2), (4, 2), (2, 4), (4, 4)):
             tpw = ops.attention_prefill_tokens_per_wave(nh, nkv, r)
             tiles = ops.prefill_tiles([40, 1, 1], tpw, DEV)
             out.fill_(float("nan"))
@@ -292,7 +292,7 @@ def test_prompt_attention_from_position_zero_and_continued(nh, nkv, hd):
     ref = attention_reference(q.double().cpu(), ks, vs, positions, seq_of, nh, scale)
     pos_t = torch.tensor(positions, dtype=torch.int32, device=DEV)
     slot_t = torch.tensor(seq_of, dtype=torch.int32, device=DEV)
-    for r, nw in ((2, 1), (4, 1), (2, 2), (4, 2)):
+    for r, nw in ((2, 1), (4, 1), (2, 2), (4, 2), (2, 4), (4, 4)):
         tiles = ops.prefill_tiles(q_lens, ops.attention_prefill_tokens_per_wave(nh, nkv, r), DEV)
         out = torch.full((n, nh * hd), float("nan"), dtype=dtype, device=DEV)
         ops.attention_prefill_mfma(q.view(n, -1), out, tiles, nh, nkv, hd, scale, kpool, vpool, table, page, pos_t,
