@@ -43,16 +43,6 @@ template <typename T> __host__ __device__ inline T from_f32(float f);
 template <> __host__ __device__ inline float from_f32<float>(float f) { return f; }
 template <> __host__ __device__ inline bf16_t from_f32<bf16_t>(float f) { return f32_to_bf16(f); }
 
-__device__ inline float wave_sum(float v) {
-#pragma unroll
-    for (int o = CPMCU_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, CPMCU_WAVE);
-    return v;
-}
-__device__ inline float wave_max(float v) {
-#pragma unroll
-    for (int o = CPMCU_WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, CPMCU_WAVE));
-    return v;
-}
 // Max / sum over the four rows of 16 lanes of a wavefront (lanes that differ in bits 4 and 5 only); every
 // lane gets the result.  gfx950's row swaps exchange rows between two registers inside the vector unit:
 // swapping a value with itself leaves (row 0, row 0, row 2, row 2) and (row 1, row 1, row 3, row 3).
@@ -69,6 +59,29 @@ __device__ inline float rows_sum(float v) {
     r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
+// Sum / max over the 64 lanes of a wavefront, the result in every lane, inside the vector unit: four steps
+// over a row of 16 lanes with the data-parallel lane patterns (neighbours, pairs, mirrored halves of 8,
+// mirrored halves of 16), then the four rows.  The order of the operations is fixed.
+// (a lane whose partner is switched off reads `idle`: 0 for sums, its own value for maxima)
+#define CPMCU_DPP(v, ctrl) __uint_as_float(__builtin_amdgcn_update_dpp(0, __float_as_uint(v), ctrl, 0xf, 0xf, false))
+#define CPMCU_DPP_SELF(v, ctrl) \
+    __uint_as_float(__builtin_amdgcn_update_dpp(__float_as_uint(v), __float_as_uint(v), ctrl, 0xf, 0xf, false))
+__device__ inline float row16_sum(float v) {
+    v += CPMCU_DPP(v, 0xB1);      // quad_perm [1,0,3,2]
+    v += CPMCU_DPP(v, 0x4E);      // quad_perm [2,3,0,1]
+    v += CPMCU_DPP(v, 0x141);     // row_half_mirror
+    v += CPMCU_DPP(v, 0x140);     // row_mirror
+    return v;
+}
+__device__ inline float row16_max(float v) {
+    v = fmaxf(v, CPMCU_DPP_SELF(v, 0xB1));
+    v = fmaxf(v, CPMCU_DPP_SELF(v, 0x4E));
+    v = fmaxf(v, CPMCU_DPP_SELF(v, 0x141));
+    v = fmaxf(v, CPMCU_DPP_SELF(v, 0x140));
+    return v;
+}
+__device__ inline float wave_sum(float v) { return rows_sum(row16_sum(v)); }
+__device__ inline float wave_max(float v) { return rows_max(row16_max(v)); }
 // Sum over a block of up to 1024 threads; every thread gets the result.
 // `red` is LDS for 17 floats.  The order of the additions is fixed, so the
 // result does not depend on timing.

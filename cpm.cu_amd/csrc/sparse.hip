@@ -171,6 +171,101 @@ __global__ __launch_bounds__(256) void sparse_select_kernel(const T* __restrict_
     }
 }
 
+// ---------------------------------------------------------------------------
+// From the scores of the visible compressed keys (LDS score[0, n_vis)) to the ascending block list of one
+// (token, kv head): pool the scores over each candidate block, rank the candidates by (larger pooled score,
+// lower index), flag the first topk ranks and the window, write the flagged blocks in ascending order.
+// A candidate's pooled score and index make one 64-bit key (the float's bits made monotone, then the index
+// counted down), so that its rank is the number of larger keys: one comparison a pair.  When the block has
+// more threads than candidates, several threads share a candidate's scan.
+// work: LDS for select_work_floats(max_blocks) floats, 16-byte aligned; every thread of the block calls this.
+// ---------------------------------------------------------------------------
+__host__ __device__ inline int select_work_floats(int max_blocks) { return 4 * ((max_blocks + 3) / 4 * 4) + 4; }
+
+template <int NW>
+__device__ inline void blocks_from_scores(const float* score, float* work, int* wave_tot, const SelectParams& sp,
+                                          int n_vis, int q_block, int n_cand, long out_idx,
+                                          int* __restrict__ sel_blocks, int* __restrict__ sel_count) {
+    constexpr int NT = NW * 64;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int mb4 = (sp.max_blocks + 3) / 4 * 4;
+    unsigned long long* keys = (unsigned long long*)work;        // [mb4]
+    int* rank = (int*)(work + 2 * mb4);                          // [mb4]
+    int* flag = rank + mb4;                                      // [mb4]
+    const int n_cand2 = (n_cand + 1) / 2 * 2;
+    for (int b = tid; b < n_cand2; b += NT) {
+        float v = -INFINITY;
+        if (b < sp.init_blocks && b < n_cand) {
+            v = INFINITY;
+        } else if (b < n_cand) {
+            const int lo_tok = sp.bs * b - sp.ks + 1;
+            const int j_lo = lo_tok <= 0 ? 0 : (lo_tok + sp.st - 1) / sp.st;
+            const int j_hi = min((sp.bs * (b + 1) - 1) / sp.st, n_vis - 1);
+            for (int j = j_lo; j <= j_hi; ++j) v = fmaxf(v, score[j]);
+        }
+        unsigned u = __float_as_uint(v);
+        u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);           // larger float, larger unsigned
+        // the padding entry (n_cand odd) gets the smallest key of all: it is counted by nobody
+        keys[b] = b < n_cand ? (((unsigned long long)u << 32) | (unsigned)(0x7fffffff - b)) : 0ull;
+        rank[b] = 0;
+    }
+    __syncthreads();
+    if (n_cand > 0) {
+        const int nb_pad = (n_cand + 63) / 64 * 64;
+        const int parts = nb_pad < NT ? NT / nb_pad : 1;          // threads that share a candidate's scan
+        const int chunk = ((n_cand2 + parts - 1) / parts + 1) / 2 * 2;
+        for (int e = tid; e < parts * nb_pad; e += NT) {
+            const int b = e % nb_pad, part = e / nb_pad;
+            if (b >= n_cand) continue;
+            const unsigned long long mine = keys[b];
+            const int o0 = part * chunk, o1 = min(o0 + chunk, n_cand2);
+            int r = 0;
+            // two keys a read, eight reads in flight, so that the latencies of LDS overlap
+#pragma unroll 8
+            for (int o = o0; o < o1; o += 2) {
+                const ulonglong2 k2 = *(const ulonglong2*)(keys + o);
+                r += (k2.x > mine ? 1 : 0) + (k2.y > mine ? 1 : 0);
+            }
+            if (parts > 1) atomicAdd(&rank[b], r);                // integers: the order does not matter
+            else rank[b] = r;
+        }
+    }
+    __syncthreads();
+    for (int b = tid; b <= q_block; b += NT) flag[b] = b < n_cand ? (rank[b] < sp.topk ? 1 : 0) : 1;   // window: all
+    __syncthreads();
+    // ascending list: a prefix count over the flags, one block a thread a round
+    int* dst = sel_blocks + out_idx * sp.max_sel;
+    int base = 0;
+    for (int b0 = 0; b0 <= q_block; b0 += NT) {
+        const int b = b0 + tid;
+        const int f = (b <= q_block) ? flag[b] : 0;
+        const unsigned long long mask = __builtin_amdgcn_ballot_w64(f != 0);
+        const int before = __popcll(mask & ((1ull << lane) - 1ull));
+        if (lane == 0) wave_tot[wave] = __popcll(mask);
+        __syncthreads();
+        int off = base;
+        for (int w = 0; w < wave; ++w) off += wave_tot[w];
+        if (f && off + before < sp.max_sel) dst[off + before] = b;
+        for (int w = 0; w < NW; ++w) base += wave_tot[w];
+        __syncthreads();
+    }
+    if (tid == 0) sel_count[out_idx] = min(base, sp.max_sel);
+}
+
+// steps of few tokens: three kernels (defined at the end of this file)
+struct SelectScratch {
+    float* sraw;      // [token * kv head][head of the group][max_ck]      raw scores * scale * log2(e)
+    float* stats;     // [token * kv head][group of 64 keys][head][2]      (max, sum of 2^(s - max)) of the group
+    float* score;     // [token * kv head][max_ck]                          softmax summed over the heads
+    int n_groups;
+};
+template <int HD>
+__global__ void select_scores_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ ckpool, PagedView pv,
+                                     const int* __restrict__ positions, const int* __restrict__ tok_slot,
+                                     SelectParams sp, SelectScratch sc);
+__global__ void select_normalise_kernel(const int* __restrict__ positions, SelectParams sp, SelectScratch sc);
+__global__ void select_blocks_kernel(const int* __restrict__ positions, SelectParams sp, SelectScratch sc,
+                                     int* __restrict__ sel_blocks, int* __restrict__ sel_count);
 template <int HD, int NW>
 __global__ void sparse_select_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ ckpool, PagedView pv,
                                           const int* __restrict__ positions, const int* __restrict__ tok_slot,
@@ -181,7 +276,7 @@ extern "C" const char* cpmcu_sparse_select(const void* q, const void* ckpool, in
                                            int page_size, const int* positions, const int* tok_slot, int ks, int st,
                                            int bs, int init_blocks, int topk, int window_blocks, int dense_len,
                                            int max_pos, int* sel_blocks, int* sel_count, int max_sel,
-                                           int force_plain, hipStream_t stream) {
+                                           int force_plain, float* scratch, long scratch_floats, hipStream_t stream) {
     CPMCU_REQUIRE(n > 0 && nh > 0 && nkv > 0 && hd > 0 && nh % nkv == 0, "sparse_select: bad shape");
     CPMCU_REQUIRE(hd % 8 == 0, "sparse_select: compressed keys lie in pieces of 8 elements; head_dim %d is no multiple", hd);
     CPMCU_REQUIRE(st > 0 && ks >= st && bs % st == 0 && page_size % st == 0,
@@ -197,14 +292,49 @@ extern "C" const char* cpmcu_sparse_select(const void* q, const void* ckpool, in
     sp.max_ck = max_pos < ks ? 1 : (max_pos - ks) / st + 1;
     sp.max_blocks = max_pos / bs + 1;
     sp.max_sel = max_sel;
-    const size_t lds = sizeof(float) * ((size_t)2 * sp.max_ck + 2 * sp.max_blocks + hd);
+    const size_t lds = sizeof(float) * ((size_t)2 * sp.max_ck + 2 * sp.max_blocks + hd + 8);
     CPMCU_REQUIRE(lds <= 60 * 1024,
                   "sparse_select: a context of %d tokens needs %zu bytes of LDS for its block scores (limit 61440)",
                   max_pos + 1, lds);
     dim3 grid(n, nkv);
     PagedView pv{page_table, table_width, page_size};
     if (dtype == CPMCU_BF16 && !force_plain && (hd == 16 || hd == 32 || hd == 64 || hd == 128)) {
-        const size_t lds2 = sizeof(float) * ((size_t)sp.max_ck + 2 * sp.max_blocks);
+        const size_t lds2 = sizeof(float) * ((size_t)sp.max_ck + 4 + select_work_floats(sp.max_blocks));
+        CPMCU_REQUIRE(lds2 <= 60 * 1024,
+                      "sparse_select: a context of %d tokens needs %zu bytes of LDS for its block scores (limit 61440)",
+                      max_pos + 1, lds2);
+        const int G = nh / nkv;
+        if (scratch && n * nkv <= 256) {
+            // few tokens: raw scores and their softmax by many small workgroups through `scratch`, then one
+            // workgroup a (token, kv head) for the block list
+            SelectScratch sc;
+            sc.n_groups = (sp.max_ck + 63) / 64;
+            const long rows = (long)n * nkv;
+            const long need = rows * ((long)sp.max_ck * (G + 1) + (long)sc.n_groups * G * 2);
+            CPMCU_REQUIRE(scratch_floats >= need, "sparse_select: scratch of %ld floats, %ld needed", scratch_floats, need);
+            sc.sraw = scratch;
+            sc.stats = sc.sraw + rows * sp.max_ck * G;
+            sc.score = sc.stats + rows * sc.n_groups * G * 2;
+            dim3 sgrid(n, nkv * ((G + 15) / 16), sc.n_groups);
+            CPMCU_REQUIRE(sgrid.y <= 65535 && sgrid.z <= 65535, "sparse_select: too many head tiles or compressed keys");
+            CPMCU_REQUIRE(G <= 256, "sparse_select: %d heads a kv head (256 are taken)", G);
+#define SCORES(HDv)                                                                                               \
+            select_scores_kernel<HDv><<<sgrid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)ckpool, pv, positions, \
+                                                                 tok_slot, sp, sc)
+            if (hd == 16) SCORES(16);
+            else if (hd == 32) SCORES(32);
+            else if (hd == 64) SCORES(64);
+            else SCORES(128);
+#undef SCORES
+            CPMCU_LAUNCH_CHECK("select_scores");
+            const size_t lds3 = sizeof(float) * ((size_t)sc.n_groups * G * 2 + 2 * G);
+            CPMCU_REQUIRE(lds3 <= 60 * 1024, "sparse_select: %d groups of compressed keys x %d heads exceed LDS", sc.n_groups, G);
+            select_normalise_kernel<<<dim3(n, nkv, (sp.max_ck + 255) / 256), 256, lds3, stream>>>(positions, sp, sc);
+            CPMCU_LAUNCH_CHECK("select_normalise");
+            select_blocks_kernel<<<grid, 1024, lds2, stream>>>(positions, sp, sc, sel_blocks, sel_count);
+            CPMCU_LAUNCH_CHECK("select_blocks");
+            return nullptr;
+        }
         // few tokens (decode steps): 16 wavefronts share a (token, kv head)'s compressed keys; many: 4
 #define LAUNCH(HDv)                                                                                          \
         do {                                                                                                 \
@@ -261,8 +391,7 @@ __global__ __launch_bounds__(NW * 64) void sparse_select_mfma_kernel(
     __shared__ float stat_s[NW][16][2];
     __shared__ int wave_tot[NW];
     float* score = lds;
-    float* pool = score + sp.max_ck;
-    int* flag = (int*)(pool + sp.max_blocks);
+    float* work = score + (sp.max_ck + 3) / 4 * 4;
 
     const int t = blockIdx.x, kvh = blockIdx.y, tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63, n = lane & 15, g = lane >> 4;
@@ -376,49 +505,151 @@ __global__ __launch_bounds__(NW * 64) void sparse_select_mfma_kernel(
         }
     }
     __syncthreads();
-    // pool the scores of the compressed keys that overlap each candidate block
-    for (int b = tid; b < n_cand; b += blockDim.x) {
-        float v = -INFINITY;
-        if (b < sp.init_blocks) {
-            v = INFINITY;
-        } else {
-            const int lo_tok = sp.bs * b - sp.ks + 1;
-            const int j_lo = lo_tok <= 0 ? 0 : (lo_tok + sp.st - 1) / sp.st;
-            const int j_hi = min((sp.bs * (b + 1) - 1) / sp.st, n_vis - 1);
-            for (int j = j_lo; j <= j_hi; ++j) v = fmaxf(v, score[j]);
+    blocks_from_scores<NW>(score, work, wave_tot, sp, n_vis, q_block, n_cand, out_idx, sel_blocks, sel_count);
+}
+
+// ===========================================================================
+// Steps of few tokens (decode): three kernels, because one workgroup for a (token, kv head) would pull the
+// compressed keys of a long context through a single CU, one memory latency after the other.
+//   select_scores_kernel:    a wavefront a tile of 16 compressed keys, a workgroup 64 keys: raw scores
+//                            sraw = q_head . ck_key * scale * log2(e), and per head the group's (max, sum)
+//   select_normalise_kernel: a thread a key: merges the groups' (max, sum) per head, then
+//                            score[key] = sum over heads of 2^(s - max) / sum
+//   select_blocks_kernel:    a workgroup a (token, kv head): blocks_from_scores
+// ===========================================================================
+template <int HD>
+__global__ __launch_bounds__(256) void select_scores_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ ckpool, PagedView pv,
+    const int* __restrict__ positions, const int* __restrict__ tok_slot, SelectParams sp, SelectScratch sc) {
+    constexpr int KSTEPS = (HD + 31) / 32;
+    __shared__ float st_s[4][16][2];
+    const int G = sp.nh / sp.nkv;
+    const int t = blockIdx.x, kvh = blockIdx.y % sp.nkv, ht = blockIdx.y / sp.nkv, grp = blockIdx.z;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
+    const int tile = grp * 4 + wave;
+    const int p = positions[t];
+    if (p + 1 <= sp.dense_len) return;
+    const int n_vis = p < sp.ks ? 0 : (p - sp.ks) / sp.st + 1;
+    if (grp * 64 >= n_vis) return;
+    const long row = (long)t * sp.nkv + kvh;
+    const int* ptab = pv.page_table + (long)tok_slot[t] * pv.table_width;
+    const int rpp = pv.page_size / sp.st;
+    // B operand first (two dependent loads): lane (key n, g) holds CK[key][32*ks + 8g .. +8]
+    const int j = min(tile * 16 + n, n_vis - 1);
+    const int pg = j / rpp;
+    const bf16_t* ck = ckpool + ck_index(ptab[pg], j - pg * rpp, kvh, sp.nkv, HD, rpp) + g * rpp * 8;
+    sbf16x8_t bf[KSTEPS], qf[KSTEPS];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+        sbf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (ks * 32 + g * 8 < HD) v = *(const sbf16x8_t*)(ck + ks * 4 * rpp * 8);
+        bf[ks] = v;
+    }
+    // A operand: lane (head r = n, g) holds Q[head][32*ks + 8g .. +8]
+    const bool head_ok = ht * 16 + n < G;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+        sbf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+        const int d = ks * 32 + g * 8;
+        if (head_ok && d < HD) v = *(const sbf16x8_t*)(q + ((long)t * sp.nh + (long)kvh * G + ht * 16 + n) * HD + d);
+        qf[ks] = v;
+    }
+    sfloatx4_t st = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ks], bf[ks], st, 0, 0, 0);
+    // st[i]: head ht*16 + 4g + i x key tile*16 + n
+    const bool key_ok = tile * 16 + n < n_vis;
+    const float c = sp.scale * 1.4426950408889634f;
+    float m[4], l[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float v = st[i] * c;
+        if (key_ok && ht * 16 + 4 * g + i < G) sc.sraw[(row * G + ht * 16 + 4 * g + i) * sp.max_ck + tile * 16 + n] = v;
+        m[i] = row16_max(key_ok ? v : -INFINITY);                 // over the tile's 16 keys
+        l[i] = row16_sum(key_ok ? exp2f(v - m[i]) : 0.f);
+    }
+    // the workgroup's 4 tiles into one (max, sum) per head
+    if (n == 0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            st_s[wave][4 * g + i][0] = m[i];
+            st_s[wave][4 * g + i][1] = l[i];
         }
-        pool[b] = v;
     }
     __syncthreads();
-    for (int b = tid; b <= q_block; b += blockDim.x) {
-        int f = 1;                                   // sliding window, the query's own block included
-        if (b < n_cand) {
-            const float v = pool[b];
-            int rank = 0;
-            for (int o = 0; o < n_cand; ++o) {
-                const float w = pool[o];
-                rank += (w > v || (w == v && o < b)) ? 1 : 0;
-            }
-            f = rank < sp.topk;
+    if (threadIdx.x < 16 && ht * 16 + (int)threadIdx.x < G) {
+        const int h = threadIdx.x;
+        float mm = -INFINITY;
+        for (int w = 0; w < 4; ++w) mm = fmaxf(mm, st_s[w][h][0]);
+        float ll = 0.f;
+        for (int w = 0; w < 4; ++w)
+            if (st_s[w][h][0] != -INFINITY) ll += st_s[w][h][1] * exp2f(st_s[w][h][0] - mm);
+        float* dst = sc.stats + ((row * sc.n_groups + grp) * G + ht * 16 + h) * 2;
+        dst[0] = mm;
+        dst[1] = ll;
+    }
+}
+
+__global__ __launch_bounds__(256) void select_normalise_kernel(const int* __restrict__ positions, SelectParams sp,
+                                                               SelectScratch sc) {
+    extern __shared__ float2 gst[];          // [group][head] (max, sum), then ms/inv behind it
+    const int t = blockIdx.x, kvh = blockIdx.y, tid = threadIdx.x;
+    const int p = positions[t];
+    if (p + 1 <= sp.dense_len) return;
+    const int G = sp.nh / sp.nkv;
+    const int n_vis = p < sp.ks ? 0 : (p - sp.ks) / sp.st + 1;
+    if ((int)blockIdx.z * 256 >= n_vis) return;
+    const long row = (long)t * sp.nkv + kvh;
+    const int groups = (n_vis + 63) / 64;
+    float* ms = (float*)(gst + (long)sc.n_groups * G);
+    float* inv = ms + G;
+    // all threads fetch the groups' (max, sum) at once; then a thread a head merges them in their order,
+    // so the result does not depend on which workgroup forms it
+    const float2* st = (const float2*)(sc.stats + row * sc.n_groups * G * 2);
+    for (int i = tid; i < groups * G; i += 256) gst[i] = st[i];
+    __syncthreads();
+    if (tid < G) {
+        float mm = -INFINITY;
+        for (int gi = 0; gi < groups; ++gi) mm = fmaxf(mm, gst[gi * G + tid].x);
+        float ll = 0.f;
+        for (int gi = 0; gi < groups; ++gi) {
+            const float2 v = gst[gi * G + tid];
+            ll += v.y * exp2f(v.x - mm);
         }
-        flag[b] = f;
+        ms[tid] = mm;
+        inv[tid] = ll > 0.f ? 1.0f / ll : 0.f;
     }
     __syncthreads();
-    // ascending list: a prefix count over the flags, one block a thread a round
-    int* dst = sel_blocks + out_idx * sp.max_sel;
-    int base = 0;
-    for (int b0 = 0; b0 <= q_block; b0 += NW * 64) {
-        const int b = b0 + tid;
-        const int f = (b <= q_block) ? flag[b] : 0;
-        const unsigned long long mask = __builtin_amdgcn_ballot_w64(f != 0);
-        const int before = __popcll(mask & ((1ull << lane) - 1ull));
-        if (lane == 0) wave_tot[wave] = __popcll(mask);
-        __syncthreads();
-        int off = base;
-        for (int w = 0; w < wave; ++w) off += wave_tot[w];
-        if (f && off + before < sp.max_sel) dst[off + before] = b;
-        for (int w = 0; w < NW; ++w) base += wave_tot[w];
-        __syncthreads();
+    const int j = blockIdx.z * 256 + tid;
+    if (j < n_vis) {
+        const float* s = sc.sraw + row * G * sp.max_ck + j;
+        float a = 0.f;
+#pragma unroll 16
+        for (int h = 0; h < G; ++h) a += exp2f(s[(long)h * sp.max_ck] - ms[h]) * inv[h];
+        sc.score[row * sp.max_ck + j] = a;
     }
-    if (tid == 0) sel_count[out_idx] = min(base, sp.max_sel);
+}
+
+__global__ __launch_bounds__(1024) void select_blocks_kernel(const int* __restrict__ positions, SelectParams sp,
+                                                             SelectScratch sc, int* __restrict__ sel_blocks,
+                                                             int* __restrict__ sel_count) {
+    constexpr int NW = 16;
+    extern __shared__ float lds[];
+    __shared__ int wave_tot[NW];
+    float* score = lds;
+    float* work = score + (sp.max_ck + 3) / 4 * 4;
+    const int t = blockIdx.x, kvh = blockIdx.y, tid = threadIdx.x;
+    const int p = positions[t];
+    const long out_idx = (long)t * sp.nkv + kvh;
+    if (p + 1 <= sp.dense_len) {
+        if (tid == 0) sel_count[out_idx] = -1;
+        return;
+    }
+    const int n_vis = p < sp.ks ? 0 : (p - sp.ks) / sp.st + 1;
+    const int q_block = p / sp.bs;
+    const int n_cand = max(q_block - sp.window_blocks + 1, 0);
+    for (int j = tid; j < n_vis; j += NW * 64) score[j] = sc.score[out_idx * sp.max_ck + j];
+    __syncthreads();
+    blocks_from_scores<NW>(score, work, wave_tot, sp, n_vis, q_block, n_cand, out_idx, sel_blocks, sel_count);
 }

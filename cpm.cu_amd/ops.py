@@ -315,12 +315,24 @@ def compress_keys(kpool: torch.Tensor, ckpool: torch.Tensor, nkv: int, page_tabl
                                                 _stream()))
 
 
+def sparse_select_scratch(n: int, nh: int, nkv: int, max_pos: int, kernel_size: int, kernel_stride: int) -> int:
+    """Floats of scratch with which sparse_select runs a step of few tokens as three kernels (raw scores and their
+    softmax by many small workgroups, then one workgroup a (token, kv head)); 0: the step has too many tokens
+    to gain."""
+    if n * nkv > 256:
+        return 0
+    max_ck = 1 if max_pos < kernel_size else (max_pos - kernel_size) // kernel_stride + 1
+    G = nh // nkv
+    return n * nkv * (max_ck * (G + 1) + -(-max_ck // 64) * G * 2)
+
+
 def sparse_select(q: torch.Tensor, ckpool: torch.Tensor, nh: int, nkv: int, hd: int, scale: float,
                   page_table: torch.Tensor, page_size: int, positions: torch.Tensor, tok_slot: torch.Tensor,
                   kernel_size: int, kernel_stride: int, block_size: int, init_blocks: int, topk: int,
                   window_blocks: int, dense_len: int, max_pos: int, sel_blocks: torch.Tensor, sel_count: torch.Tensor,
-                  force_plain: bool = False):
-    """Block list per (token, kv head): sel_count -1 = dense, else the ascending blocks to attend to."""
+                  force_plain: bool = False, scratch: Optional[torch.Tensor] = None):
+    """Block list per (token, kv head): sel_count -1 = dense, else the ascending blocks to attend to.
+    scratch: float32 of at least sparse_select_scratch(...) elements (bf16 steps of few tokens use it)."""
     _need(q, "select q", shape=(None, nh * hd))
     n = q.shape[0]
     _need(ckpool, "select compressed keys", q.dtype, (None, page_size // max(kernel_stride, 1), nkv * hd))
@@ -329,12 +341,15 @@ def sparse_select(q: torch.Tensor, ckpool: torch.Tensor, nh: int, nkv: int, hd: 
     _need(tok_slot, "select token slots", torch.int32, (n,))
     _need(sel_count, "select counts", torch.int32, (n, nkv))
     _need(sel_blocks, "select block list", torch.int32, (n, nkv, None))
+    if scratch is not None:
+        _need(scratch, "select scratch", torch.float32, (None,))
     _check(_fn("sparse", "cpmcu_sparse_select")(
         _p(q), _p(ckpool), c_int(_code(q)), c_int(n), c_int(nh), c_int(nkv), c_int(hd), c_float(scale),
         _p(page_table), c_int(page_table.shape[1]), c_int(page_size), _p(positions), _p(tok_slot),
         c_int(kernel_size), c_int(kernel_stride), c_int(block_size), c_int(init_blocks), c_int(topk),
         c_int(window_blocks), c_int(dense_len), c_int(max_pos), _p(sel_blocks), _p(sel_count),
-        c_int(sel_blocks.shape[2]), c_int(1 if force_plain else 0), _stream()))
+        c_int(sel_blocks.shape[2]), c_int(1 if force_plain else 0), _p(scratch),
+        c_long(scratch.numel() if scratch is not None else 0), _stream()))
 
 
 def argmax(logits: torch.Tensor, out: torch.Tensor):

@@ -112,10 +112,15 @@ class InfLLMv2Attention(GQAAttention):
             max_sel = self.topk + self.window_blocks
             sel_blocks = ctx.ws.get("attn.sel_blocks", (n, self.nkv, max_sel), torch.int32)
             sel_count = ctx.ws.get("attn.sel_count", (n, self.nkv), torch.int32)
+            scratch = None
+            if q.dtype == torch.bfloat16:
+                need = ops.sparse_select_scratch(n, self.nh, self.nkv, ctx.max_pos, self.ks, self.st)
+                if need:
+                    scratch = ctx.ws.get("attn.sel_scores", (need,), torch.float32)
             ops.sparse_select(q, cache.streams["ck"], self.nh, self.nkv, self.hd, self.scale, cache.page_table,
                               cache.page_size, ctx.positions, ctx.tok_slot, self.ks, self.st, self.bs,
                               self.init_blocks, self.topk, self.window_blocks, self.dense_len, ctx.max_pos,
-                              sel_blocks, sel_count)
+                              sel_blocks, sel_count, scratch=scratch)
             sel = (sel_blocks, sel_count, self.bs, self.window_blocks)
         a = self.attend(q, ctx, cache, sel)
         return self.o.forward(a, ctx, "attn.o", out_dtype=torch.float32, partials=True)

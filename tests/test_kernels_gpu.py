@@ -475,13 +475,17 @@ def test_block_selection_equals_the_plain_selection(dtype, nh, nkv, hd, ks, st, 
     sel_count = torch.full((n, nkv), -7, dtype=torch.int32, device=DEV)
     # plain selection from the same (rounded) keys; compressed keys in the cache's own precision
     ck_ref = plain.compressed_keys(kseq[0], ks, st).to(dtype).double()
-    for force_plain in ((False, True) if dtype == torch.bfloat16 else (True,)):     # matrix-core kernel and plain twin
+    # the matrix-core kernel, its two-kernel form for steps of few tokens, and the plain twin
+    scratch = torch.full((ops.sparse_select_scratch(n, nh, nkv, max(positions), ks, st),), float("nan"), device=DEV)
+    for force_plain, scr in (((False, None), (False, scratch), (True, None)) if dtype == torch.bfloat16
+                             else ((True, None),)):
         sel_blocks.fill_(-7)
         sel_count.fill_(-7)
         ops.sparse_select(q.view(n, -1), ck, nh, nkv, hd, hd ** -0.5, table, page,
                           torch.tensor(positions, dtype=torch.int32, device=DEV),
                           torch.zeros(n, dtype=torch.int32, device=DEV),
-                          ks, st, bs, init, topk, lb, dense_len, max(positions), sel_blocks, sel_count, force_plain)
+                          ks, st, bs, init, topk, lb, dense_len, max(positions), sel_blocks, sel_count, force_plain,
+                          scratch=scr)
         for t, p in enumerate(positions):
             want = plain.infllm_select(q[t].double().cpu(), ck_ref, p, sc, nkv)
             for h in range(nkv):
@@ -489,7 +493,7 @@ def test_block_selection_equals_the_plain_selection(dtype, nh, nkv, hd, ks, st, 
                 if want is None:
                     assert c == -1, (p, h)
                 else:
-                    assert sel_blocks[t, h, :c].tolist() == want[h], (p, h, want[h], force_plain)
+                    assert sel_blocks[t, h, :c].tolist() == want[h], (p, h, want[h], force_plain, scr is not None)
 
 
 def test_block_selection_ties_and_forced_blocks():
@@ -507,7 +511,12 @@ def test_block_selection_ties_and_forced_blocks():
         for init, topk, want in ((0, 3, [0, 1, 2, 11, 12]), (2, 2, [0, 1, 11, 12]), (1, 20, list(range(13)))):
             sb = torch.zeros(1, 1, topk + 2, dtype=torch.int32, device=DEV)
             cnt = torch.zeros(1, 1, dtype=torch.int32, device=DEV)
-            ops.sparse_select(q.to(dtype), ck.to(dtype), nh, nkv, hd, 0.25, table, page,
-                              torch.tensor([200], dtype=torch.int32, device=DEV),
-                              torch.zeros(1, dtype=torch.int32, device=DEV), ks, st, bs, init, topk, 2, 0, 200, sb, cnt)
-            assert sb[0, 0, :int(cnt[0, 0])].tolist() == want, dtype
+            for scr in ((None, torch.zeros(ops.sparse_select_scratch(1, nh, nkv, 200, ks, st), device=DEV))
+                        if dtype == torch.bfloat16 else (None,)):
+                sb.zero_()
+                cnt.zero_()
+                ops.sparse_select(q.to(dtype), ck.to(dtype), nh, nkv, hd, 0.25, table, page,
+                                  torch.tensor([200], dtype=torch.int32, device=DEV),
+                                  torch.zeros(1, dtype=torch.int32, device=DEV), ks, st, bs, init, topk, 2, 0, 200, sb,
+                                  cnt, scratch=scr)
+                assert sb[0, 0, :int(cnt[0, 0])].tolist() == want, (dtype, scr is not None)
