@@ -29,6 +29,7 @@ MODULES: Dict[str, List[str]] = {
     "gemm": ["gemm.hip"],
     "attention": ["attention.hip"],
     "sparse": ["sparse.hip"],
+    "qkv": ["qkv_rope.hip"],
 }
 HEADERS = ["common.h"]
 

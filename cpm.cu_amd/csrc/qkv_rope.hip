@@ -1,0 +1,139 @@
+// q, k, v projection of a decode step fused with the rotation and the cache write (bf16, at most 16 tokens).
+//
+// A decode step is a chain of small kernels, each of which costs a few microseconds whatever it does; this one
+// replaces the split-K product + the kernel that summed its partial sums, rotated and stored.
+//
+// The weight [q heads; k heads; v heads] x hidden is tiled as for the skinny product ([strip of 16 rows]
+// [128-column block][i][lane][8], ops.TiledWeight) but with the rows of every q and k head permuted so that
+// strip s of a head holds the features 8s .. 8s+7 and their rotation partners hd/2 + 8s .. hd/2 + 8s+7: a
+// workgroup that owns one strip then holds both halves of 8 rotation pairs.  v heads keep their order.
+//
+// One workgroup of 4 wavefronts a strip: the wavefronts take a quarter of the columns each (x straight from
+// global memory into the B operand: at most 16 tokens, so one tile), add their results through LDS, and the
+// first wavefront rotates and writes: queries to q_out [token][head][d], keys and values into the cache pages
+// in the matrix cores' order (common.h: key_index, value_index).
+// theta = pos * inv_freq[c]; (a, b) = (x[c], x[c+hd/2]) -> (a cos - b sin, a sin + b cos), cos and sin times
+// `mscale` (reference: src/model/rotary.cuh:7-34; cache rows src/model/attn.cuh:14-21; the fused decode
+// projection src/model/minicpm4/minicpm4_attn.cuh:209-223).
+#include "common.h"
+
+typedef __bf16 qbf16x8_t __attribute__((ext_vector_type(8)));
+typedef float qfloatx4_t __attribute__((ext_vector_type(4)));
+
+template <int PF, int NW>  // 128-column blocks of the weight a wavefront keeps in flight; wavefronts a workgroup
+__global__ __launch_bounds__(NW * 64) void qkv_rope_kernel(
+    const bf16_t* __restrict__ X, long ldx, const bf16_t* __restrict__ W, int M, int K, bf16_t* __restrict__ q_out,
+    int nh, int nkv, int hd, const int* __restrict__ positions, const int* __restrict__ tok_slot,
+    const float* __restrict__ inv_freq, float mscale, bf16_t* __restrict__ kpool, bf16_t* __restrict__ vpool,
+    PagedView pv) {
+    __shared__ float red[NW - 1][4][64];
+    const int strip = blockIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+    const int nkb = (K + 127) / 128;
+    const int per_wave = (nkb + NW - 1) / NW;
+    const int kb0 = wave * per_wave, kb1 = min(kb0 + per_wave, nkb);
+    const bf16_t* wp = W + (long)strip * nkb * 2048 + lane * 8;
+    const bf16_t* xp = X + (long)min(r, M - 1) * ldx + g * 8;       // rows beyond the step repeat its last token
+
+    qbf16x8_t a[PF][4];
+    auto load_w = [&](int kb, qbf16x8_t (&dst)[4]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            qbf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (kb < kb1) v = __builtin_nontemporal_load((const qbf16x8_t*)(wp + ((long)kb * 4 + i) * 512));
+            dst[i] = v;
+        }
+    };
+    auto load_x = [&](int kb, qbf16x8_t (&dst)[4]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            qbf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (kb < kb1 && kb * 128 + i * 32 + g * 8 < K) v = *(const qbf16x8_t*)(xp + (long)kb * 128 + i * 32);
+            dst[i] = v;
+        }
+    };
+#pragma unroll
+    for (int j = 0; j < PF; ++j) load_w(kb0 + j, a[j]);
+    qfloatx4_t acc = {0.f, 0.f, 0.f, 0.f};
+    for (int kb = kb0; kb < kb1; kb += PF) {
+#pragma unroll
+        for (int j = 0; j < PF; ++j) {
+            qbf16x8_t b[4];
+            load_x(kb + j, b);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j][i], b[i], acc, 0, 0, 0);
+            load_w(kb + j + PF, a[j]);
+        }
+    }
+    // lane (token r, g): acc[i] is feature row 4g + i of the strip; the other wavefronts hand theirs to the first
+    if (wave > 0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) red[wave - 1][i][lane] = acc[i];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int w = 0; w < NW - 1; ++w) acc[i] += red[w][i][lane];
+
+    const int spt = hd / 16;                       // strips a head
+    const int head = strip / spt, s = strip - head * spt;
+    const bool tok_ok = r < M;
+    const int pos = positions[min(r, M - 1)];
+    if (head < nh + nkv) {
+        // rows 0..7 of the strip are d = 8s .. 8s+7, rows 8..15 their partners d + hd/2: lanes g and g+2 hold a
+        // pair; after the swap every lane has both (the first half of the wavefront's value, then the second's)
+        float lo[4], hi[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const cpmcu_u32x2_t sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc[i]), __float_as_uint(acc[i]), false, false);
+            lo[i] = __uint_as_float(sw[0]);
+            hi[i] = __uint_as_float(sw[1]);
+        }
+        const bool second = g >= 2;
+        bf16_t* dst = nullptr;
+        bool is_q = head < nh;
+        if (tok_ok) {
+            if (is_q) dst = q_out + ((long)r * nh + head) * hd;
+            else dst = kpool + key_index(paged_row(pv, tok_slot[r], pos), head - nh, nkv, hd);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = 8 * s + 4 * (g & 1) + i;             // index of the pair
+            float cs = 1.f, sn = 0.f;
+            if (inv_freq) {
+                const float ang = (float)pos * inv_freq[c];
+                cs = cosf(ang) * mscale;
+                sn = sinf(ang) * mscale;
+            }
+            const float v = second ? lo[i] * sn + hi[i] * cs : lo[i] * cs - hi[i] * sn;
+            const int d = second ? c + hd / 2 : c;
+            if (tok_ok) dst[is_q ? d : key_d_offset(d)] = f32_to_bf16(v);
+        }
+    } else if (tok_ok) {
+        bf16_t* dst = vpool + value_index(paged_row(pv, tok_slot[r], pos), head - nh - nkv, nkv, hd);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dst[value_d_offset(16 * s + 4 * g + i)] = f32_to_bf16(acc[i]);
+    }
+}
+
+extern "C" const char* cpmcu_qkv_rope(const void* X, long ldx, const void* W, int M, int K, void* q_out, int nh,
+                                      int nkv, int hd, const int* positions, const int* tok_slot,
+                                      const float* inv_freq, float mscale, void* kpool, void* vpool,
+                                      const int* page_table, int table_width, int page_size, hipStream_t stream) {
+    CPMCU_REQUIRE(M > 0 && M <= 16, "qkv_rope: %d tokens (1..16 are taken; more go through the split product)", M);
+    CPMCU_REQUIRE(nh > 0 && nkv > 0 && hd > 0 && hd % 16 == 0, "qkv_rope: bad shape heads=%d kv_heads=%d head_dim=%d", nh, nkv, hd);
+    CPMCU_REQUIRE(K > 0 && K % 8 == 0 && ldx % 8 == 0 && ldx >= K, "qkv_rope: K=%d, row stride %ld must be multiples of 8", K, ldx);
+    CPMCU_REQUIRE(((uintptr_t)X % 16 == 0) && ((uintptr_t)W % 16 == 0), "qkv_rope: operands must be 16-byte aligned");
+    CPMCU_REQUIRE(q_out && kpool && vpool && page_table && positions && tok_slot, "qkv_rope: null pointer");
+    CPMCU_REQUIRE(page_size % 32 == 0, "qkv_rope: a cache page of %d tokens is not a multiple of 32", page_size);
+    PagedView pv{page_table, table_width, page_size};
+    const int strips = (nh + 2 * nkv) * (hd / 16);
+    qkv_rope_kernel<4, 4><<<strips, 256, 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, M, K, (bf16_t*)q_out, nh,
+                                                   nkv, hd, positions, tok_slot, inv_freq, mscale, (bf16_t*)kpool,
+                                                   (bf16_t*)vpool, pv);
+    CPMCU_LAUNCH_CHECK("qkv_rope");
+    return nullptr;
+}

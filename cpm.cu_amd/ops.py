@@ -392,6 +392,46 @@ class TiledWeight:
         self.N, self.K = N, K
 
 
+QKV_ROPE_MAX_ROWS = 16
+
+
+def qkv_rope_weight(w: torch.Tensor, nh: int, nkv: int, hd: int) -> TiledWeight:
+    """The stacked [q heads; k heads; v heads] x hidden weight for qkv_rope: tiled, the rows of every q and k head
+    in the order (8s .. 8s+7, hd/2 + 8s .. hd/2 + 8s+7 for s = 0, 1, ...), so that a strip of 16 rows holds
+    both halves of 8 rotation pairs; v heads keep their order."""
+    _need(w, "qkv weight", torch.bfloat16, ((nh + 2 * nkv) * hd, None))
+    if hd % 16:
+        raise KernelError(f"qkv_rope: head_dim {hd} is no multiple of 16")
+    s = torch.arange(hd // 16).view(-1, 1, 1)
+    order = (8 * s + torch.tensor([0, hd // 2]).view(1, 2, 1) + torch.arange(8).view(1, 1, 8)).reshape(-1)
+    rows = torch.arange((nh + 2 * nkv) * hd).view(nh + 2 * nkv, hd)
+    rows[:nh + nkv] = rows[:nh + nkv, :1] + order
+    return TiledWeight(w[rows.reshape(-1).to(w.device)])
+
+
+def qkv_rope(x: torch.Tensor, w: TiledWeight, q_out: torch.Tensor, nh: int, nkv: int, hd: int,
+             positions: torch.Tensor, tok_slot: torch.Tensor, inv_freq: Optional[torch.Tensor], mscale: float,
+             kpool: torch.Tensor, vpool: torch.Tensor, page_table: torch.Tensor, page_size: int):
+    """q, k, v = x . w^T for a step of at most 16 tokens, rotated (inv_freq None: not) and written: q to q_out
+    [n, nh*hd], k and v into the paged cache.  w from qkv_rope_weight."""
+    _need(x, "qkv x", torch.bfloat16, (None, w.K))
+    n = x.shape[0]
+    if w.N != (nh + 2 * nkv) * hd:
+        raise KernelError(f"qkv_rope: weight of {w.N} rows, {(nh + 2 * nkv) * hd} expected")
+    _need(q_out, "qkv q_out", torch.bfloat16, (n, nh * hd))
+    _need(positions, "qkv positions", torch.int32, (n,))
+    _need(tok_slot, "qkv token slots", torch.int32, (n,))
+    if inv_freq is not None:
+        _need(inv_freq, "qkv inv_freq", torch.float32, (hd // 2,))
+    _need(kpool, "qkv key pool", torch.bfloat16, (None, page_size, nkv * hd))
+    _need(vpool, "qkv value pool", torch.bfloat16, tuple(kpool.shape))
+    _need(page_table, "qkv page table", torch.int32, (None, None))
+    _check(_fn("qkv", "cpmcu_qkv_rope")(_p(x), c_long(x.stride(0)), _p(w.data), c_int(n), c_int(w.K), _p(q_out),
+                                        c_int(nh), c_int(nkv), c_int(hd), _p(positions), _p(tok_slot), _p(inv_freq),
+                                        c_float(mscale), _p(kpool), _p(vpool), _p(page_table),
+                                        c_int(page_table.shape[1]), c_int(page_size), _stream()))
+
+
 def gemm_skinny(x: torch.Tensor, w, out: torch.Tensor, alpha: float = 1.0, mode: str = "plain"):
     """bf16 product for at most 64 rows of x on the matrix cores, streaming w once; w is [N, K] as in the
     checkpoint or a TiledWeight.

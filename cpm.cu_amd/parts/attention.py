@@ -47,6 +47,7 @@ class GQAAttention(Mixer):
 
     def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime):
         self.rt = rt
+        self._qkv_fused = None               # the q/k/v weight re-laid for the fused decode kernel, made at first use
 
     def cache_needs(self) -> CacheNeeds:
         w = self.nkv * self.hd
@@ -57,6 +58,17 @@ class GQAAttention(Mixer):
         n = h.shape[0]
         nh, nkv, hd = self.nh, self.nkv, self.hd
         plain_rotation = self.position is None or self.position.rotary_params() is not None
+        if (writes_cache and plain_rotation and n <= ops.QKV_ROPE_MAX_ROWS and h.dtype == torch.bfloat16
+                and self.qkv.tiled is not None and hd % 16 == 0 and cache.page_size % 32 == 0):
+            # decode steps: projection, rotation and cache write in one kernel (one kernel of the chain less)
+            if self._qkv_fused is None:
+                self._qkv_fused = ops.qkv_rope_weight(self.qkv.weight, nh, nkv, hd)
+            rot = self.position.rotary_params() if self.position is not None else None
+            inv_freq, mag = (rot if rot is not None else (None, 1.0))
+            q = ctx.ws.get("attn.q", (n, nh * hd), self.rt.dtype)
+            ops.qkv_rope(h, self._qkv_fused, q, nh, nkv, hd, ctx.positions, ctx.tok_slot, inv_freq, mag,
+                         cache.streams["k"], cache.streams["v"], cache.page_table, cache.page_size)
+            return q
         qkv = self.qkv.forward(h, ctx, "attn.qkv", rows=None if writes_cache else nh * hd, partials=plain_rotation)
         rot = self.position.rotary_params() if self.position is not None else None
         inv_freq, mag = (rot if rot is not None else (None, 1.0))

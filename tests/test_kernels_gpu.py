@@ -424,6 +424,58 @@ def test_block_lists_of_a_prompt_chunk_in_any_visiting_order(first):
     assert float((out.double().cpu().view(n, nh, hd) - ref).abs().max()) <= 2 ** -7
 
 
+# ---------------------------------------------------------------------------- fused projection of decode steps
+def read_cache_rows(pool, table, page, nkv, hd, slot, positions, tiles):
+    """Rows [position][kv head][d] out of a paged pool whose pages lie as `tiles` (key_tiles / value_tiles) lays them."""
+    probe = torch.arange(page * nkv * hd, dtype=torch.float64).view(page, nkv, hd)
+    where = tiles(probe).reshape(-1).long()                      # flat place -> (token, kv head, d) index
+    inv = torch.empty_like(where)
+    inv[where] = torch.arange(where.numel())
+    out = []
+    for p in positions:
+        flat = pool[int(table[slot, p // page])].reshape(-1).cpu()
+        out.append(flat[inv.view(page, nkv, hd)[p % page]])
+    return torch.stack(out)
+
+
+@pytest.mark.parametrize("n,nh,nkv,hd,H,rotate", [(1, 4, 2, 16, 64, True), (8, 32, 2, 128, 512, True), (16, 3, 1, 32, 96, True),
+                                                  (5, 6, 3, 64, 200, False), (13, 2, 2, 48, 264, True)])
+def test_fused_projection_rotation_and_cache_write(n, nh, nkv, hd, H, rotate):
+    """q, k, v of a decode step in one kernel: against the float64 product, rotation (pairs c, c + hd/2) and the
+    cache rows read back through the pages' layout; tokens of several slots at scattered positions."""
+    from cpmcu_amd import ops
+    page = 64
+    w = rnd((nh + 2 * nkv) * hd, H, seed=1, dtype=torch.bfloat16, scale=H ** -0.5)
+    x = rnd(n, H, seed=2, dtype=torch.bfloat16)
+    g = torch.Generator().manual_seed(n)
+    slots = torch.randint(0, 3, (n,), generator=g)
+    positions = torch.randperm(190, generator=g)[:n]             # distinct, so no two tokens share a cache row
+    table = torch.randperm(12, generator=g)[:9].view(3, 3).to(torch.int32)
+    inv_freq = (torch.rand(hd // 2, generator=g) * 0.5 + 0.01) if rotate else None
+    mscale = 1.25
+    kpool = torch.zeros(12, page, nkv * hd, dtype=torch.bfloat16, device=DEV)
+    vpool = torch.zeros_like(kpool)
+    q_out = torch.empty(n, nh * hd, dtype=torch.bfloat16, device=DEV)
+    wt = ops.qkv_rope_weight(w, nh, nkv, hd)
+    ops.qkv_rope(x, wt, q_out, nh, nkv, hd, positions.to(torch.int32).to(DEV), slots.to(torch.int32).to(DEV),
+                 inv_freq.to(DEV) if rotate else None, mscale if rotate else 1.0, kpool, vpool, table.to(DEV), page)
+    y = (x.double().cpu() @ w.double().cpu().T).view(n, nh + 2 * nkv, hd)
+    if rotate:
+        ang = positions.double()[:, None] * inv_freq.float().double()[None, :]          # angles formed in float32 on the GPU
+        cs, sn = (torch.cos(ang) * mscale)[:, None, :], (torch.sin(ang) * mscale)[:, None, :]
+        a, b = y[:, :nh + nkv, :hd // 2], y[:, :nh + nkv, hd // 2:]
+        y[:, :nh + nkv] = torch.cat([a * cs - b * sn, a * sn + b * cs], dim=-1)
+    tol = 2 ** -7 * max(1.0, float(y.abs().max()))
+    assert float((q_out.double().cpu().view(n, nh, hd) - y[:, :nh]).abs().max()) <= tol
+    for t in range(n):
+        k_row = read_cache_rows(kpool, table, page, nkv, hd, int(slots[t]), [int(positions[t])], key_tiles)[0]
+        v_row = read_cache_rows(vpool, table, page, nkv, hd, int(slots[t]), [int(positions[t])], value_tiles)[0]
+        assert float((k_row.double() - y[t, nh:nh + nkv]).abs().max()) <= tol, t
+        assert float((v_row.double() - y[t, nh + nkv:]).abs().max()) <= tol, t
+    # nothing but the n rows was written
+    assert int((kpool != 0).sum()) <= n * nkv * hd and int((vpool != 0).sum()) <= n * nkv * hd
+
+
 # ---------------------------------------------------------------------------- InfLLM-v2 kernels
 @pytest.mark.parametrize("ks,st", [(8, 4), (32, 16), (16, 16), (12, 4)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
