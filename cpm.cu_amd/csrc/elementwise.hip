@@ -258,47 +258,145 @@ __global__ void rope_store_kernel(const IT* __restrict__ qkv, long width, int np
                                   T* __restrict__ q_out, int nh, int nkv, int hd, const int* __restrict__ positions,
                                   const int* __restrict__ tok_slot, const float* __restrict__ inv_freq, float mscale,
                                   T* __restrict__ kpool, T* __restrict__ vpool, PagedView pv, int write_kv) {
-    // 64 threads per (token, head): heads [0, nh) are queries, then nkv key heads, then nkv value heads;
-    // a block holds blockDim.x / 64 heads of one token
+    // 64 threads a (token, head) at a time: heads [0, nh) are queries, then nkv key heads, then nkv value heads.
+    // The groups of 64 threads of the token's blocks take its heads in turn; a group forms the angles' cos and
+    // sin once (they are the same for every head) and keeps them for the pairs c = lane and lane + 64.
     const long t = blockIdx.x;
-    const int head = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int groups = gridDim.y * (blockDim.x >> 6);
+    const int group = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
-    if (head >= nh + (write_kv ? 2 * nkv : 0)) return;
+    const int heads = nh + (write_kv ? 2 * nkv : 0);
+    if (group >= heads) return;
     const int half = hd / 2;
     const int pos = positions[t];
-    const IT* row = qkv + t * width + (long)head * hd;
-    auto load = [&](int i) {
-        float s = 0.f;
-        for (int p = 0; p < nparts; ++p) s += to_f32(row[p * part_stride + i]);
-        return s;
+    auto trig = [&](int c, float& cs, float& sn) {
+        cs = 1.f;
+        sn = 0.f;
+        if (inv_freq && c < half) {
+            const float ang = (float)pos * inv_freq[c];
+            cs = cosf(ang) * mscale;
+            sn = sinf(ang) * mscale;
+        }
     };
-    long kv_row = 0;
-    if (head >= nh) kv_row = paged_row(pv, tok_slot[t], pos);
-    if (head < nh + nkv) {
-        // queries go out as plain rows; keys into their page in the matrix cores' order (key_index)
-        const bool is_q = head < nh;
-        T* dst = q_out;
-        if (is_q) {
-            dst = q_out + (t * nh + head) * (long)hd;
-        } else {
-            dst = kpool + key_index(kv_row, head - nh, nkv, hd);
-        }
-        auto at = [&](int d) { return is_q ? d : key_d_offset(d); };
-        for (int c = lane; c < half; c += 64) {
-            float cs = 1.f, sn = 0.f;
-            if (inv_freq) {
-                const float ang = (float)pos * inv_freq[c];
-                cs = cosf(ang) * mscale;
-                sn = sinf(ang) * mscale;
+    float cs0, sn0, cs1, sn1;
+    trig(lane, cs0, sn0);
+    trig(lane + 64, cs1, sn1);
+    const long kv_row = write_kv ? paged_row(pv, tok_slot[t], pos) : 0;
+    for (int head = group; head < heads; head += groups) {
+        const IT* row = qkv + t * width + (long)head * hd;
+        auto load = [&](int i) {
+            float s = 0.f;
+            for (int p = 0; p < nparts; ++p) s += to_f32(row[p * part_stride + i]);
+            return s;
+        };
+        if (head < nh + nkv) {
+            // queries go out as plain rows; keys into their page in the matrix cores' order (key_index)
+            const bool is_q = head < nh;
+            T* dst = is_q ? q_out + (t * nh + head) * (long)hd : kpool + key_index(kv_row, head - nh, nkv, hd);
+            auto at = [&](int d) { return is_q ? d : key_d_offset(d); };
+            for (int c = lane; c < half; c += 64) {
+                float cs = cs0, sn = sn0;
+                if (c >= 64) {
+                    cs = cs1;
+                    sn = sn1;
+                }
+                if (c >= 128) trig(c, cs, sn);
+                const float a = load(c), b = load(c + half);
+                dst[at(c)] = from_f32<T>(a * cs - b * sn);
+                dst[at(c + half)] = from_f32<T>(a * sn + b * cs);
             }
-            const float a = load(c), b = load(c + half);
-            dst[at(c)] = from_f32<T>(a * cs - b * sn);
-            dst[at(c + half)] = from_f32<T>(a * sn + b * cs);
+        } else {
+            // values go into their page transposed, in the matrix cores' order (value_index)
+            T* dst = vpool + value_index(kv_row, head - nh - nkv, nkv, hd);
+            for (int d = lane; d < hd; d += 64) dst[value_d_offset(d)] = from_f32<T>(load(d));
         }
-    } else {
-        // values go into their page transposed, in the matrix cores' order (value_index)
-        T* dst = vpool + value_index(kv_row, head - nh - nkv, nkv, hd);
-        for (int d = lane; d < hd; d += 64) dst[value_d_offset(d)] = from_f32<T>(load(d));
+    }
+}
+
+// The same for steps of many tokens in bf16 (one input slice): 16-byte accesses.  A block takes 8 tokens; lane
+// (token, piece) of a wavefront owns the 8 rotation pairs c = 8 piece .. 8 piece + 7 of its token, forms their
+// cos and sin once and applies them to every head the wavefront takes (every fourth); values are written by
+// a thread a (kv head, d) for the block's 8 tokens.  head_dim is a multiple of 16, at most 128.
+typedef __bf16 ebf16x8_t __attribute__((ext_vector_type(8)));
+__global__ __launch_bounds__(256) void rope_store_rows_kernel(
+    const bf16_t* __restrict__ qkv, long width, bf16_t* __restrict__ q_out, int n, int nh, int nkv, int hd,
+    const int* __restrict__ positions, const int* __restrict__ tok_slot, const float* __restrict__ inv_freq,
+    float mscale, bf16_t* __restrict__ kpool, bf16_t* __restrict__ vpool, PagedView pv, int write_kv) {
+    __shared__ long rows_s[8];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int half = hd / 2, pieces = half / 8;           // pieces <= 8
+    if (threadIdx.x < 8) {
+        const long tk = (long)blockIdx.x * 8 + threadIdx.x;
+        rows_s[threadIdx.x] = (write_kv && tk < n) ? paged_row(pv, tok_slot[tk], positions[tk]) : -1;
+    }
+    const long t = (long)blockIdx.x * 8 + (lane >> 3);
+    const int piece = lane & 7;
+    const bool mine = t < n && piece < pieces;
+    float cs[8], sn[8];
+    if (mine) {
+        const int pos = positions[t];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            cs[e] = 1.f;
+            sn[e] = 0.f;
+            if (inv_freq) {
+                const float ang = (float)pos * inv_freq[8 * piece + e];
+                cs[e] = cosf(ang) * mscale;
+                sn[e] = sinf(ang) * mscale;
+            }
+        }
+    }
+    __syncthreads();
+    if (mine) {
+        const long kv_row = rows_s[lane >> 3];
+        const int heads = nh + (write_kv ? nkv : 0);
+        const bf16_t* row = qkv + t * width + 8 * piece;
+        // three heads' loads in flight at a time (a head beyond the last asks for the last once more)
+        for (int head0 = wave; head0 < heads; head0 += 12) {
+            ebf16x8_t a[3], b[3];
+#pragma unroll
+            for (int u = 0; u < 3; ++u) {
+                const int head = min(head0 + 4 * u, heads - 1);
+                a[u] = *(const ebf16x8_t*)(row + (long)head * hd);
+                b[u] = *(const ebf16x8_t*)(row + (long)head * hd + half);
+            }
+#pragma unroll
+            for (int u = 0; u < 3; ++u) {
+                const int head = head0 + 4 * u;
+                if (head >= heads) break;
+                ebf16x8_t lo, hi;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float x = (float)a[u][e], y = (float)b[u][e];
+                    lo[e] = (__bf16)(x * cs[e] - y * sn[e]);
+                    hi[e] = (__bf16)(x * sn[e] + y * cs[e]);
+                }
+                if (head < nh) {
+                    bf16_t* dst = q_out + (t * nh + head) * (long)hd + 8 * piece;
+                    *(ebf16x8_t*)dst = lo;
+                    *(ebf16x8_t*)(dst + half) = hi;
+                } else {
+                    // d = 8 piece + e lies at key_d_offset = piece * 128 + e: one 16-byte piece
+                    bf16_t* dst = kpool + key_index(kv_row, head - nh, nkv, hd);
+                    *(ebf16x8_t*)(dst + piece * 128) = lo;
+                    *(ebf16x8_t*)(dst + (piece + pieces) * 128) = hi;
+                }
+            }
+        }
+    }
+    if (!write_kv) return;
+    // values: thread (kv head, d), the block's 8 tokens one after the other
+    for (int e = threadIdx.x; e < nkv * hd; e += 256) {
+        const int kvh = e / hd, d = e - kvh * hd;
+        bf16_t v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const long tk = min((long)blockIdx.x * 8 + k, (long)n - 1);
+            v[k] = qkv[tk * width + (long)(nh + nkv + kvh) * hd + d];
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            if (rows_s[k] >= 0) vpool[value_index(rows_s[k], kvh, nkv, hd) + value_d_offset(d)] = v[k];
     }
 }
 
@@ -319,12 +417,20 @@ extern "C" const char* cpmcu_rope_store(const void* qkv, long row_width, int in_
                   "rope_store: a row of %ld elements cannot hold %d query%s heads of %d", row_width, nh,
                   write_kv ? " and key/value" : "", hd);
     PagedView pv{page_table, table_width, page_size};
-    // few tokens (decode steps): a block a head, for more blocks; many: 4 heads a block
+    if (n >= 64 && in_dtype == CPMCU_BF16 && dtype == CPMCU_BF16 && nparts == 1 && hd % 16 == 0 && hd <= 128 &&
+        row_width % 8 == 0 && ((uintptr_t)qkv % 16 == 0) && ((uintptr_t)q_out % 16 == 0)) {
+        rope_store_rows_kernel<<<(n + 7) / 8, 256, 0, stream>>>((const bf16_t*)qkv, row_width, (bf16_t*)q_out, n, nh, nkv,
+                                                                hd, positions, tok_slot, inv_freq, mscale,
+                                                                (bf16_t*)kpool, (bf16_t*)vpool, pv, write_kv);
+        CPMCU_LAUNCH_CHECK("rope_store_rows");
+        return nullptr;
+    }
+    // few tokens (decode steps): a block a head, for more blocks; many: one block of 4 groups a token, each
+    // group taking every fourth head with the same cos and sin
     const int heads = nh + (write_kv ? 2 * nkv : 0);
-    const int hpb = n >= 64 ? 4 : 1;
-    const int block = 64 * hpb;
+    const int block = n >= 64 ? 256 : 64;
     CPMCU_REQUIRE(heads <= 65535, "rope_store: %d heads exceed the launch grid", heads);
-    dim3 grid(n, (heads + hpb - 1) / hpb);
+    dim3 grid(n, n >= 64 ? 1 : heads);
 #define LAUNCH(IT, T)                                                                                          \
     rope_store_kernel<IT, T><<<grid, block, 0, stream>>>((const IT*)qkv, row_width, nparts, part_stride, (T*)q_out, nh, nkv, \
                                                       hd, positions, tok_slot, inv_freq, mscale, (T*)kpool,   \

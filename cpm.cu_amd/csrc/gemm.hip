@@ -199,12 +199,12 @@ if (TILED) {
         if (c + 1 < nchunk) load_x(c + 1);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
+            // consecutive matrix instructions go to different accumulators (tiles of rows, then strips)
 #pragma unroll
-            for (int t = 0; t < MT; ++t) {
-                const bf16_t* xrow = xs + (t * 16 + r) * SK_XS + j * 128 + g * 8;
+            for (int i = 0; i < 4; ++i) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const bf16x8_t b = *(const bf16x8_t*)(xrow + i * 32);
+                for (int t = 0; t < MT; ++t) {
+                    const bf16x8_t b = *(const bf16x8_t*)(xs + (t * 16 + r) * SK_XS + j * 128 + g * 8 + i * 32);
 #pragma unroll
                     for (int s = 0; s < SPW; ++s)
                         acc[s][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j][s][i], b, acc[s][t], 0, 0, 0);

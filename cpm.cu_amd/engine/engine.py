@@ -64,6 +64,9 @@ class Engine:
         if not torch.cuda.is_available():
             raise RuntimeError("no GPU is visible: the engine's kernels cannot run")
         self.dtype = _DTYPES[options.dtype]
+        if options.page_size <= 0 or options.page_size % 32:
+            raise ValueError(f"page_size {options.page_size}: the cache kernels lay a page out in chunks of 32 tokens; "
+                             f"give a positive multiple of 32")
         max_seq_len = options.max_seq_len or getattr(config, "max_position_embeddings", None) or options.max_tokens
         self.max_seq_len = int(max_seq_len)
         self.workspace = Workspace(self.device)

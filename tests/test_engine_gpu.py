@@ -187,6 +187,8 @@ def test_steps_that_cannot_run_are_refused_and_change_nothing(model_dirs):
     assert eng.step([StepEntry(s, [1, 2, 3], [])]) is None and eng.length(s) == 3
     eng.release(s)
     eng.cache.check()
+    with pytest.raises(ValueError, match="multiple of 32"):
+        engine_for(model_dirs, "A", "float32", page_size=48)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
