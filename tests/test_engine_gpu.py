@@ -233,3 +233,41 @@ def test_overlapped_generation_loop_equals_the_plain_loop(model_dirs, references
     plain_loop = run(gen._run_batch, stops)
     assert any(r == "stop" for _, r in plain_loop) and any(r == "length" for _, r in plain_loop)
     assert run(gen._run_batch_overlapped, stops) == plain_loop
+
+
+ODD = {
+    # head size 48 (no matrix-core attention kernel: the plain one runs), 5 query heads a kv head, sizes that are
+    # multiples of 8 but of nothing more
+    "hd48": dict(num_hidden_layers=2, hidden_size=200, num_attention_heads=10, num_key_value_heads=2, head_dim=48,
+                 intermediate_size=344, vocab_size=777, rms_norm_eps=3e-6, rope_theta=7000.0, max_position_embeddings=192,
+                 scale_emb=3, dim_model_base=100, scale_depth=2.0, tie_word_embeddings=False),
+    # every query head its own kv head, head size 80, an intermediate size that is no multiple of 8 (the products
+    # over it take the plain kernel), an odd vocabulary
+    "mha80": dict(num_hidden_layers=1, hidden_size=72, num_attention_heads=6, num_key_value_heads=6, head_dim=80,
+                  intermediate_size=100, vocab_size=1001, rms_norm_eps=1e-5, rope_theta=10000.0,
+                  max_position_embeddings=192, scale_emb=1, dim_model_base=72, scale_depth=1.0, tie_word_embeddings=True),
+    # block-sparse attention with 5 query heads on one kv head and blocks of 32
+    "sparse5": dict(num_hidden_layers=2, hidden_size=160, num_attention_heads=5, num_key_value_heads=1, head_dim=32,
+                    intermediate_size=208, vocab_size=300, rms_norm_eps=1e-6, rope_theta=20000.0,
+                    max_position_embeddings=192, scale_emb=2, dim_model_base=80, scale_depth=1.0,
+                    tie_word_embeddings=True,
+                    sparse_config={"kernel_size": 16, "kernel_stride": 8, "block_size": 32, "init_blocks": 1, "topk": 2,
+                                   "window_size": 32, "dense_len": 40}),
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(ODD))
+def test_sizes_that_are_no_power_of_two(tmp_path, name, dtype):
+    """Whole, and the last 20 tokens one by one, against the plain implementation, at sizes the two tiny
+    configurations do not have."""
+    from cpmcu_amd import Engine, EngineOptions
+    raw = dict(architectures=["MiniCPMForCausalLM"], model_type="minicpm", hidden_act="silu", **ODD[name])
+    d = tiny.write_model(raw, str(tmp_path / name), seed=len(name), norm_std=0.1)
+    cfg, w = tiny.read_model(d)
+    reqs = {"x": tiny.random_tokens(150, raw["vocab_size"], 5), "y": tiny.random_tokens(37, raw["vocab_size"], 6)}
+    refs = {r: plain.forward(cfg, w, t).float() for r, t in reqs.items()}
+    eng = Engine.from_dir(d, EngineOptions(dtype=dtype, max_tokens=512, max_slots=2))
+    check(schedules.whole(eng, reqs), refs, dtype, f"{name} whole")
+    check(schedules.tail(eng, reqs, 20), refs, dtype, f"{name} tail-20")
+    eng.cache.check()
