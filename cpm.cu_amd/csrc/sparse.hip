@@ -394,7 +394,8 @@ __global__ __launch_bounds__(NW * 64) void sparse_select_mfma_kernel(
     float* work = score + (sp.max_ck + 3) / 4 * 4;
 
     const int t = blockIdx.x, kvh = blockIdx.y, tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63, n = lane & 15, g = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63, n = lane & 15, g = lane >> 4;
     const int p = positions[t];
     const long out_idx = (long)t * sp.nkv + kvh;
     if (p + 1 <= sp.dense_len) {
@@ -425,36 +426,54 @@ __global__ __launch_bounds__(NW * 64) void sparse_select_mfma_kernel(
             if (head_ok && d < HD) v = *(const sbf16x8_t*)(q + ((long)t * sp.nh + (long)kvh * G + ht * 16 + n) * HD + d);
             qf[ks] = v;
         }
-        auto scores_of_tile = [&](int tile) {
-            // B operand: lane (key n, g) holds CK[key][32*ks + 8g .. +8]
+        // The wavefront's tiles of 16 compressed keys in turn, f(tile, scores).  B operand: lane (key n, g) holds
+        // CK[key][32*ks + 8g .. +8].  A tile's page is looked up two tiles ahead and its keys are asked for one
+        // tile ahead, so that neither latency stands between two tiles' arithmetic.
+        auto page_of = [&](int tile) { return ptab[min(tile * 16 + n, n_vis - 1) / rows_per_page]; };
+        auto load_b = [&](int tile, int page, sbf16x8_t (&b)[KSTEPS]) {
             const int j = min(tile * 16 + n, n_vis - 1);
-            const int first = sp.st * j;
-            const int page = ptab[first / pv.page_size];
-            const bf16_t* ck = ckpool + ck_index(page, (first % pv.page_size) / sp.st, kvh, sp.nkv, HD, rows_per_page) +
+            const bf16_t* ck = ckpool + ck_index(page, j % rows_per_page, kvh, sp.nkv, HD, rows_per_page) +
                                g * rows_per_page * 8;
-            sfloatx4_t st = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ks = 0; ks < KSTEPS; ++ks) {
-                sbf16x8_t b = {0, 0, 0, 0, 0, 0, 0, 0};
-                if (ks * 32 + g * 8 < HD) b = *(const sbf16x8_t*)(ck + ks * 4 * rows_per_page * 8);
-                st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ks], b, st, 0, 0, 0);
+                sbf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+                if (ks * 32 + g * 8 < HD) v = *(const sbf16x8_t*)(ck + ks * 4 * rows_per_page * 8);
+                b[ks] = v;
             }
-            return st;                      // st[i]: head 4g+i (of this head tile) x key tile*16+n
+        };
+        auto for_tiles = [&](auto f) {
+            if (wave >= n_tiles) return;
+            sbf16x8_t b[KSTEPS], bn[KSTEPS];
+            load_b(wave, page_of(wave), b);
+            int page_next = page_of(wave + NW);               // (tiles beyond the last repeat the last key)
+            for (int tile = wave; tile < n_tiles; tile += NW) {
+                const int page_after = page_of(tile + 2 * NW);
+                load_b(tile + NW, page_next, bn);
+                sfloatx4_t st = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < KSTEPS; ++ks) st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ks], b[ks], st, 0, 0, 0);
+                f(tile, st);                    // st[i]: head 4g+i (of this head tile) x key tile*16+n
+#pragma unroll
+                for (int ks = 0; ks < KSTEPS; ++ks) b[ks] = bn[ks];
+                page_next = page_after;
+            }
         };
         // pass 1: running max and sum per head, per lane
         float m[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY}, l[4] = {0.f, 0.f, 0.f, 0.f};
-        for (int tile = wave; tile < n_tiles; tile += NW) {
-            const sfloatx4_t st = scores_of_tile(tile);
+        for_tiles([&](int tile, const sfloatx4_t& st) {
             if (tile * 16 + n < n_vis) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
+                    // one exponential an element: of the two terms of the running sum, the one that belongs to
+                    // the larger of (old max, new score) has weight 1 (the bare hardware exponential: its
+                    // argument is <= 0, and what underflows adds nothing)
                     const float s = st[i] * scale_log2e;
-                    const float m_new = fmaxf(m[i], s);
-                    l[i] = l[i] * exp2f(m[i] - m_new) + exp2f(s - m_new);
-                    m[i] = m_new;
+                    const float e = __builtin_amdgcn_exp2f(-fabsf(s - m[i]));
+                    l[i] = s > m[i] ? l[i] * e + 1.0f : l[i] + e;
+                    m[i] = fmaxf(m[i], s);
                 }
             }
-        }
+        });
         // merge over the 16 key lanes of a group, then over the wavefronts
 #pragma unroll
         for (int off = 1; off < 16; off <<= 1) {
@@ -492,17 +511,15 @@ __global__ __launch_bounds__(NW * 64) void sparse_select_mfma_kernel(
             invL[i] = (ht * 16 + 4 * g + i < G && ll > 0.f) ? 1.0f / ll : 0.f;
         }
         // pass 2: normalised scores summed over the heads of the group
-        for (int tile = wave; tile < n_tiles; tile += NW) {
-            const sfloatx4_t st = scores_of_tile(tile);
+        for_tiles([&](int tile, const sfloatx4_t& st) {
             float v = 0.f;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                if (invL[i] > 0.f) v += exp2f(st[i] * scale_log2e - M[i]) * invL[i];
-            v += __shfl_xor(v, 16, 64);
-            v += __shfl_xor(v, 32, 64);
+                if (invL[i] > 0.f) v += __builtin_amdgcn_exp2f(__builtin_fmaf(st[i], scale_log2e, -M[i])) * invL[i];
+            v = rows_sum(v);
             const int j = tile * 16 + n;
             if (g == 0 && j < n_vis) score[j] += v;
-        }
+        });
     }
     __syncthreads();
     blocks_from_scores<NW>(score, work, wave_tot, sp, n_vis, q_block, n_cand, out_idx, sel_blocks, sel_count);
