@@ -425,12 +425,11 @@ extern "C" const char* cpmcu_rope_store(const void* qkv, long row_width, int in_
         CPMCU_LAUNCH_CHECK("rope_store_rows");
         return nullptr;
     }
-    // few tokens (decode steps): a block a head, for more blocks; many: one block of 4 groups a token, each
-    // group taking every fourth head with the same cos and sin
+    // few tokens (decode steps): a block a head, for more blocks; many: 4 heads a block
     const int heads = nh + (write_kv ? 2 * nkv : 0);
     const int block = n >= 64 ? 256 : 64;
     CPMCU_REQUIRE(heads <= 65535, "rope_store: %d heads exceed the launch grid", heads);
-    dim3 grid(n, n >= 64 ? 1 : heads);
+    dim3 grid(n, n >= 64 ? (heads + 3) / 4 : heads);
 #define LAUNCH(IT, T)                                                                                          \
     rope_store_kernel<IT, T><<<grid, block, 0, stream>>>((const IT*)qkv, row_width, nparts, part_stride, (T*)q_out, nh, nkv, \
                                                       hd, positions, tok_slot, inv_freq, mscale, (T*)kpool,   \
