@@ -1,4 +1,4 @@
-// q, k, v projection of a decode step fused with the rotation and the cache write (bf16, at most 16 tokens).
+// q, k, v projection of a decode step fused with the rotation and the cache write (bf16, at most 64 tokens).
 //
 // A decode step is a chain of small kernels, each of which costs a few microseconds whatever it does; this one
 // replaces the split-K product + the kernel that summed its partial sums, rotated and stored.
@@ -9,7 +9,7 @@
 // workgroup that owns one strip then holds both halves of 8 rotation pairs.  v heads keep their order.
 //
 // One workgroup of 4 wavefronts a strip: the wavefronts take a quarter of the columns each (x straight from
-// global memory into the B operand: at most 16 tokens, so one tile), add their results through LDS, and the
+// global memory into the B operand, one tile of 16 tokens after the other), add their results through LDS, and the
 // first wavefront rotates and writes: queries to q_out [token][head][d], keys and values into the cache pages
 // in the matrix cores' order (common.h: key_index, value_index).
 // theta = pos * inv_freq[c]; (a, b) = (x[c], x[c+hd/2]) -> (a cos - b sin, a sin + b cos), cos and sin times
@@ -20,13 +20,14 @@
 typedef __bf16 qbf16x8_t __attribute__((ext_vector_type(8)));
 typedef float qfloatx4_t __attribute__((ext_vector_type(4)));
 
-template <int PF, int NW>  // 128-column blocks of the weight a wavefront keeps in flight; wavefronts a workgroup
+// PF: 128-column blocks of the weight a wavefront keeps in flight; NW: wavefronts a workgroup; MT: tiles of 16 tokens
+template <int PF, int NW, int MT>
 __global__ __launch_bounds__(NW * 64) void qkv_rope_kernel(
     const bf16_t* __restrict__ X, long ldx, const bf16_t* __restrict__ W, int M, int K, bf16_t* __restrict__ q_out,
     int nh, int nkv, int hd, const int* __restrict__ positions, const int* __restrict__ tok_slot,
     const float* __restrict__ inv_freq, float mscale, bf16_t* __restrict__ kpool, bf16_t* __restrict__ vpool,
     PagedView pv) {
-    __shared__ float red[NW - 1][4][64];
+    __shared__ float red[NW - 1][MT][4][64];
     const int strip = blockIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
@@ -34,7 +35,9 @@ __global__ __launch_bounds__(NW * 64) void qkv_rope_kernel(
     const int per_wave = (nkb + NW - 1) / NW;
     const int kb0 = wave * per_wave, kb1 = min(kb0 + per_wave, nkb);
     const bf16_t* wp = W + (long)strip * nkb * 2048 + lane * 8;
-    const bf16_t* xp = X + (long)min(r, M - 1) * ldx + g * 8;       // rows beyond the step repeat its last token
+    const bf16_t* xp[MT];                                  // rows beyond the step repeat its last token
+#pragma unroll
+    for (int t = 0; t < MT; ++t) xp[t] = X + (long)min(t * 16 + r, M - 1) * ldx + g * 8;
 
     qbf16x8_t a[PF][4];
     auto load_w = [&](int kb, qbf16x8_t (&dst)[4]) {
@@ -45,77 +48,93 @@ __global__ __launch_bounds__(NW * 64) void qkv_rope_kernel(
             dst[i] = v;
         }
     };
-    auto load_x = [&](int kb, qbf16x8_t (&dst)[4]) {
+    auto load_x = [&](int kb, int t, qbf16x8_t (&dst)[4]) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             qbf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (kb < kb1 && kb * 128 + i * 32 + g * 8 < K) v = *(const qbf16x8_t*)(xp + (long)kb * 128 + i * 32);
+            if (kb < kb1 && kb * 128 + i * 32 + g * 8 < K) v = *(const qbf16x8_t*)(xp[t] + (long)kb * 128 + i * 32);
             dst[i] = v;
         }
     };
 #pragma unroll
     for (int j = 0; j < PF; ++j) load_w(kb0 + j, a[j]);
-    qfloatx4_t acc = {0.f, 0.f, 0.f, 0.f};
+    qfloatx4_t acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[t] = qfloatx4_t{0.f, 0.f, 0.f, 0.f};
     for (int kb = kb0; kb < kb1; kb += PF) {
 #pragma unroll
         for (int j = 0; j < PF; ++j) {
-            qbf16x8_t b[4];
-            load_x(kb + j, b);
+            qbf16x8_t b[MT][4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j][i], b[i], acc, 0, 0, 0);
+            for (int t = 0; t < MT; ++t) load_x(kb + j, t, b[t]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int t = 0; t < MT; ++t)
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j][i], b[t][i], acc[t], 0, 0, 0);
             load_w(kb + j + PF, a[j]);
         }
     }
-    // lane (token r, g): acc[i] is feature row 4g + i of the strip; the other wavefronts hand theirs to the first
+    // lane (token r, g) of tile t: acc[t][i] is feature row 4g + i of the strip; the other wavefronts hand theirs
+    // to the first
     if (wave > 0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) red[wave - 1][i][lane] = acc[i];
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[wave - 1][t][i][lane] = acc[t][i];
     }
     __syncthreads();
     if (wave > 0) return;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int t = 0; t < MT; ++t)
 #pragma unroll
-        for (int w = 0; w < NW - 1; ++w) acc[i] += red[w][i][lane];
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int w = 0; w < NW - 1; ++w) acc[t][i] += red[w][t][i][lane];
 
     const int spt = hd / 16;                       // strips a head
     const int head = strip / spt, s = strip - head * spt;
-    const bool tok_ok = r < M;
-    const int pos = positions[min(r, M - 1)];
-    if (head < nh + nkv) {
-        // rows 0..7 of the strip are d = 8s .. 8s+7, rows 8..15 their partners d + hd/2: lanes g and g+2 hold a
-        // pair; after the swap every lane has both (the first half of the wavefront's value, then the second's)
-        float lo[4], hi[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const cpmcu_u32x2_t sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc[i]), __float_as_uint(acc[i]), false, false);
-            lo[i] = __uint_as_float(sw[0]);
-            hi[i] = __uint_as_float(sw[1]);
-        }
-        const bool second = g >= 2;
-        bf16_t* dst = nullptr;
-        bool is_q = head < nh;
-        if (tok_ok) {
-            if (is_q) dst = q_out + ((long)r * nh + head) * hd;
-            else dst = kpool + key_index(paged_row(pv, tok_slot[r], pos), head - nh, nkv, hd);
-        }
+    for (int t = 0; t < MT; ++t) {
+        const int tok = t * 16 + r;
+        const bool tok_ok = tok < M;
+        const int pos = positions[min(tok, M - 1)];
+        if (head < nh + nkv) {
+            // rows 0..7 of the strip are d = 8s .. 8s+7, rows 8..15 their partners d + hd/2: lanes g and g+2 hold
+            // a pair; after the swap every lane has both (the first half of the wavefront's value, then the second's)
+            float lo[4], hi[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int c = 8 * s + 4 * (g & 1) + i;             // index of the pair
-            float cs = 1.f, sn = 0.f;
-            if (inv_freq) {
-                const float ang = (float)pos * inv_freq[c];
-                cs = cosf(ang) * mscale;
-                sn = sinf(ang) * mscale;
+            for (int i = 0; i < 4; ++i) {
+                const cpmcu_u32x2_t sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc[t][i]),
+                                                                          __float_as_uint(acc[t][i]), false, false);
+                lo[i] = __uint_as_float(sw[0]);
+                hi[i] = __uint_as_float(sw[1]);
             }
-            const float v = second ? lo[i] * sn + hi[i] * cs : lo[i] * cs - hi[i] * sn;
-            const int d = second ? c + hd / 2 : c;
-            if (tok_ok) dst[is_q ? d : key_d_offset(d)] = f32_to_bf16(v);
-        }
-    } else if (tok_ok) {
-        bf16_t* dst = vpool + value_index(paged_row(pv, tok_slot[r], pos), head - nh - nkv, nkv, hd);
+            const bool second = g >= 2;
+            const bool is_q = head < nh;
+            bf16_t* dst = nullptr;
+            if (tok_ok) {
+                if (is_q) dst = q_out + ((long)tok * nh + head) * hd;
+                else dst = kpool + key_index(paged_row(pv, tok_slot[tok], pos), head - nh, nkv, hd);
+            }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) dst[value_d_offset(16 * s + 4 * g + i)] = f32_to_bf16(acc[i]);
+            for (int i = 0; i < 4; ++i) {
+                const int c = 8 * s + 4 * (g & 1) + i;             // index of the pair
+                float cs = 1.f, sn = 0.f;
+                if (inv_freq) {
+                    const float ang = (float)pos * inv_freq[c];
+                    cs = cosf(ang) * mscale;
+                    sn = sinf(ang) * mscale;
+                }
+                const float v = second ? lo[i] * sn + hi[i] * cs : lo[i] * cs - hi[i] * sn;
+                const int d = second ? c + hd / 2 : c;
+                if (tok_ok) dst[is_q ? d : key_d_offset(d)] = f32_to_bf16(v);
+            }
+        } else if (tok_ok) {
+            bf16_t* dst = vpool + value_index(paged_row(pv, tok_slot[tok], pos), head - nh - nkv, nkv, hd);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) dst[value_d_offset(16 * s + 4 * g + i)] = f32_to_bf16(acc[t][i]);
+        }
     }
 }
 
@@ -123,7 +142,7 @@ extern "C" const char* cpmcu_qkv_rope(const void* X, long ldx, const void* W, in
                                       int nkv, int hd, const int* positions, const int* tok_slot,
                                       const float* inv_freq, float mscale, void* kpool, void* vpool,
                                       const int* page_table, int table_width, int page_size, hipStream_t stream) {
-    CPMCU_REQUIRE(M > 0 && M <= 16, "qkv_rope: %d tokens (1..16 are taken; more go through the split product)", M);
+    CPMCU_REQUIRE(M > 0 && M <= 64, "qkv_rope: %d tokens (1..64 are taken; more go through the library's product)", M);
     CPMCU_REQUIRE(nh > 0 && nkv > 0 && hd > 0 && hd % 16 == 0, "qkv_rope: bad shape heads=%d kv_heads=%d head_dim=%d", nh, nkv, hd);
     CPMCU_REQUIRE(K > 0 && K % 8 == 0 && ldx % 8 == 0 && ldx >= K, "qkv_rope: K=%d, row stride %ld must be multiples of 8", K, ldx);
     CPMCU_REQUIRE(((uintptr_t)X % 16 == 0) && ((uintptr_t)W % 16 == 0), "qkv_rope: operands must be 16-byte aligned");
@@ -131,9 +150,14 @@ extern "C" const char* cpmcu_qkv_rope(const void* X, long ldx, const void* W, in
     CPMCU_REQUIRE(page_size % 32 == 0, "qkv_rope: a cache page of %d tokens is not a multiple of 32", page_size);
     PagedView pv{page_table, table_width, page_size};
     const int strips = (nh + 2 * nkv) * (hd / 16);
-    qkv_rope_kernel<4, 4><<<strips, 256, 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, M, K, (bf16_t*)q_out, nh,
-                                                   nkv, hd, positions, tok_slot, inv_freq, mscale, (bf16_t*)kpool,
-                                                   (bf16_t*)vpool, pv);
+#define LAUNCH(MTv)                                                                                              \
+    qkv_rope_kernel<4, 4, MTv><<<strips, 256, 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, M, K, (bf16_t*)q_out, \
+                                                           nh, nkv, hd, positions, tok_slot, inv_freq, mscale,       \
+                                                           (bf16_t*)kpool, (bf16_t*)vpool, pv)
+    if (M <= 16) LAUNCH(1);
+    else if (M <= 32) LAUNCH(2);
+    else LAUNCH(4);
+#undef LAUNCH
     CPMCU_LAUNCH_CHECK("qkv_rope");
     return nullptr;
 }
