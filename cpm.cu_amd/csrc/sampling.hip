@@ -9,34 +9,67 @@
 #include "common.h"
 
 // ties go to the lowest index
+__device__ inline void argmax_take(float v, int i, float& best, int& idx) {
+    if (v > best || (v == best && i < idx)) {
+        best = v;
+        idx = i;
+    }
+}
+// VEC: rows are 16-byte aligned and V is a multiple of 4: four logits a load, four loads in flight
+template <bool VEC>
 __global__ void argmax_kernel(const float* __restrict__ logits, long ld, int V, int* __restrict__ out) {
     __shared__ float bv[16];
     __shared__ int bi[16];
     const float* row = logits + (long)blockIdx.x * ld;
     float best = -INFINITY;
     int idx = 0x7fffffff;
-    for (int i = threadIdx.x; i < V; i += blockDim.x) {
-        const float v = row[i];
-        if (v > best || (v == best && i < idx)) { best = v; idx = i; }
+    if (VEC) {
+        const int V4 = V / 4, step = blockDim.x;
+        int i = threadIdx.x;
+        for (; i + 3 * step < V4; i += 4 * step) {
+            float4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = *(const float4*)(row + 4 * (i + u * step));
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int c = 4 * (i + u * step);
+                argmax_take(v[u].x, c, best, idx);
+                argmax_take(v[u].y, c + 1, best, idx);
+                argmax_take(v[u].z, c + 2, best, idx);
+                argmax_take(v[u].w, c + 3, best, idx);
+            }
+        }
+        for (; i < V4; i += step) {
+            const float4 v = *(const float4*)(row + 4 * i);
+            argmax_take(v.x, 4 * i, best, idx);
+            argmax_take(v.y, 4 * i + 1, best, idx);
+            argmax_take(v.z, 4 * i + 2, best, idx);
+            argmax_take(v.w, 4 * i + 3, best, idx);
+        }
+    } else {
+        for (int i = threadIdx.x; i < V; i += blockDim.x) argmax_take(row[i], i, best, idx);
     }
     for (int o = 32; o > 0; o >>= 1) {
         const float ov = __shfl_xor(best, o, 64);
         const int oi = __shfl_xor(idx, o, 64);
-        if (ov > best || (ov == best && oi < idx)) { best = ov; idx = oi; }
+        argmax_take(ov, oi, best, idx);
     }
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
     if (lane == 0) { bv[w] = best; bi[w] = idx; }
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int i = 1; i < nw; ++i)
-            if (bv[i] > best || (bv[i] == best && bi[i] < idx)) { best = bv[i]; idx = bi[i]; }
+        for (int i = 1; i < nw; ++i) argmax_take(bv[i], bi[i], best, idx);
         out[blockIdx.x] = idx == 0x7fffffff ? 0 : idx;
     }
 }
 
 extern "C" const char* cpmcu_argmax(const float* logits, long ld, int rows, int V, int* out, hipStream_t stream) {
     CPMCU_REQUIRE(rows > 0 && V > 0 && ld >= V, "argmax: bad shape rows=%d V=%d ld=%ld", rows, V, ld);
-    argmax_kernel<<<rows, V >= 4096 ? 1024 : 256, 0, stream>>>(logits, ld, V, out);
+    const int block = V >= 4096 ? 1024 : 256;
+    if (V % 4 == 0 && ld % 4 == 0 && ((uintptr_t)logits % 16 == 0))
+        argmax_kernel<true><<<rows, block, 0, stream>>>(logits, ld, V, out);
+    else
+        argmax_kernel<false><<<rows, block, 0, stream>>>(logits, ld, V, out);
     CPMCU_LAUNCH_CHECK("argmax");
     return nullptr;
 }

@@ -6,16 +6,19 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-def test_argmax_ties_go_to_the_lowest_index():
+@pytest.mark.parametrize("V", [7001, 73448, 20000, 36])       # odd (one logit a load) and multiples of 4 (four)
+def test_argmax_ties_go_to_the_lowest_index(V):
     from cpmcu_amd import ops
-    lg = torch.randn(5, 7001, generator=torch.Generator().manual_seed(0)).to(DEV)
-    lg[1, 6000] = lg[1, 17] = 50.0
+    lg = torch.randn(5, V, generator=torch.Generator().manual_seed(0)).to(DEV)
+    lg[1, V - 1001 if V > 2000 else V - 3] = lg[1, 17] = 50.0
     lg[2, 0] = 60.0
-    lg[3, 7000] = 60.0
+    lg[3, V - 1] = 60.0
+    lg[4, V // 2 + 1] = lg[4, V // 2 + 2] = 70.0
     out = torch.empty(5, dtype=torch.int32, device=DEV)
     ops.argmax(lg, out)
     want = lg.argmax(-1).tolist()
     want[1] = 17
+    want[4] = V // 2 + 1
     assert out.tolist() == want
 
 
