@@ -90,54 +90,61 @@ __device__ inline void philox4x32(uint32_t c[4], uint32_t k0, uint32_t k1) {
     }
 }
 
-// One block per row.  Thread i owns the contiguous vocabulary segment
-// [i*seg, (i+1)*seg); the thread whose range of the cumulative sum holds
-// u * total walks its segment.
-__global__ __launch_bounds__(256) void sample_kernel(const float* __restrict__ logits, long ld, int V,
-                                                    float inv_temperature, uint32_t seed_lo, uint32_t seed_hi,
-                                                    const int* __restrict__ request_ids, const int* __restrict__ steps,
-                                                    int* __restrict__ out, float* __restrict__ u_out) {
+// One block per row.  Thread i owns the vocabulary entries i, i + T, i + 2T, ... (T threads: neighbouring
+// threads read neighbouring logits).  The cumulative distribution runs over the entries in the order (thread 0's,
+// thread 1's, ...): any fixed order of the vocabulary gives a draw from the same distribution, and this one
+// depends on the row alone.  The thread whose range of the cumulative sum holds u * total walks its entries.
+__global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ logits, long ld, int V,
+                                                     float inv_temperature, uint32_t seed_lo, uint32_t seed_hi,
+                                                     const int* __restrict__ request_ids, const int* __restrict__ steps,
+                                                     int* __restrict__ out, float* __restrict__ u_out) {
     __shared__ float red[17];
-    __shared__ float seg_sum[256];
-    __shared__ float seg_pre[257];
+    __shared__ float wave_incl[16];
     __shared__ int owner;
-    const int r = blockIdx.x, tid = threadIdx.x;
+    const int r = blockIdx.x, tid = threadIdx.x, T = blockDim.x, lane = tid & 63, wave = tid >> 6;
     const float* row = logits + (long)r * ld;
     float mx = -INFINITY;
-    for (int i = tid; i < V; i += blockDim.x) mx = fmaxf(mx, row[i]);
+#pragma unroll 8
+    for (int i = tid; i < V; i += T) mx = fmaxf(mx, row[i]);
     mx = block_max(mx, red);
-    const int seg = (V + blockDim.x - 1) / blockDim.x;
-    const int i0 = min(tid * seg, V), i1 = min(i0 + seg, V);
     float s = 0.f;
-    for (int i = i0; i < i1; ++i) s += expf((row[i] - mx) * inv_temperature);
-    seg_sum[tid] = s;
+#pragma unroll 8
+    for (int i = tid; i < V; i += T) s += expf((row[i] - mx) * inv_temperature);
+    // inclusive prefix of the threads' sums: inside a wavefront, then the wavefronts before it
+    float incl = s;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const float up = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += up;
+    }
+    if (lane == 63) wave_incl[wave] = incl;
+    if (tid == 0) owner = 0;
     __syncthreads();
+    float before = 0.f, total = 0.f;
+    for (int w = 0; w < (T >> 6); ++w) {
+        if (w < wave) before += wave_incl[w];
+        total += wave_incl[w];
+    }
+    const float pre = before + incl - s;                  // sum of the threads before this one
     uint32_t ctr[4] = {(uint32_t)request_ids[r], (uint32_t)steps[r], 0u, 0u};
     philox4x32(ctr, seed_lo, seed_hi);
     const float u = (float)(ctr[0] >> 8) * (1.0f / 16777216.0f);   // [0, 1)
-    if (tid == 0) {
-        float c = 0.f;
-        for (int i = 0; i < (int)blockDim.x; ++i) { seg_pre[i] = c; c += seg_sum[i]; }
-        seg_pre[blockDim.x] = c;
-        // the owner: the last thread with a non-empty segment that starts at or before the target
-        const float tg = u * c;
-        int o = 0;
-        for (int i = 0; i < (int)blockDim.x; ++i)
-            if (seg_sum[i] > 0.f && seg_pre[i] <= tg) o = i;
-        owner = o;
-        if (u_out) u_out[r] = u;
-    }
+    const float target = u * total;
+    if (tid == 0 && u_out) u_out[r] = u;
+    // the owner: the last thread with a non-empty share that starts at or before the target
+    if (s > 0.f && pre <= target) atomicMax(&owner, tid);
     __syncthreads();
-    const float target = u * seg_pre[blockDim.x];
-    const bool mine = tid == owner;
-    if (mine) {
-        float c = seg_pre[tid];
-        int pick = -1, last = i0;
-        for (int i = i0; i < i1; ++i) {
+    if (tid == owner) {
+        float c = pre;
+        int pick = -1, last = tid < V ? tid : 0;
+        for (int i = tid; i < V; i += T) {
             const float e = expf((row[i] - mx) * inv_temperature);
             if (e > 0.f) last = i;
             c += e;
-            if (c > target) { pick = i; break; }
+            if (c > target) {
+                pick = i;
+                break;
+            }
         }
         out[r] = pick >= 0 ? pick : last;
     }
@@ -148,7 +155,7 @@ extern "C" const char* cpmcu_sample(const float* logits, long ld, int rows, int 
                                     float* u_out, hipStream_t stream) {
     CPMCU_REQUIRE(rows > 0 && V > 0 && ld >= V, "sample: bad shape rows=%d V=%d ld=%ld", rows, V, ld);
     CPMCU_REQUIRE(temperature > 0.f, "sample: temperature %g must be positive (0 is greedy: use argmax)", temperature);
-    sample_kernel<<<rows, 256, 0, stream>>>(logits, ld, V, 1.0f / temperature, (uint32_t)seed,
+    sample_kernel<<<rows, V >= 4096 ? 1024 : 256, 0, stream>>>(logits, ld, V, 1.0f / temperature, (uint32_t)seed,
                                             (uint32_t)(seed >> 32), request_ids, steps, out, u_out);
     CPMCU_LAUNCH_CHECK("sample");
     return nullptr;
