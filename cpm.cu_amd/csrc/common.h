@@ -109,6 +109,45 @@ __device__ inline float block_max(float v, float* red) {
     return t;
 }
 
+// ---- the norm's row factor, for products that apply it at their end ----
+// add_norm_columns leaves x * w and, for every row, the sums of x^2 over slices of NORM_SLICE columns;
+// r = rsqrt(sum of the slices / width + eps).  A workgroup of NT threads forms r for its ROWS rows at its
+// start: NT / ROWS neighbouring lanes share a row, each adds a contiguous run of the slices (16-byte loads,
+// four in flight, when the rows are aligned: a loop of dependent 4-byte loads cost 9 us in a 64-row product),
+// the lanes' shares meet inside the vector unit and the first lane writes r to rs_out[row] (LDS; the caller's
+// next barrier makes it visible).
+#define NORM_SLICE 64
+template <int TPR>
+__device__ inline float lanes_sum(float v) {
+    static_assert(TPR == 1 || TPR == 2 || TPR == 4 || TPR == 8 || TPR == 16, "lanes a row");
+    if (TPR >= 2) v += CPMCU_DPP(v, 0xB1);      // quad_perm [1,0,3,2]
+    if (TPR >= 4) v += CPMCU_DPP(v, 0x4E);      // quad_perm [2,3,0,1]
+    if (TPR >= 8) v += CPMCU_DPP(v, 0x141);     // row_half_mirror
+    if (TPR >= 16) v += CPMCU_DPP(v, 0x140);    // row_mirror
+    return v;
+}
+template <int NT, int ROWS>
+__device__ inline void row_scales(const float* __restrict__ row_ss, int n_slices, int n_rows, float inv_width,
+                                  float eps, float* rs_out) {
+    constexpr int TPR = NT / ROWS;
+    const int row = threadIdx.x / TPR, part = threadIdx.x % TPR;
+    const float* src = row_ss + (long)min(row, n_rows - 1) * n_slices;
+    const int per = ((n_slices + TPR - 1) / TPR + 3) & ~3;
+    const int i0 = part * per, i1 = min(i0 + per, n_slices);
+    float s = 0.f;
+    if ((n_slices & 3) == 0) {
+#pragma unroll 4
+        for (int i = i0; i < i1; i += 4) {
+            const float4 v = *(const float4*)(src + i);
+            s += (v.x + v.y) + (v.z + v.w);
+        }
+    } else {
+        for (int i = i0; i < i1; ++i) s += src[i];
+    }
+    s = lanes_sum<TPR>(s);
+    if (part == 0) rs_out[row] = 1.0f / sqrtf(s * inv_width + eps);
+}
+
 // ---- error convention ----
 inline char* cpmcu_errbuf() {
     static thread_local char buf[512];

@@ -182,6 +182,67 @@ extern "C" const char* cpmcu_add_rms_norm(float* x, const void* branch, int bran
     return nullptr;
 }
 
+// The norm of a step of few rows, cut by columns instead of rows.  rmsnorm(x) . W^T = r * ((x * w) . W^T) with
+// r = rsqrt(mean(x^2) + eps) one number a row: the product that follows can multiply by r at its end, so
+// nothing here needs a whole row.  A workgroup takes 64 columns of 16 rows: x += bscale * sum of the branch's
+// parts (in place), out = bf16(x * w), and row_ss[row][slice] = the slice's sum of x^2; the consumer adds the
+// slices up (common.h: row_scale_of).  A row a workgroup reads its partial sums through one CU at 6-7 us for
+// 8 rows of 4,096 columns; cut this way the same work is spread over 64 CUs.
+// (reference: src/model/norm.cuh:53-99, add and norm in one kernel, one block a row)
+template <typename BT>
+__global__ __launch_bounds__(256) void add_norm_columns_kernel(float* __restrict__ x, const BT* __restrict__ branch,
+                                                               int nparts, long part_stride, float bscale,
+                                                               const float* __restrict__ w, bf16_t* __restrict__ out,
+                                                               float* __restrict__ row_ss, int n, int H, int n_slices) {
+    const int slice = blockIdx.x, l16 = threadIdx.x & 15;
+    const int row = blockIdx.y * 16 + (threadIdx.x >> 4);
+    const int c = slice * NORM_SLICE + l16 * 4;
+    const bool ok = row < n && c < H;
+    const long off = (long)min(row, n - 1) * H + min(c, H - 4);
+    float4 v = *(const float4*)(x + off);
+    if (branch) {
+        float4 b = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll 8
+        for (int p = 0; p < nparts; ++p) {
+            const float4 t = load4(branch + p * part_stride + off);
+            b.x += t.x; b.y += t.y; b.z += t.z; b.w += t.w;
+        }
+        v.x += bscale * b.x; v.y += bscale * b.y; v.z += bscale * b.z; v.w += bscale * b.w;
+    }
+    float ss = 0.f;
+    if (ok) {
+        if (branch) *(float4*)(x + off) = v;
+        const float4 wv = *(const float4*)(w + c);
+        const bf16_t o0 = f32_to_bf16(v.x * wv.x), o1 = f32_to_bf16(v.y * wv.y);
+        const bf16_t o2 = f32_to_bf16(v.z * wv.z), o3 = f32_to_bf16(v.w * wv.w);
+        *(uint2*)(out + off) = make_uint2((uint32_t)o0.v | ((uint32_t)o1.v << 16), (uint32_t)o2.v | ((uint32_t)o3.v << 16));
+        ss = v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+    }
+    ss = row16_sum(ss);                      // the 16 lanes of a row of x are one row of lanes
+    if (l16 == 0 && row < n) row_ss[(long)row * n_slices + slice] = ss;
+}
+
+extern "C" const char* cpmcu_add_norm_columns(float* x, const void* branch, int branch_dtype, int nparts,
+                                              long part_stride, float bscale, const float* w, void* out,
+                                              float* row_ss, int n, int H, hipStream_t stream) {
+    CPMCU_REQUIRE(n > 0 && H > 0 && H % 4 == 0, "add_norm_columns: rows=%d, H=%d must be a positive multiple of 4", n, H);
+    CPMCU_REQUIRE(!branch || (nparts >= 1 && part_stride % 4 == 0), "add_norm_columns: nparts=%d stride=%ld", nparts, part_stride);
+    CPMCU_REQUIRE(x && w && out && row_ss, "add_norm_columns: null pointer");
+    CPMCU_REQUIRE(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0) && ((uintptr_t)out % 8 == 0) &&
+                  (!branch || (uintptr_t)branch % 16 == 0), "add_norm_columns: operands must be 16-byte aligned");
+    const int n_slices = (H + NORM_SLICE - 1) / NORM_SLICE;
+    dim3 grid(n_slices, (n + 15) / 16);
+    if (!branch || branch_dtype == CPMCU_F32)
+        add_norm_columns_kernel<float><<<grid, 256, 0, stream>>>(x, (const float*)branch, nparts, part_stride, bscale, w,
+                                                                 (bf16_t*)out, row_ss, n, H, n_slices);
+    else if (branch_dtype == CPMCU_BF16)
+        add_norm_columns_kernel<bf16_t><<<grid, 256, 0, stream>>>(x, (const bf16_t*)branch, nparts, part_stride, bscale,
+                                                                  w, (bf16_t*)out, row_ss, n, H, n_slices);
+    else CPMCU_FAIL("add_norm_columns: unknown branch dtype %d", branch_dtype);
+    CPMCU_LAUNCH_CHECK("add_norm_columns");
+    return nullptr;
+}
+
 // ---------------------------------------------------------------------------
 // out[r,c] = silu(gu[r,c]) * gu[r,c+I],  silu(g) = g / (1 + exp(-g))
 // (reference: src/model/activation.cuh:6-18, gate columns first, then up)

@@ -106,7 +106,8 @@ template <int MT, int MODE, typename OT, int SPW, int NW, bool TILED>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ X, long ldx,
                                                              const bf16_t* __restrict__ W, long ldw,
                                                              OT* __restrict__ Y, long ldy, int M, int N, int K, int KS,
-                                                             float alpha, int I, long part_stride) {
+                                                             float alpha, int I, long part_stride,
+                                                             const float* __restrict__ row_ss, float eps) {
     static_assert(MODE != 2 || SPW == 2, "gated output pairs a gate strip with an up strip");
     constexpr int NT = NW * 64;
     constexpr int XV = MT * 16 * 64 / NT;     // 16-byte vectors of X a thread stages per chunk
@@ -191,6 +192,10 @@ if (TILED) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) load_w(j, a[j]);
     load_x(0);
+    // X may be x * w of a norm whose row factor is still to come (common.h: row_scales); the loop's first
+    // barrier makes rs_s visible
+    __shared__ float rs_s[MT * 16];
+    if (row_ss) row_scales<NT, MT * 16>(row_ss, (K + NORM_SLICE - 1) / NORM_SLICE, M, 1.0f / (float)K, eps, rs_s);
     const int nchunk = (nkb + 3) / 4;
     for (int c = 0; c < nchunk; ++c) {
         __syncthreads();
@@ -220,12 +225,13 @@ if (TILED) {
     for (int t = 0; t < MT; ++t) {
         const int tok = t * 16 + r;
         if (tok >= M) continue;
+        const float rs_t = row_ss ? rs_s[tok] : 1.0f;
         if (MODE == 2) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int col = out_base[0] + 4 * g + i;
                 if (col < I) {
-                    const float gt = acc[0][t][i], up = acc[SPW - 1][t][i];
+                    const float gt = acc[0][t][i] * rs_t, up = acc[SPW - 1][t][i] * rs_t;
                     Yp[(long)tok * ldy + col] = from_f32<OT>(gt / (1.0f + expf(-gt)) * up);
                 }
             }
@@ -235,7 +241,7 @@ if (TILED) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int col = out_base[s] + 4 * g + i;
-                    if (col < N) Yp[(long)tok * ldy + col] = from_f32<OT>(alpha * acc[s][t][i]);
+                    if (col < N) Yp[(long)tok * ldy + col] = from_f32<OT>(alpha * rs_t * acc[s][t][i]);
                 }
         }
     }
@@ -243,9 +249,12 @@ if (TILED) {
 
 // out_mode: 0 = Y[m,N] in out_dtype; 1 = float partial sums Y[ksplit][m][N]; 2 = gated (N = 2*I rows of W, Y[m,I] bf16)
 // variant (gated output only): 0 = 4 waves a workgroup, 1 = 2 waves
+// row_ss (or null): X is x * w of add_norm_columns, whose sums of squares [M][ceil(K/64)] these are; the
+// output is multiplied by rsqrt(sum / K + eps) row by row
 extern "C" const char* cpmcu_gemm_skinny_v(const void* X, long ldx, const void* W, long ldw, void* Y, long ldy,
                                            int out_dtype, int out_mode, int M, int N, int K, int ksplit, float alpha,
-                                           int variant, int tiled, hipStream_t stream) {
+                                           int variant, int tiled, const float* row_ss, float eps,
+                                           hipStream_t stream) {
     CPMCU_REQUIRE(M > 0 && M <= 64, "gemm_skinny: %d rows (1..64 are taken; more rows belong to the tiled product)", M);
     CPMCU_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "gemm_skinny: K=%d must be a positive multiple of 8 (N=%d)", K, N);
     CPMCU_REQUIRE(ldx % 8 == 0 && ldx >= K && (tiled || (ldw % 8 == 0 && ldw >= K)),
@@ -268,10 +277,12 @@ extern "C" const char* cpmcu_gemm_skinny_v(const void* X, long ldx, const void* 
         dim3 grid(((MODEv == 2 ? I : N) + rows_wg - 1) / rows_wg, ksplit);                                        \
         if (tiled)                                                                                                \
             gemm_skinny_kernel<MTv, MODEv, OT, SPW, NW, true><<<grid, NW * 64, 0, stream>>>(                      \
-                (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (OT*)Y, ldy, M, N, K, KS, alpha, I, part_stride);   \
+                (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (OT*)Y, ldy, M, N, K, KS, alpha, I, part_stride,    \
+                row_ss, eps);                                                                                     \
         else                                                                                                      \
             gemm_skinny_kernel<MTv, MODEv, OT, SPW, NW, false><<<grid, NW * 64, 0, stream>>>(                     \
-                (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (OT*)Y, ldy, M, N, K, KS, alpha, I, part_stride);   \
+                (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (OT*)Y, ldy, M, N, K, KS, alpha, I, part_stride,    \
+                row_ss, eps);                                                                                     \
     } while (0)
 // shapes that measured best: one strip a wave in workgroups of 4 waves; gated output in workgroups of
 // 2 waves up to 16 rows of X (variant 1), of 4 waves above (variant 0)
@@ -304,8 +315,8 @@ extern "C" const char* cpmcu_gemm_skinny_v(const void* X, long ldx, const void* 
 // workgroups balance better over 256 CUs); gated output with 2 waves a workgroup up to 16 rows.
 extern "C" const char* cpmcu_gemm_skinny(const void* X, long ldx, const void* W, long ldw, void* Y, long ldy,
                                          int out_dtype, int out_mode, int M, int N, int K, int ksplit, float alpha,
-                                         int tiled, hipStream_t stream) {
+                                         int tiled, const float* row_ss, float eps, hipStream_t stream) {
     const int variant = out_mode == 2 ? (M <= 16 ? 1 : 0) : 2;
     return cpmcu_gemm_skinny_v(X, ldx, W, ldw, Y, ldy, out_dtype, out_mode, M, N, K, ksplit, alpha, variant, tiled,
-                               stream);
+                               row_ss, eps, stream);
 }

@@ -26,8 +26,9 @@ __global__ __launch_bounds__(NW * 64) void qkv_rope_kernel(
     const bf16_t* __restrict__ X, long ldx, const bf16_t* __restrict__ W, int M, int K, bf16_t* __restrict__ q_out,
     int nh, int nkv, int hd, const int* __restrict__ positions, const int* __restrict__ tok_slot,
     const float* __restrict__ inv_freq, float mscale, bf16_t* __restrict__ kpool, bf16_t* __restrict__ vpool,
-    PagedView pv) {
+    PagedView pv, const float* __restrict__ row_ss, float eps) {
     __shared__ float red[NW - 1][MT][4][64];
+    __shared__ float rs_s[MT * 16];            // the norm's row factors (common.h: row_scales), if x lacks them
     const int strip = blockIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
@@ -58,6 +59,7 @@ __global__ __launch_bounds__(NW * 64) void qkv_rope_kernel(
     };
 #pragma unroll
     for (int j = 0; j < PF; ++j) load_w(kb0 + j, a[j]);
+    if (row_ss) row_scales<NW * 64, MT * 16>(row_ss, (K + NORM_SLICE - 1) / NORM_SLICE, M, 1.0f / (float)K, eps, rs_s);
     qfloatx4_t acc[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[t] = qfloatx4_t{0.f, 0.f, 0.f, 0.f};
@@ -86,11 +88,17 @@ __global__ __launch_bounds__(NW * 64) void qkv_rope_kernel(
     __syncthreads();
     if (wave > 0) return;
 #pragma unroll
-    for (int t = 0; t < MT; ++t)
+    for (int t = 0; t < MT; ++t) {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
             for (int w = 0; w < NW - 1; ++w) acc[t][i] += red[w][t][i][lane];
+        if (row_ss) {          // X was x * w of a norm whose row factor comes now
+            const float rs = rs_s[t * 16 + r];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[t][i] *= rs;
+        }
+    }
 
     const int spt = hd / 16;                       // strips a head
     const int head = strip / spt, s = strip - head * spt;
@@ -141,7 +149,8 @@ __global__ __launch_bounds__(NW * 64) void qkv_rope_kernel(
 extern "C" const char* cpmcu_qkv_rope(const void* X, long ldx, const void* W, int M, int K, void* q_out, int nh,
                                       int nkv, int hd, const int* positions, const int* tok_slot,
                                       const float* inv_freq, float mscale, void* kpool, void* vpool,
-                                      const int* page_table, int table_width, int page_size, hipStream_t stream) {
+                                      const int* page_table, int table_width, int page_size, const float* row_ss,
+                                      float eps, hipStream_t stream) {
     CPMCU_REQUIRE(M > 0 && M <= 64, "qkv_rope: %d tokens (1..64 are taken; more go through the library's product)", M);
     CPMCU_REQUIRE(nh > 0 && nkv > 0 && hd > 0 && hd % 16 == 0, "qkv_rope: bad shape heads=%d kv_heads=%d head_dim=%d", nh, nkv, hd);
     CPMCU_REQUIRE(K > 0 && K % 8 == 0 && ldx % 8 == 0 && ldx >= K, "qkv_rope: K=%d, row stride %ld must be multiples of 8", K, ldx);
@@ -153,7 +162,7 @@ extern "C" const char* cpmcu_qkv_rope(const void* X, long ldx, const void* W, in
 #define LAUNCH(MTv)                                                                                              \
     qkv_rope_kernel<4, 4, MTv><<<strips, 256, 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, M, K, (bf16_t*)q_out, \
                                                            nh, nkv, hd, positions, tok_slot, inv_freq, mscale,       \
-                                                           (bf16_t*)kpool, (bf16_t*)vpool, pv)
+                                                           (bf16_t*)kpool, (bf16_t*)vpool, pv, row_ss, eps)
     if (M <= 16) LAUNCH(1);
     else if (M <= 32) LAUNCH(2);
     else LAUNCH(4);

@@ -110,6 +110,52 @@ def add_rms_norm(x: torch.Tensor, branch: Optional[torch.Tensor], branch_scale: 
                                              c_int(_code(out)), _p(rows), c_int(n_out), c_int(H), _stream()))
 
 
+NORM_SLICE = 64        # columns a slice of add_norm_columns (common.h)
+# rows up to which the norm cut by columns wins (MI355X, 4,096 columns, after a product's partial sums: 4.7
+# against 6.6 us at 8 rows; at 64 rows 4.8 against 5.0 us, and the gated product that finishes it 58.4 against 57 us)
+NORM_COLUMNS_MAX_ROWS = 16
+
+
+class RowScale:
+    """What a product needs to finish a norm that add_norm_columns began: the rows' sums of squares by slices
+    of NORM_SLICE columns, float32 [n, ceil(H / NORM_SLICE)], and eps.  The product multiplies its rows by
+    rsqrt(sum / H + eps), H being its own input width."""
+    __slots__ = ("sums", "eps")
+
+    def __init__(self, sums: torch.Tensor, eps: float):
+        self.sums, self.eps = sums, float(eps)
+
+
+def norm_slices(H: int) -> int:
+    return -(-H // NORM_SLICE)
+
+
+def add_norm_columns(x: torch.Tensor, branch: Optional[torch.Tensor], branch_scale: float, weight: torch.Tensor,
+                     out: torch.Tensor, sums: torch.Tensor):
+    """The norm of a step of few rows without its row factor: x += branch_scale * branch (in place; summed over
+    the leading axis if branch is [P,n,H]); out = bfloat16(x * weight); sums[r, s] = sum of x[r]^2 over slice s.
+    rmsnorm(x) * weight = out * rsqrt(sums.sum(1) / H + eps) row by row, which the product that reads `out`
+    applies to its result (gemm_skinny, qkv_rope: row_scale)."""
+    _need(x, "norm x", torch.float32, (None, None))
+    n, H = x.shape
+    if H % 4:
+        raise KernelError(f"add_norm_columns: a width of {H} is no multiple of 4")
+    _need(weight, "norm weight", torch.float32, (H,))
+    nparts, stride, bcode = 1, 0, F32
+    if branch is not None:
+        if branch.dim() == 3:
+            _need(branch, "norm branch", shape=(None, n, H))
+            nparts, stride = branch.shape[0], n * H
+        else:
+            _need(branch, "norm branch", shape=(n, H))
+        bcode = _code(branch)
+    _need(out, "norm out", torch.bfloat16, (n, H))
+    _need(sums, "norm row sums", torch.float32, (n, norm_slices(H)))
+    _check(_fn("core", "cpmcu_add_norm_columns")(_p(x), _p(branch), c_int(bcode), c_int(nparts), c_long(stride),
+                                                 c_float(branch_scale), _p(weight), _p(out), _p(sums), c_int(n),
+                                                 c_int(H), _stream()))
+
+
 def silu_mul(gate_up: torch.Tensor, out: torch.Tensor):
     """out[r,c] = silu(gate_up[r,c]) * gate_up[r,c+I];  gate_up [n,2I], out [n,I]."""
     _need(gate_up, "silu_mul input", shape=(None, None))
@@ -413,11 +459,15 @@ def qkv_rope_weight(w: torch.Tensor, nh: int, nkv: int, hd: int) -> TiledWeight:
 
 def qkv_rope(x: torch.Tensor, w: TiledWeight, q_out: torch.Tensor, nh: int, nkv: int, hd: int,
              positions: torch.Tensor, tok_slot: torch.Tensor, inv_freq: Optional[torch.Tensor], mscale: float,
-             kpool: torch.Tensor, vpool: torch.Tensor, page_table: torch.Tensor, page_size: int):
+             kpool: torch.Tensor, vpool: torch.Tensor, page_table: torch.Tensor, page_size: int,
+             row_scale: Optional[RowScale] = None):
     """q, k, v = x . w^T for a step of at most 64 tokens, rotated (inv_freq None: not) and written: q to q_out
-    [n, nh*hd], k and v into the paged cache.  w from qkv_rope_weight."""
+    [n, nh*hd], k and v into the paged cache.  w from qkv_rope_weight.  With row_scale, x is the x * w of
+    add_norm_columns and the rows of the product are multiplied by the norm's factor before the rotation."""
     _need(x, "qkv x", torch.bfloat16, (None, w.K))
     n = x.shape[0]
+    if row_scale is not None:
+        _need(row_scale.sums, "qkv row sums", torch.float32, (n, norm_slices(w.K)))
     if w.N != (nh + 2 * nkv) * hd:
         raise KernelError(f"qkv_rope: weight of {w.N} rows, {(nh + 2 * nkv) * hd} expected")
     _need(q_out, "qkv q_out", torch.bfloat16, (n, nh * hd))
@@ -431,16 +481,23 @@ def qkv_rope(x: torch.Tensor, w: TiledWeight, q_out: torch.Tensor, nh: int, nkv:
     _check(_fn("qkv", "cpmcu_qkv_rope")(_p(x), c_long(x.stride(0)), _p(w.data), c_int(n), c_int(w.K), _p(q_out),
                                         c_int(nh), c_int(nkv), c_int(hd), _p(positions), _p(tok_slot), _p(inv_freq),
                                         c_float(mscale), _p(kpool), _p(vpool), _p(page_table),
-                                        c_int(page_table.shape[1]), c_int(page_size), _stream()))
+                                        c_int(page_table.shape[1]), c_int(page_size),
+                                        _p(row_scale.sums if row_scale is not None else None),
+                                        c_float(row_scale.eps if row_scale is not None else 0.0), _stream()))
 
 
-def gemm_skinny(x: torch.Tensor, w, out: torch.Tensor, alpha: float = 1.0, mode: str = "plain"):
+def gemm_skinny(x: torch.Tensor, w, out: torch.Tensor, alpha: float = 1.0, mode: str = "plain",
+                row_scale: Optional[RowScale] = None):
     """bf16 product for at most 64 rows of x on the matrix cores, streaming w once; w is [N, K] as in the
     checkpoint or a TiledWeight.
     mode 'plain': out [m,N] float32 or bfloat16; 'partial': out float32 [S,m,N], S slices of K to be summed by
-    the consumer; 'gated': w holds gate rows then up rows, out bfloat16 [m,N/2] = silu(gate) * up."""
+    the consumer; 'gated': w holds gate rows then up rows, out bfloat16 [m,N/2] = silu(gate) * up.
+    With row_scale, x is the x * w of add_norm_columns: the rows of the product are multiplied by the norm's
+    factor (before the gate's nonlinearity)."""
     _need(x, "gemm x", torch.bfloat16, (None, None))
     M, K = x.shape
+    if row_scale is not None:
+        _need(row_scale.sums, "gemm row sums", torch.float32, (M, norm_slices(K)))
     tiled = isinstance(w, TiledWeight)
     if tiled:
         if w.K != K:
@@ -463,7 +520,9 @@ def gemm_skinny(x: torch.Tensor, w, out: torch.Tensor, alpha: float = 1.0, mode:
         raise KernelError(f"gemm_skinny: unknown mode '{mode}'")
     _check(_fn("gemm", "cpmcu_gemm_skinny")(_p(x), c_long(K), _p(wt), c_long(K), _p(out), c_long(ldy),
                                             c_int(_code(out)), c_int(omode), c_int(M), c_int(N), c_int(K),
-                                            c_int(ksplit), c_float(alpha), c_int(1 if tiled else 0), _stream()))
+                                            c_int(ksplit), c_float(alpha), c_int(1 if tiled else 0),
+                                            _p(row_scale.sums if row_scale is not None else None),
+                                            c_float(row_scale.eps if row_scale is not None else 0.0), _stream()))
 
 
 SKINNY_MAX_ROWS = 64

@@ -54,21 +54,33 @@ class GQAAttention(Mixer):
         return CacheNeeds(streams=(("k", StreamSpec(w)), ("v", StreamSpec(w))))
 
     # -- steps of forward, so that a subclass can put its own between them --
-    def project_and_store(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool) -> torch.Tensor:
+    def _fused_projection(self, n: int, dtype, cache: Optional[CacheView], writes_cache: bool) -> bool:
+        """Decode steps: projection, rotation and cache write in one kernel (one kernel of the chain less)."""
+        plain_rotation = self.position is None or self.position.rotary_params() is not None
+        return (writes_cache and cache is not None and plain_rotation and n <= ops.QKV_ROPE_MAX_ROWS
+                and dtype == torch.bfloat16 and self.qkv.tiled is not None and self.hd % 16 == 0
+                and cache.page_size % 32 == 0)
+
+    def takes_row_scale(self, n: int, ctx: StepContext, cache, writes_cache: bool) -> bool:
+        return self._fused_projection(n, self.rt.dtype, cache, writes_cache)
+
+    def project_and_store(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool, row_scale=None
+                          ) -> torch.Tensor:
         n = h.shape[0]
         nh, nkv, hd = self.nh, self.nkv, self.hd
         plain_rotation = self.position is None or self.position.rotary_params() is not None
-        if (writes_cache and plain_rotation and n <= ops.QKV_ROPE_MAX_ROWS and h.dtype == torch.bfloat16
-                and self.qkv.tiled is not None and hd % 16 == 0 and cache.page_size % 32 == 0):
-            # decode steps: projection, rotation and cache write in one kernel (one kernel of the chain less)
+        if self._fused_projection(n, h.dtype, cache, writes_cache):
             if self._qkv_fused is None:
                 self._qkv_fused = ops.qkv_rope_weight(self.qkv.weight, nh, nkv, hd)
             rot = self.position.rotary_params() if self.position is not None else None
             inv_freq, mag = (rot if rot is not None else (None, 1.0))
             q = ctx.ws.get("attn.q", (n, nh * hd), self.rt.dtype)
             ops.qkv_rope(h, self._qkv_fused, q, nh, nkv, hd, ctx.positions, ctx.tok_slot, inv_freq, mag,
-                         cache.streams["k"], cache.streams["v"], cache.page_table, cache.page_size)
+                         cache.streams["k"], cache.streams["v"], cache.page_table, cache.page_size,
+                         row_scale=row_scale)
             return q
+        if row_scale is not None:
+            raise ValueError("attention: a row scale needs the fused projection (takes_row_scale)")
         qkv = self.qkv.forward(h, ctx, "attn.qkv", rows=None if writes_cache else nh * hd, partials=plain_rotation)
         rot = self.position.rotary_params() if self.position is not None else None
         inv_freq, mag = (rot if rot is not None else (None, 1.0))
@@ -89,8 +101,9 @@ class GQAAttention(Mixer):
                       cache.page_table, cache.page_size, ctx, sel_blocks, sel_count, bs, window_blocks)
         return out
 
-    def forward(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool = True) -> torch.Tensor:
-        q = self.project_and_store(h, ctx, cache, writes_cache)
+    def forward(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool = True, row_scale=None
+                ) -> torch.Tensor:
+        q = self.project_and_store(h, ctx, cache, writes_cache, row_scale)
         a = self.attend(q, ctx, cache)
         return self.o.forward(a, ctx, "attn.o", out_dtype=torch.float32, partials=True)
 
@@ -113,8 +126,9 @@ class InfLLMv2Attention(GQAAttention):
         w = self.nkv * self.hd
         return CacheNeeds(streams=(("k", StreamSpec(w)), ("v", StreamSpec(w)), ("ck", StreamSpec(w, every=self.st))))
 
-    def forward(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool = True) -> torch.Tensor:
-        q = self.project_and_store(h, ctx, cache, writes_cache)
+    def forward(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool = True, row_scale=None
+                ) -> torch.Tensor:
+        q = self.project_and_store(h, ctx, cache, writes_cache, row_scale)
         if writes_cache:
             ops.compress_keys(cache.streams["k"], cache.streams["ck"], self.nkv, cache.page_table, cache.page_size,
                               ctx.positions, ctx.tok_slot, self.ks, self.st)

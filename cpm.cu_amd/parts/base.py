@@ -146,6 +146,15 @@ class Norm(Part):
                 rows: Optional[torch.Tensor] = None, tag: str = "norm") -> torch.Tensor:
         raise NotImplementedError
 
+    def forward_unscaled(self, x: torch.Tensor, branch: Optional[torch.Tensor], branch_scale: float,
+                         ctx: StepContext, tag: str = "norm"):
+        """For a norm whose result is (one number a row) * (something computed column by column), and a consumer
+        that begins with a linear layer: add the branch as forward does and return (rows without the row
+        factor, ops.RowScale that yields it), for the consumer's product to multiply its result by.  None if
+        this norm, or this step, has no such form; the caller then uses forward.  Only called when the
+        consumer's takes_row_scale() said yes."""
+        return None
+
 
 class PositionEncoding(Part):
     def rotary_params(self) -> Optional[Tuple[torch.Tensor, float]]:
@@ -167,10 +176,18 @@ class Mixer(Part):
                 ) -> torch.Tensor:
         raise NotImplementedError
 
+    def takes_row_scale(self, n: int, ctx: StepContext, cache: Optional[CacheView], writes_cache: bool) -> bool:
+        """True if forward, for this step of n tokens, accepts ``row_scale=`` (Norm.forward_unscaled) beside h."""
+        return False
+
 
 class FeedForward(Part):
     def forward(self, h: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         raise NotImplementedError
+
+    def takes_row_scale(self, n: int, ctx: StepContext) -> bool:
+        """True if forward, for this step of n tokens, accepts ``row_scale=`` (Norm.forward_unscaled) beside h."""
+        return False
 
 
 class Block(Part):

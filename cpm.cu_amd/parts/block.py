@@ -27,21 +27,43 @@ class PreNormBlock(Block):
     def parts(self) -> List[Part]:
         return [self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward]
 
+    @staticmethod
+    def _normed(norm: Norm, deferred: bool, x, branch, branch_scale, ctx):
+        """The normed rows and None, or (if the consumer finishes the norm itself) the rows without the norm's
+        row factor and that factor's ingredients."""
+        if deferred:
+            hs = norm.forward_unscaled(x, branch, branch_scale, ctx, tag="block.h")
+            if hs is not None:
+                return hs
+        return norm.forward(x, branch, branch_scale, ctx, tag="block.h"), None
+
+    def _mix(self, stream, ctx, cache, writes_cache):
+        n = stream.x.shape[0]
+        h, rs = self._normed(self.mixer_norm, self.mixer.takes_row_scale(n, ctx, cache, writes_cache),
+                             stream.x, stream.pending, stream.pending_scale, ctx)
+        if rs is None:
+            return self.mixer.forward(h, ctx, cache, writes_cache)
+        return self.mixer.forward(h, ctx, cache, writes_cache, row_scale=rs)
+
+    def _feed(self, stream, a, ctx):
+        n = stream.x.shape[0]
+        h, rs = self._normed(self.ff_norm, self.feed_forward.takes_row_scale(n, ctx),
+                             stream.x, a, self.residual_scale, ctx)
+        if rs is None:
+            return self.feed_forward.forward(h, ctx)
+        return self.feed_forward.forward(h, ctx, row_scale=rs)
+
     def forward(self, stream: ResidualStream, ctx: StepContext, cache: Optional[CacheView], writes_cache: bool = True):
         if ctx.perf is not None and ctx.perf.enabled:
             # the reference's timer labels distinguish prefill from decode and attention from feed-forward
             # (src/model/minicpm4/minicpm4_layer.cuh:46-83)
             phase = "decode" if ctx.single_token else "prefill"
             with ctx.perf.gpu(f"{phase}_attn"):
-                h = self.mixer_norm.forward(stream.x, stream.pending, stream.pending_scale, ctx, tag="block.h")
-                a = self.mixer.forward(h, ctx, cache, writes_cache)
+                a = self._mix(stream, ctx, cache, writes_cache)
             with ctx.perf.gpu(f"{phase}_ffn"):
-                h = self.ff_norm.forward(stream.x, a, self.residual_scale, ctx, tag="block.h")
-                stream.pending = self.feed_forward.forward(h, ctx)
+                stream.pending = self._feed(stream, a, ctx)
             stream.pending_scale = self.residual_scale
             return
-        h = self.mixer_norm.forward(stream.x, stream.pending, stream.pending_scale, ctx, tag="block.h")
-        a = self.mixer.forward(h, ctx, cache, writes_cache)
-        h = self.ff_norm.forward(stream.x, a, self.residual_scale, ctx, tag="block.h")
-        stream.pending = self.feed_forward.forward(h, ctx)
+        a = self._mix(stream, ctx, cache, writes_cache)
+        stream.pending = self._feed(stream, a, ctx)
         stream.pending_scale = self.residual_scale

@@ -26,6 +26,9 @@ class GatedFFN(FeedForward):
     def parts(self) -> List[Part]:
         return [self.gate_up, self.down]
 
-    def forward(self, h: torch.Tensor, ctx: StepContext) -> torch.Tensor:
-        act = self.gate_up.forward_gated(h, ctx, "ffn.gate_up")
+    def takes_row_scale(self, n: int, ctx: StepContext) -> bool:
+        return self.gate_up.gated_takes_row_scale(n)
+
+    def forward(self, h: torch.Tensor, ctx: StepContext, row_scale=None) -> torch.Tensor:
+        act = self.gate_up.forward_gated(h, ctx, "ffn.gate_up", row_scale=row_scale)
         return self.down.forward(act, ctx, "ffn.down", out_dtype=torch.float32, partials=True)

@@ -55,13 +55,24 @@ class Linear(Part):
         ops.linear(x, w, out, alpha, w_tiled=wt)
         return out
 
-    def forward_gated(self, x: torch.Tensor, ctx: StepContext, tag: str) -> torch.Tensor:
+    def _gated_skinny(self, n: int, dtype) -> bool:
+        return (dtype == torch.bfloat16 and n <= ops.SKINNY_MAX_ROWS and self.in_features % 8 == 0
+                and (self.tiled is None or (self.out_features // 2) % 16 == 0))
+
+    def gated_takes_row_scale(self, n: int) -> bool:
+        """Whether forward_gated, for n rows, runs the kernel that can finish a norm (ops.RowScale)."""
+        return self._gated_skinny(n, self.rt.dtype)
+
+    def forward_gated(self, x: torch.Tensor, ctx: StepContext, tag: str, row_scale=None) -> torch.Tensor:
         """For a weight of gate rows stacked on up rows: silu(x Wg^T) * (x Wu^T), [n, out/2]."""
         n, half = x.shape[0], self.out_features // 2
         act = ctx.ws.get(tag + ".act", (n, half), x.dtype)
-        if ops.skinny_ok(x) and (self.tiled is None or half % 16 == 0):
-            ops.gemm_skinny(x, self.tiled if self.tiled is not None else self.weight, act, mode="gated")
+        if self._gated_skinny(n, x.dtype):
+            ops.gemm_skinny(x, self.tiled if self.tiled is not None else self.weight, act, mode="gated",
+                            row_scale=row_scale)
         else:
+            if row_scale is not None:
+                raise ValueError("forward_gated: a row scale needs the few-rows kernel (gated_takes_row_scale)")
             gu = self.forward(x, ctx, tag)
             ops.silu_mul(gu, act)
         return act

@@ -33,3 +33,14 @@ class RMSNorm(Norm):
         out = ctx.ws.get(tag, (n_out, self.hidden_size), self.rt.dtype)
         ops.add_rms_norm(x, branch, branch_scale, self.weight, self.eps, out, rows)
         return out
+
+    def forward_unscaled(self, x, branch, branch_scale, ctx: StepContext, tag="norm"):
+        # decode steps: a row a workgroup leaves most of the chip idle, so the work is cut by columns and the
+        # row factor rsqrt(mean(x^2) + eps) is left to the product that follows
+        n = x.shape[0]
+        if self.rt.dtype != torch.bfloat16 or n > ops.NORM_COLUMNS_MAX_ROWS or self.hidden_size % 4:
+            return None
+        out = ctx.ws.get(tag, (n, self.hidden_size), torch.bfloat16)
+        sums = ctx.ws.get(tag + ".sums", (n, ops.norm_slices(self.hidden_size)), torch.float32)
+        ops.add_norm_columns(x, branch, branch_scale, self.weight, out, sums)
+        return out, ops.RowScale(sums, self.eps)

@@ -146,6 +146,47 @@ def test_add_rms_norm(H, n, bdtype, odtype):
     assert float((o - c / math.sqrt(c * c + eps)).abs().max()) < 1e-6
 
 
+@pytest.mark.parametrize("H,n", [(64, 1), (200, 7), (4096 + 8, 16), (328, 17), (96, 64)])
+@pytest.mark.parametrize("bdtype,parts", [(torch.float32, 0), (torch.float32, 1), (torch.float32, 5), (torch.bfloat16, 1)])
+def test_norm_cut_by_columns_and_finished_by_the_product(H, n, bdtype, parts):
+    """add_norm_columns leaves x * w and slice sums of x^2; the products multiply their rows by
+    rsqrt(sum / H + eps): together they equal product(rmsnorm(x) * w), gated and plain and in partial sums."""
+    from cpmcu_amd import ops
+    eps = 3e-4
+    x0, w = rnd(n, H, seed=1), rnd(H, seed=2) + 1.0
+    b = rnd(parts, n, H, seed=3, dtype=bdtype) if parts else None
+    x = x0.clone()
+    xw = torch.empty(n, H, dtype=torch.bfloat16, device=DEV)
+    sums = torch.full((n, ops.norm_slices(H)), float("nan"), device=DEV)
+    ops.add_norm_columns(x, None if b is None else (b if parts > 1 else b[0]), 0.7, w, xw, sums)
+    xs = x0.double() + (0.7 * b.double().sum(0) if parts else 0.0)
+    assert float((x.double() - xs).abs().max()) <= 1e-5
+    assert float((xw.double() - xs * w.double()).abs().max()) <= 2 ** -8 * float((xs * w.double()).abs().max())
+    ss = (xs * xs).sum(1)
+    assert float((sums.double().sum(1) - ss).abs().max()) <= 1e-5 * float(ss.max())
+    assert float((sums[:, 0].double() - (xs[:, :64] ** 2).sum(1)).abs().max()) <= 1e-5 * float(ss.max())
+    # the products finish the norm: against the float64 product of the rounded x * w, scaled row by row
+    rs = ops.RowScale(sums, eps)
+    r = torch.rsqrt(ss / H + eps)[:, None]
+    if H % 8:
+        return
+    N = 160
+    wm = rnd(N, H, seed=4, dtype=torch.bfloat16, scale=H ** -0.5)
+    for weight in (wm, ops.TiledWeight(wm)):
+        y = (xw.double() @ wm.double().T) * r
+        out = torch.empty(n, N, device=DEV)
+        ops.gemm_skinny(xw, weight, out, 0.5, row_scale=rs)
+        assert float((out.double() - 0.5 * y).abs().max()) <= 1e-4 * float(y.abs().max())
+        part = torch.empty(2, n, N, device=DEV)
+        if H > 128:                            # two slices of whole 128-column blocks
+            ops.gemm_skinny(xw, weight, part, 1.0, mode="partial", row_scale=rs)
+            assert float((part.double().sum(0) - y).abs().max()) <= 1e-4 * float(y.abs().max())
+        act = torch.empty(n, N // 2, dtype=torch.bfloat16, device=DEV)
+        ops.gemm_skinny(xw, weight, act, mode="gated", row_scale=rs)
+        ref = F.silu(y[:, :N // 2]) * y[:, N // 2:]
+        assert float((act.double() - ref).abs().max()) <= 2 ** -7 * max(1.0, float(ref.abs().max()))
+
+
 @pytest.mark.parametrize("I", [77, 160, 1000])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_silu_mul(dtype, I):
@@ -441,7 +482,8 @@ def read_cache_rows(pool, table, page, nkv, hd, slot, positions, tiles):
 @pytest.mark.parametrize("n,nh,nkv,hd,H,rotate", [(1, 4, 2, 16, 64, True), (8, 32, 2, 128, 512, True), (16, 3, 1, 32, 96, True),
                                                   (5, 6, 3, 64, 200, False), (13, 2, 2, 48, 264, True),
                                                   (17, 4, 2, 32, 136, True), (40, 2, 1, 64, 384, True), (64, 6, 2, 16, 72, True)])
-def test_fused_projection_rotation_and_cache_write(n, nh, nkv, hd, H, rotate):
+@pytest.mark.parametrize("scaled", [False, True])
+def test_fused_projection_rotation_and_cache_write(n, nh, nkv, hd, H, rotate, scaled):
     """q, k, v of a decode step in one kernel: against the float64 product, rotation (pairs c, c + hd/2) and the
     cache rows read back through the pages' layout; tokens of several slots at scattered positions."""
     from cpmcu_amd import ops
@@ -458,9 +500,16 @@ def test_fused_projection_rotation_and_cache_write(n, nh, nkv, hd, H, rotate):
     vpool = torch.zeros_like(kpool)
     q_out = torch.empty(n, nh * hd, dtype=torch.bfloat16, device=DEV)
     wt = ops.qkv_rope_weight(w, nh, nkv, hd)
+    # with the row factor of a norm cut by columns (the sums need not belong to x: any positive numbers do)
+    row_scale, r = None, 1.0
+    if scaled:
+        sums = torch.rand(n, ops.norm_slices(H), generator=g) + 0.1
+        row_scale = ops.RowScale(sums.to(DEV), 1e-3)
+        r = torch.rsqrt(sums.double().sum(1) / H + 1e-3).view(n, 1, 1)
     ops.qkv_rope(x, wt, q_out, nh, nkv, hd, positions.to(torch.int32).to(DEV), slots.to(torch.int32).to(DEV),
-                 inv_freq.to(DEV) if rotate else None, mscale if rotate else 1.0, kpool, vpool, table.to(DEV), page)
-    y = (x.double().cpu() @ w.double().cpu().T).view(n, nh + 2 * nkv, hd)
+                 inv_freq.to(DEV) if rotate else None, mscale if rotate else 1.0, kpool, vpool, table.to(DEV), page,
+                 row_scale=row_scale)
+    y = (x.double().cpu() @ w.double().cpu().T).view(n, nh + 2 * nkv, hd) * r
     if rotate:
         ang = positions.double()[:, None] * inv_freq.float().double()[None, :]          # angles formed in float32 on the GPU
         cs, sn = (torch.cos(ang) * mscale)[:, None, :], (torch.sin(ang) * mscale)[:, None, :]
