@@ -1,4 +1,4 @@
-// q, k, v projection of a decode step fused with the rotation and the cache write (bf16, at most 64 tokens).
+// q, k, v projection of a decode step fused with the rotation and the cache write (bf16, at most 32 tokens).
 //
 // A decode step is a chain of small kernels, each of which costs a few microseconds whatever it does; this one
 // replaces the split-K product + the kernel that summed its partial sums, rotated and stored.
@@ -9,7 +9,7 @@
 // workgroup that owns one strip then holds both halves of 8 rotation pairs.  v heads keep their order.
 //
 // One workgroup of 4 wavefronts a strip: the wavefronts take a quarter of the columns each (x straight from
-// global memory into the B operand, one tile of 16 tokens after the other), add their results through LDS, and the
+// global memory into the B operand, asked for together with the weight's block), add their results through LDS, and the
 // first wavefront rotates and writes: queries to q_out [token][head][d], keys and values into the cache pages
 // in the matrix cores' order (common.h: key_index, value_index).
 // theta = pos * inv_freq[c]; (a, b) = (x[c], x[c+hd/2]) -> (a cos - b sin, a sin + b cos), cos and sin times
@@ -38,43 +38,48 @@ __global__ __launch_bounds__(NW * 64) void qkv_rope_kernel(
     const bf16_t* wp = W + (long)strip * nkb * 2048 + lane * 8;
     const bf16_t* xp[MT];                                  // rows beyond the step repeat its last token
 #pragma unroll
-    for (int t = 0; t < MT; ++t) xp[t] = X + (long)min(t * 16 + r, M - 1) * ldx + g * 8;
+    for (int t = 0; t < MT; ++t) xp[t] = X + (long)min(t * 16 + r, M - 1) * ldx;
 
-    qbf16x8_t a[PF][4];
-    auto load_w = [&](int kb, qbf16x8_t (&dst)[4]) {
+    // Loads return in the order of their issue, so the x of a block is asked for together with its w, PF blocks
+    // ahead (asked for only at its use, it would make the wavefront wait for every w behind it: one trip to
+    // memory a block).  No load stands in a branch that depends on data: addresses are clamped instead (a block
+    // beyond the wavefront's last repeats it and is not multiplied; columns beyond K repeat the row's last 8
+    // and meet the weight's zero padding), so the waits count exactly.
+    qbf16x8_t a[PF][4], bx[PF][MT][4];
+    auto load_block = [&](int kb, qbf16x8_t (&wd)[4], qbf16x8_t (&xd)[MT][4]) {
+        const int kbc = min(kb, nkb - 1);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            qbf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (kb < kb1) v = __builtin_nontemporal_load((const qbf16x8_t*)(wp + ((long)kb * 4 + i) * 512));
-            dst[i] = v;
-        }
+        for (int i = 0; i < 4; ++i) wd[i] = __builtin_nontemporal_load((const qbf16x8_t*)(wp + ((long)kbc * 4 + i) * 512));
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) xd[t][i] = *(const qbf16x8_t*)(xp[t] + min(kbc * 128 + i * 32 + g * 8, K - 8));
     };
-    auto load_x = [&](int kb, int t, qbf16x8_t (&dst)[4]) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            qbf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (kb < kb1 && kb * 128 + i * 32 + g * 8 < K) v = *(const qbf16x8_t*)(xp[t] + (long)kb * 128 + i * 32);
-            dst[i] = v;
-        }
-    };
-#pragma unroll
-    for (int j = 0; j < PF; ++j) load_w(kb0 + j, a[j]);
-    if (row_ss) row_scales<NW * 64, MT * 16>(row_ss, (K + NORM_SLICE - 1) / NORM_SLICE, M, 1.0f / (float)K, eps, rs_s);
     qfloatx4_t acc[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[t] = qfloatx4_t{0.f, 0.f, 0.f, 0.f};
-    for (int kb = kb0; kb < kb1; kb += PF) {
+    auto multiply = [&](qbf16x8_t (&wd)[4], qbf16x8_t (&xd)[MT][4]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wd[i], xd[t][i], acc[t], 0, 0, 0);
+    };
+#pragma unroll
+    for (int j = 0; j < PF; ++j) load_block(kb0 + j, a[j], bx[j]);
+    if (row_ss) row_scales<NW * 64, MT * 16>(row_ss, (K + NORM_SLICE - 1) / NORM_SLICE, M, 1.0f / (float)K, eps, rs_s);
+    int kb = kb0;
+    for (; kb + 2 * PF <= kb1; kb += PF) {           // every block and every block asked for exists
 #pragma unroll
         for (int j = 0; j < PF; ++j) {
-            qbf16x8_t b[MT][4];
+            multiply(a[j], bx[j]);
+            load_block(kb + j + PF, a[j], bx[j]);
+        }
+    }
+    for (; kb < kb1; kb += PF) {                      // the last blocks: nothing more, or only what exists, is asked for
 #pragma unroll
-            for (int t = 0; t < MT; ++t) load_x(kb + j, t, b[t]);
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int t = 0; t < MT; ++t)
-                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j][i], b[t][i], acc[t], 0, 0, 0);
-            load_w(kb + j + PF, a[j]);
+        for (int j = 0; j < PF; ++j) {
+            if (kb + j < kb1) multiply(a[j], bx[j]);
+            if (kb + j + PF < kb1) load_block(kb + j + PF, a[j], bx[j]);
         }
     }
     // lane (token r, g) of tile t: acc[t][i] is feature row 4g + i of the strip; the other wavefronts hand theirs
@@ -151,7 +156,7 @@ extern "C" const char* cpmcu_qkv_rope(const void* X, long ldx, const void* W, in
                                       const float* inv_freq, float mscale, void* kpool, void* vpool,
                                       const int* page_table, int table_width, int page_size, const float* row_ss,
                                       float eps, hipStream_t stream) {
-    CPMCU_REQUIRE(M > 0 && M <= 64, "qkv_rope: %d tokens (1..64 are taken; more go through the library's product)", M);
+    CPMCU_REQUIRE(M > 0 && M <= 32, "qkv_rope: %d tokens (1..32 are taken; more go through the split product and the rotary kernel)", M);
     CPMCU_REQUIRE(nh > 0 && nkv > 0 && hd > 0 && hd % 16 == 0, "qkv_rope: bad shape heads=%d kv_heads=%d head_dim=%d", nh, nkv, hd);
     CPMCU_REQUIRE(K > 0 && K % 8 == 0 && ldx % 8 == 0 && ldx >= K, "qkv_rope: K=%d, row stride %ld must be multiples of 8", K, ldx);
     CPMCU_REQUIRE(((uintptr_t)X % 16 == 0) && ((uintptr_t)W % 16 == 0), "qkv_rope: operands must be 16-byte aligned");
@@ -164,8 +169,7 @@ extern "C" const char* cpmcu_qkv_rope(const void* X, long ldx, const void* W, in
                                                            nh, nkv, hd, positions, tok_slot, inv_freq, mscale,       \
                                                            (bf16_t*)kpool, (bf16_t*)vpool, pv, row_ss, eps)
     if (M <= 16) LAUNCH(1);
-    else if (M <= 32) LAUNCH(2);
-    else LAUNCH(4);
+    else LAUNCH(2);
 #undef LAUNCH
     CPMCU_LAUNCH_CHECK("qkv_rope");
     return nullptr;

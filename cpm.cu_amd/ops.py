@@ -440,8 +440,7 @@ class TiledWeight:
         self.N, self.K = N, K
 
 
-# qkv_rope takes up to 64 tokens; it wins up to 16 (MI355X, 8B shape: 13.4 against 16.8 us at 8 tokens, 16.2 against
-# 18.0 at 16, 24.7 against 21.5 at 32: x then comes from L2 four tiles at a time without LDS)
+# qkv_rope takes up to 32 tokens; it wins up to 16 (MI355X, 8B shape; figures at QKV_ROPE_MAX_ROWS' users)
 QKV_ROPE_MAX_ROWS = 16
 
 
@@ -463,7 +462,7 @@ def qkv_rope(x: torch.Tensor, w: TiledWeight, q_out: torch.Tensor, nh: int, nkv:
              positions: torch.Tensor, tok_slot: torch.Tensor, inv_freq: Optional[torch.Tensor], mscale: float,
              kpool: torch.Tensor, vpool: torch.Tensor, page_table: torch.Tensor, page_size: int,
              row_scale: Optional[RowScale] = None):
-    """q, k, v = x . w^T for a step of at most 64 tokens, rotated (inv_freq None: not) and written: q to q_out
+    """q, k, v = x . w^T for a step of at most 32 tokens, rotated (inv_freq None: not) and written: q to q_out
     [n, nh*hd], k and v into the paged cache.  w from qkv_rope_weight.  With row_scale, x is the x * w of
     add_norm_columns and the rows of the product are multiplied by the norm's factor before the rotation."""
     _need(x, "qkv x", torch.bfloat16, (None, w.K))

@@ -481,7 +481,7 @@ def read_cache_rows(pool, table, page, nkv, hd, slot, positions, tiles):
 
 @pytest.mark.parametrize("n,nh,nkv,hd,H,rotate", [(1, 4, 2, 16, 64, True), (8, 32, 2, 128, 512, True), (16, 3, 1, 32, 96, True),
                                                   (5, 6, 3, 64, 200, False), (13, 2, 2, 48, 264, True),
-                                                  (17, 4, 2, 32, 136, True), (40, 2, 1, 64, 384, True), (64, 6, 2, 16, 72, True)])
+                                                  (17, 4, 2, 32, 136, True), (24, 2, 1, 64, 1160, True), (32, 6, 2, 16, 72, True)])
 @pytest.mark.parametrize("scaled", [False, True])
 def test_fused_projection_rotation_and_cache_write(n, nh, nkv, hd, H, rotate, scaled):
     """q, k, v of a decode step in one kernel: against the float64 product, rotation (pairs c, c + hd/2) and the
