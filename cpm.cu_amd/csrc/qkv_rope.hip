@@ -26,7 +26,8 @@ __global__ __launch_bounds__(NW * 64) void qkv_rope_kernel(
     const bf16_t* __restrict__ X, long ldx, const bf16_t* __restrict__ W, int M, int K, bf16_t* __restrict__ q_out,
     int nh, int nkv, int hd, const int* __restrict__ positions, const int* __restrict__ tok_slot,
     const float* __restrict__ inv_freq, float mscale, bf16_t* __restrict__ kpool, bf16_t* __restrict__ vpool,
-    PagedView pv, const float* __restrict__ row_ss, float eps) {
+    PagedView pv, const float* __restrict__ row_ss, float eps, bf16_t* __restrict__ ckpool, int ck_size,
+    int ck_stride) {
     __shared__ float red[NW - 1][MT][4][64];
     __shared__ float rs_s[MT * 16];            // the norm's row factors (common.h: row_scales), if x lacks them
     const int strip = blockIdx.x;
@@ -107,11 +108,14 @@ __global__ __launch_bounds__(NW * 64) void qkv_rope_kernel(
 
     const int spt = hd / 16;                       // strips a head
     const int head = strip / spt, s = strip - head * spt;
+    float own[MT][4];                              // a key head's values as the cache holds them
+    int tok_pos[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
         const int tok = t * 16 + r;
         const bool tok_ok = tok < M;
         const int pos = positions[min(tok, M - 1)];
+        tok_pos[t] = pos;
         if (head < nh + nkv) {
             // rows 0..7 of the strip are d = 8s .. 8s+7, rows 8..15 their partners d + hd/2: lanes g and g+2 hold
             // a pair; after the swap every lane has both (the first half of the wavefront's value, then the second's)
@@ -141,12 +145,57 @@ __global__ __launch_bounds__(NW * 64) void qkv_rope_kernel(
                 }
                 const float v = second ? lo[i] * sn + hi[i] * cs : lo[i] * cs - hi[i] * sn;
                 const int d = second ? c + hd / 2 : c;
-                if (tok_ok) dst[is_q ? d : key_d_offset(d)] = f32_to_bf16(v);
+                const bf16_t vb = f32_to_bf16(v);
+                own[t][i] = to_f32(vb);
+                if (tok_ok) dst[is_q ? d : key_d_offset(d)] = vb;
             }
         } else if (tok_ok) {
             bf16_t* dst = vpool + value_index(paged_row(pv, tok_slot[tok], pos), head - nh - nkv, nkv, hd);
 #pragma unroll
             for (int i = 0; i < 4; ++i) dst[value_d_offset(16 * s + 4 * g + i)] = f32_to_bf16(acc[t][i]);
+        }
+    }
+
+    // Compressed keys (sparse.hip: compress_keys_kernel, the same sums in the same order): the token at position
+    // p completes the mean of the keys p+1-ck_size .. p when p+1-ck_size is a non-negative multiple of ck_stride.
+    // This workgroup wrote its 16 features of all the step's keys itself; the fence makes them readable, and
+    // is paid only in the steps in which a token completes one.
+    if (ckpool && head >= nh && head < nh + nkv) {
+        const int kvh = head - nh;
+        const int d0 = 8 * s + 4 * (g & 1) + (g >= 2 ? hd / 2 : 0);        // this lane's 4 features
+        bool mine[MT], any = false;
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            const int p1 = tok_pos[t] + 1;
+            mine[t] = t * 16 + r < M && p1 >= ck_size && (p1 - ck_size) % ck_stride == 0;
+            any = any || mine[t];
+        }
+        if (__any(any)) {
+            __threadfence();
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                if (!mine[t]) continue;
+                const int slot = tok_slot[t * 16 + r];
+                const int first = tok_pos[t] + 1 - ck_size;
+                float sum[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+                for (int k = 0; k < ck_size - 1; ++k) {
+                    const uint2 u = *(const uint2*)(kpool + key_index(paged_row(pv, slot, first + k), kvh, nkv, hd) +
+                                                    key_d_offset(d0));
+                    sum[0] += __uint_as_float(u.x << 16);
+                    sum[1] += __uint_as_float(u.x & 0xffff0000u);
+                    sum[2] += __uint_as_float(u.y << 16);
+                    sum[3] += __uint_as_float(u.y & 0xffff0000u);
+                }
+                uint32_t o[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) o[i] = f32_to_bf16((sum[i] + own[t][i]) / (float)ck_size).v;
+                const int page = pv.page_table[(long)slot * pv.table_width + first / pv.page_size];
+                const int rpp = pv.page_size / ck_stride;
+                bf16_t* dst = ckpool + ck_index(page, (first % pv.page_size) / ck_stride, kvh, nkv, hd, rpp) +
+                              ck_d_offset(d0, rpp);
+                *(uint2*)dst = make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+            }
         }
     }
 }
@@ -155,19 +204,23 @@ extern "C" const char* cpmcu_qkv_rope(const void* X, long ldx, const void* W, in
                                       int nkv, int hd, const int* positions, const int* tok_slot,
                                       const float* inv_freq, float mscale, void* kpool, void* vpool,
                                       const int* page_table, int table_width, int page_size, const float* row_ss,
-                                      float eps, hipStream_t stream) {
+                                      float eps, void* ckpool, int ck_size, int ck_stride, hipStream_t stream) {
     CPMCU_REQUIRE(M > 0 && M <= 32, "qkv_rope: %d tokens (1..32 are taken; more go through the split product and the rotary kernel)", M);
     CPMCU_REQUIRE(nh > 0 && nkv > 0 && hd > 0 && hd % 16 == 0, "qkv_rope: bad shape heads=%d kv_heads=%d head_dim=%d", nh, nkv, hd);
     CPMCU_REQUIRE(K > 0 && K % 8 == 0 && ldx % 8 == 0 && ldx >= K, "qkv_rope: K=%d, row stride %ld must be multiples of 8", K, ldx);
     CPMCU_REQUIRE(((uintptr_t)X % 16 == 0) && ((uintptr_t)W % 16 == 0), "qkv_rope: operands must be 16-byte aligned");
     CPMCU_REQUIRE(q_out && kpool && vpool && page_table && positions && tok_slot, "qkv_rope: null pointer");
     CPMCU_REQUIRE(page_size % 32 == 0, "qkv_rope: a cache page of %d tokens is not a multiple of 32", page_size);
+    CPMCU_REQUIRE(!ckpool || (ck_stride > 0 && ck_size >= ck_stride && page_size % ck_stride == 0),
+                  "qkv_rope: kernel_stride %d must divide the cache page of %d tokens (kernel_size %d)", ck_stride,
+                  page_size, ck_size);
     PagedView pv{page_table, table_width, page_size};
     const int strips = (nh + 2 * nkv) * (hd / 16);
 #define LAUNCH(MTv)                                                                                              \
     qkv_rope_kernel<4, 4, MTv><<<strips, 256, 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, M, K, (bf16_t*)q_out, \
                                                            nh, nkv, hd, positions, tok_slot, inv_freq, mscale,       \
-                                                           (bf16_t*)kpool, (bf16_t*)vpool, pv, row_ss, eps)
+                                                           (bf16_t*)kpool, (bf16_t*)vpool, pv, row_ss, eps,      \
+                                                           (bf16_t*)ckpool, ck_size, ck_stride)
     if (M <= 16) LAUNCH(1);
     else LAUNCH(2);
 #undef LAUNCH

@@ -10,7 +10,7 @@ from __future__ import annotations
 
 import ctypes
 from ctypes import c_char_p, c_float, c_int, c_long, c_ulonglong, c_void_p
-from typing import Optional, Sequence
+from typing import Optional, Sequence, Tuple
 
 import torch
 
@@ -461,14 +461,22 @@ def qkv_rope_weight(w: torch.Tensor, nh: int, nkv: int, hd: int) -> TiledWeight:
 def qkv_rope(x: torch.Tensor, w: TiledWeight, q_out: torch.Tensor, nh: int, nkv: int, hd: int,
              positions: torch.Tensor, tok_slot: torch.Tensor, inv_freq: Optional[torch.Tensor], mscale: float,
              kpool: torch.Tensor, vpool: torch.Tensor, page_table: torch.Tensor, page_size: int,
-             row_scale: Optional[RowScale] = None):
+             row_scale: Optional[RowScale] = None, compress: Optional[Tuple[torch.Tensor, int, int]] = None):
     """q, k, v = x . w^T for a step of at most 32 tokens, rotated (inv_freq None: not) and written: q to q_out
     [n, nh*hd], k and v into the paged cache.  w from qkv_rope_weight.  With row_scale, x is the x * w of
-    add_norm_columns and the rows of the product are multiplied by the norm's factor before the rotation."""
+    add_norm_columns and the rows of the product are multiplied by the norm's factor before the rotation.
+    With compress = (compressed key pool, kernel_size, kernel_stride) the compressed keys that the step's tokens
+    complete are written too, as compress_keys would after this call."""
     _need(x, "qkv x", torch.bfloat16, (None, w.K))
     n = x.shape[0]
     if row_scale is not None:
         _need(row_scale.sums, "qkv row sums", torch.float32, (n, norm_slices(w.K)))
+    ckpool, ks, st = compress if compress is not None else (None, 0, 0)
+    if ckpool is not None:
+        # (compressed key pool, kernel_size, kernel_stride): the step's tokens also complete their compressed keys
+        if st <= 0 or page_size % st:
+            raise KernelError(f"qkv_rope: kernel_stride {st} must divide the cache page of {page_size} tokens")
+        _need(ckpool, "qkv compressed key pool", torch.bfloat16, (kpool.shape[0], page_size // st, nkv * hd))
     if w.N != (nh + 2 * nkv) * hd:
         raise KernelError(f"qkv_rope: weight of {w.N} rows, {(nh + 2 * nkv) * hd} expected")
     _need(q_out, "qkv q_out", torch.bfloat16, (n, nh * hd))
@@ -484,7 +492,8 @@ def qkv_rope(x: torch.Tensor, w: TiledWeight, q_out: torch.Tensor, nh: int, nkv:
                                         c_float(mscale), _p(kpool), _p(vpool), _p(page_table),
                                         c_int(page_table.shape[1]), c_int(page_size),
                                         _p(row_scale.sums if row_scale is not None else None),
-                                        c_float(row_scale.eps if row_scale is not None else 0.0), _stream()))
+                                        c_float(row_scale.eps if row_scale is not None else 0.0),
+                                        _p(ckpool), c_int(ks), c_int(st), _stream()))
 
 
 def gemm_skinny(x: torch.Tensor, w, out: torch.Tensor, alpha: float = 1.0, mode: str = "plain",

@@ -64,8 +64,11 @@ class GQAAttention(Mixer):
     def takes_row_scale(self, n: int, ctx: StepContext, cache, writes_cache: bool) -> bool:
         return self._fused_projection(n, self.rt.dtype, cache, writes_cache)
 
-    def project_and_store(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool, row_scale=None
-                          ) -> torch.Tensor:
+    def project_and_store(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool, row_scale=None,
+                          compress=None) -> torch.Tensor:
+        """q [n, heads * head_dim], position-encoded; k and v go into the cache.  ``compress`` (a pool of
+        compressed keys, kernel_size, kernel_stride) is only given where _fused_projection() holds: that kernel
+        then also writes the compressed keys that the step's tokens complete."""
         n = h.shape[0]
         nh, nkv, hd = self.nh, self.nkv, self.hd
         plain_rotation = self.position is None or self.position.rotary_params() is not None
@@ -77,10 +80,10 @@ class GQAAttention(Mixer):
             q = ctx.ws.get("attn.q", (n, nh * hd), self.rt.dtype)
             ops.qkv_rope(h, self._qkv_fused, q, nh, nkv, hd, ctx.positions, ctx.tok_slot, inv_freq, mag,
                          cache.streams["k"], cache.streams["v"], cache.page_table, cache.page_size,
-                         row_scale=row_scale)
+                         row_scale=row_scale, compress=compress)
             return q
-        if row_scale is not None:
-            raise ValueError("attention: a row scale needs the fused projection (takes_row_scale)")
+        if row_scale is not None or compress is not None:
+            raise ValueError("attention: a row scale or compressed keys need the fused projection (takes_row_scale)")
         qkv = self.qkv.forward(h, ctx, "attn.qkv", rows=None if writes_cache else nh * hd, partials=plain_rotation)
         rot = self.position.rotary_params() if self.position is not None else None
         inv_freq, mag = (rot if rot is not None else (None, 1.0))
@@ -128,8 +131,11 @@ class InfLLMv2Attention(GQAAttention):
 
     def forward(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool = True, row_scale=None
                 ) -> torch.Tensor:
-        q = self.project_and_store(h, ctx, cache, writes_cache, row_scale)
-        if writes_cache:
+        # decode steps: the projection kernel completes the compressed keys itself (one kernel of the chain less)
+        fused = self._fused_projection(h.shape[0], h.dtype, cache, writes_cache)
+        q = self.project_and_store(h, ctx, cache, writes_cache, row_scale,
+                                   compress=(cache.streams["ck"], self.ks, self.st) if fused else None)
+        if writes_cache and not fused:
             ops.compress_keys(cache.streams["k"], cache.streams["ck"], self.nkv, cache.page_table, cache.page_size,
                               ctx.positions, ctx.tok_slot, self.ks, self.st)
         sel = None

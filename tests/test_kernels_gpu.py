@@ -526,6 +526,41 @@ def test_fused_projection_rotation_and_cache_write(n, nh, nkv, hd, H, rotate, sc
     assert int((kpool != 0).sum()) <= n * nkv * hd and int((vpool != 0).sum()) <= n * nkv * hd
 
 
+@pytest.mark.parametrize("n,ks,st", [(16, 8, 4), (5, 32, 16), (32, 12, 4), (1, 32, 16)])
+def test_fused_projection_completes_compressed_keys(n, ks, st):
+    """The projection kernel of decode steps also writes the compressed keys that its tokens complete: bit for
+    bit what compress_keys writes after it, from keys of earlier steps and of this step (two sequences, each
+    with consecutive tokens in the step, at different phases of the stride)."""
+    from cpmcu_amd import ops
+    nh, nkv, hd, H, page = 4, 2, 32, 136, 64
+    w = rnd((nh + 2 * nkv) * hd, H, seed=1, dtype=torch.bfloat16, scale=H ** -0.5)
+    x = rnd(n, H, seed=2, dtype=torch.bfloat16)
+    g = torch.Generator().manual_seed(ks)
+    n0 = (n + 1) // 2
+    first = (47 if n > 1 else 16 * 5 + 32 - 1, 70)           # the lone token completes a compressed key
+    positions = torch.tensor([first[0] + i for i in range(n0)] + [first[1] + i for i in range(n - n0)], dtype=torch.int32)
+    slots = torch.tensor([0] * n0 + [1] * (n - n0), dtype=torch.int32)
+    table = torch.randperm(8, generator=g).view(2, 4).to(torch.int32)
+    inv_freq = torch.rand(hd // 2, generator=g) * 0.5 + 0.01
+    wt = ops.qkv_rope_weight(w, nh, nkv, hd)
+    results = []
+    for fused in (True, False):
+        kpool = rnd(8, page, nkv * hd, seed=5, dtype=torch.bfloat16)        # the keys of earlier steps
+        vpool = torch.zeros_like(kpool)
+        ck = torch.zeros(8, page // st, nkv * hd, dtype=torch.bfloat16, device=DEV)
+        q_out = torch.empty(n, nh * hd, dtype=torch.bfloat16, device=DEV)
+        ops.qkv_rope(x, wt, q_out, nh, nkv, hd, positions.to(DEV), slots.to(DEV), inv_freq.to(DEV), 1.0, kpool, vpool,
+                     table.to(DEV), page, compress=(ck, ks, st) if fused else None)
+        if not fused:
+            ops.compress_keys(kpool, ck, nkv, table.to(DEV), page, positions.to(DEV), slots.to(DEV), ks, st)
+        results.append((kpool, ck, q_out))
+    (ka, ca, qa), (kb, cb, qb) = results
+    assert torch.equal(ka, kb) and torch.equal(qa, qb)
+    completed = sum(1 for p in positions.tolist() if p + 1 >= ks and (p + 1 - ks) % st == 0)
+    assert completed > 0 and int((cb != 0).sum()) > 0
+    assert torch.equal(ca, cb)
+
+
 # ---------------------------------------------------------------------------- InfLLM-v2 kernels
 @pytest.mark.parametrize("ks,st", [(8, 4), (32, 16), (16, 16), (12, 4)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
