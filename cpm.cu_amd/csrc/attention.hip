@@ -137,8 +137,8 @@ extern "C" const char* cpmcu_attention_plain(const void* q, void* out, int dtype
 typedef __bf16 abf16x8_t __attribute__((ext_vector_type(8)));
 typedef float afloatx4_t __attribute__((ext_vector_type(4)));
 
-// 2^x for x <= 0 (probabilities and rescale factors): the bare hardware instruction; results below the
-// normal range come out as 0, which is what a probability that small contributes anyway
+// 2^x for x <= 8 (weights and rescale factors): the bare hardware instruction; results below the
+// normal range come out as 0, which is what a weight that small contributes anyway
 __device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 template <int HD, int NW, int TW>
@@ -297,7 +297,13 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_mfma_kernel(
                                  fmaxf(fmaxf(st[1][0], st[1][1]), fmaxf(st[1][2], st[1][3])));
                 mx = rows_max(mx);
                 // m is kept in units of the exponent: scores times scale*log2(e)
-                const float m_new = fmaxf(m, mx * scale_log2e);
+                // The exponent's reference m follows the maximum only when some row's maximum has moved up by
+                // more than 8 (weights then reach 2^8 at most, which float sums and bf16 weights take as well
+                // as 1): the 16 rows' maxima of random scores move in half of all chunks, by that much almost
+                // never after the first, and every move costs a pass over the accumulators.
+                const float m_top = fmaxf(m, mx * scale_log2e);
+                const bool moved = __builtin_amdgcn_ballot_w64(m_top > m + 8.0f) != 0;
+                const float m_new = moved ? m_top : m;
                 const float m_ref = m_new == -INFINITY ? 0.f : m_new;      // nothing seen yet: all weights 0
                 const float corr = fast_exp2(m - m_ref);
                 float rs = 0.f;
@@ -312,8 +318,7 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_mfma_kernel(
                     }
                 rs = rows_sum(rs);
                 l = l * corr + rs;
-                // the accumulators are rescaled only when some row's maximum moved (rare after the first chunks)
-                if (__builtin_amdgcn_ballot_w64(m_new != m) != 0) {
+                if (moved) {
 #pragma unroll
                     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -623,7 +628,10 @@ __global__ __launch_bounds__(NW * 64) void attention_prefill_mfma_kernel(
                 mx = rows_max(mx);
                 // running maximum in units of scaled scores (scale > 0); a row whose position lies before
                 // this chunk sees none of its keys: nothing changes for it
-                const float m_new = fmaxf(m[r], mx * scale_log2e);
+                // the reference follows the maximum only past a move of more than 8 (see attention_mfma_kernel)
+                const float m_top = fmaxf(m[r], mx * scale_log2e);
+                const bool moved = __builtin_amdgcn_ballot_w64(m_top > m[r] + 8.0f) != 0;
+                const float m_new = moved ? m_top : m[r];
                 const float m_use = m_new == -INFINITY ? 0.f : m_new;
                 const float corr = fast_exp2(m[r] - m_use);
                 float rs = 0.f;
@@ -636,8 +644,7 @@ __global__ __launch_bounds__(NW * 64) void attention_prefill_mfma_kernel(
                 }
                 rs = rows_sum(rs);
                 l[r] = l[r] * corr + rs;
-                // the accumulators are rescaled only when some row's maximum moved (rare after the first chunks)
-                if (__builtin_amdgcn_ballot_w64(m_new != m[r]) != 0) {
+                if (moved) {
 #pragma unroll
                     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
