@@ -435,8 +435,8 @@ extern "C" const char* cpmcu_attention_mfma(const void* q, void* out, float* par
                                             const int* sel_count, int max_sel, int block_size, int n_splits,
                                             int waves_per_group, int last_blocks_first, hipStream_t stream) {
     CPMCU_REQUIRE(n > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_mfma: bad shape n=%d heads=%d kv_heads=%d", n, nh, nkv);
-    CPMCU_REQUIRE(hd == 16 || hd == 32 || hd == 64 || hd == 128,
-                  "attention_mfma: head_dim %d has no matrix-core kernel (16, 32, 64, 128 have; the plain kernel takes the rest)", hd);
+    CPMCU_REQUIRE(hd >= 16 && hd <= 128 && hd % 16 == 0,
+                  "attention_mfma: head_dim %d has no matrix-core kernel (16, 32, ... 128 have; the plain kernel takes the rest)", hd);
     CPMCU_REQUIRE(page_size % 32 == 0, "attention_mfma: a cache page of %d tokens is not a multiple of 32", page_size);
     CPMCU_REQUIRE(!sel_count || (sel_blocks && max_sel > 0 && block_size > 0 && block_size % 32 == 0),
                   "attention_mfma: key blocks of %d tokens are not a multiple of 32", block_size);
@@ -465,10 +465,16 @@ extern "C" const char* cpmcu_attention_mfma(const void* q, void* out, float* par
         else if (tw == 4) LAUNCH(HDv, 1, 4);  \
         else LAUNCH(HDv, 1, 1);               \
     } while (0)
-    if (hd == 16) BY_NW(16);
-    else if (hd == 32) BY_NW(32);
-    else if (hd == 64) BY_NW(64);
-    else BY_NW(128);
+    switch (hd) {
+        case 16: BY_NW(16); break;
+        case 32: BY_NW(32); break;
+        case 48: BY_NW(48); break;
+        case 64: BY_NW(64); break;
+        case 80: BY_NW(80); break;
+        case 96: BY_NW(96); break;
+        case 112: BY_NW(112); break;
+        default: BY_NW(128); break;
+    }
 #undef BY_NW
 #undef LAUNCH
     CPMCU_LAUNCH_CHECK("attention_mfma");
@@ -726,8 +732,8 @@ extern "C" const char* cpmcu_attention_prefill_mfma(const void* q, void* out, in
                                                     int page_size, const int* positions, const int* tok_slot,
                                                     hipStream_t stream) {
     CPMCU_REQUIRE(n_tiles > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_prefill: bad shape tiles=%d heads=%d kv_heads=%d", n_tiles, nh, nkv);
-    CPMCU_REQUIRE(hd == 16 || hd == 32 || hd == 64 || hd == 128,
-                  "attention_prefill: head_dim %d has no matrix-core kernel (16, 32, 64, 128 have)", hd);
+    CPMCU_REQUIRE(hd >= 16 && hd <= 128 && hd % 16 == 0,
+                  "attention_prefill: head_dim %d has no matrix-core kernel (16, 32, ... 128 have)", hd);
     CPMCU_REQUIRE(page_size % 32 == 0, "attention_prefill: a cache page of %d tokens is not a multiple of 32", page_size);
     const int G = nh / nkv;
     const int rpt = (G < 16 && 16 % G == 0) ? G : 16;
@@ -753,10 +759,16 @@ extern "C" const char* cpmcu_attention_prefill_mfma(const void* q, void* out, in
         else if (waves_per_group == 2) LAUNCH(HDv, 2, 2);                       \
         else LAUNCH(HDv, 2, 1);                                                 \
     } while (0)
-    if (hd == 16) BY_R(16);
-    else if (hd == 32) BY_R(32);
-    else if (hd == 64) BY_R(64);
-    else BY_R(128);
+    switch (hd) {
+        case 16: BY_R(16); break;
+        case 32: BY_R(32); break;
+        case 48: BY_R(48); break;
+        case 64: BY_R(64); break;
+        case 80: BY_R(80); break;
+        case 96: BY_R(96); break;
+        case 112: BY_R(112); break;
+        default: BY_R(128); break;
+    }
 #undef BY_R
 #undef LAUNCH
     CPMCU_LAUNCH_CHECK("attention_prefill_mfma");

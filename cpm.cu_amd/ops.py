@@ -235,7 +235,7 @@ def attention_plain(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hd: i
         _p(sel_blocks), _p(sel_count), c_int(max_sel), c_int(block_size), _stream()))
 
 
-MFMA_HEAD_DIMS = (16, 32, 64, 128)
+MFMA_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128)
 
 
 def attention_mfma_ok(q: torch.Tensor, hd: int, page_size: int, block_size: int = 0) -> bool:
@@ -249,7 +249,7 @@ def attention_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hd: in
                    part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None,
                    sel_blocks: Optional[torch.Tensor] = None, sel_count: Optional[torch.Tensor] = None,
                    block_size: int = 0, waves_per_group: int = 0, last_blocks_first: int = 0):
-    """bf16 attention on the matrix cores (head_dim 16, 32, 64 or 128; pages and key blocks multiples of 32).
+    """bf16 attention on the matrix cores (head_dim 16, 32, ... 128; pages and key blocks multiples of 32).
     With n_splits > 1 every token's keys are shared among n_splits wavefronts and merged afterwards;
     part_o float32 [n, nh, n_splits, hd] and part_ml float32 [n, nh, n_splits, 2] are its scratch.
     last_blocks_first: that many blocks at the end of every block list (the window that neighbouring tokens

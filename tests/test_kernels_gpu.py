@@ -271,7 +271,8 @@ def attention_reference(qs, ks, vs, positions, seq_of, nh, scale, allowed=None):
     return torch.stack(out)
 
 
-@pytest.mark.parametrize("nh,nkv,hd", [(4, 2, 16), (3, 1, 32), (6, 3, 64), (32, 2, 128), (20, 1, 32), (2, 2, 48), (4, 1, 256)])
+@pytest.mark.parametrize("nh,nkv,hd", [(4, 2, 16), (3, 1, 32), (6, 3, 64), (32, 2, 128), (20, 1, 32), (2, 2, 48), (4, 1, 256),
+                                       (6, 2, 80), (3, 1, 96), (4, 4, 112)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_attention_over_scrambled_pages(nh, nkv, hd, dtype):
     """Prompt tokens and single tokens of three sequences at once; plain kernel, and the matrix-core kernel
@@ -313,7 +314,7 @@ def test_attention_over_scrambled_pages(nh, nkv, hd, dtype):
         assert not ops.attention_mfma_ok(q.view(n, -1), hd, page)
 
 
-@pytest.mark.parametrize("nh,nkv,hd", [(16, 1, 64), (8, 1, 32), (4, 2, 128), (5, 5, 16), (40, 2, 32)])
+@pytest.mark.parametrize("nh,nkv,hd", [(16, 1, 64), (8, 1, 32), (4, 2, 128), (5, 5, 16), (40, 2, 32), (6, 2, 48), (2, 1, 96)])
 def test_prompt_attention_from_position_zero_and_continued(nh, nkv, hd):
     """Whole prompts from position 0 (where early tiles stop before late chunks) and a chunk that continues
     a sequence already in the cache, several sequences packed."""
