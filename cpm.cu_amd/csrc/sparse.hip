@@ -298,7 +298,7 @@ extern "C" const char* cpmcu_sparse_select(const void* q, const void* ckpool, in
                   max_pos + 1, lds);
     dim3 grid(n, nkv);
     PagedView pv{page_table, table_width, page_size};
-    if (dtype == CPMCU_BF16 && !force_plain && (hd == 16 || hd == 32 || hd == 64 || hd == 128)) {
+    if (dtype == CPMCU_BF16 && !force_plain && hd >= 16 && hd <= 128 && hd % 16 == 0) {
         const size_t lds2 = sizeof(float) * ((size_t)sp.max_ck + 4 + select_work_floats(sp.max_blocks));
         CPMCU_REQUIRE(lds2 <= 60 * 1024,
                       "sparse_select: a context of %d tokens needs %zu bytes of LDS for its block scores (limit 61440)",
@@ -321,10 +321,16 @@ extern "C" const char* cpmcu_sparse_select(const void* q, const void* ckpool, in
 #define SCORES(HDv)                                                                                               \
             select_scores_kernel<HDv><<<sgrid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)ckpool, pv, positions, \
                                                                  tok_slot, sp, sc)
-            if (hd == 16) SCORES(16);
-            else if (hd == 32) SCORES(32);
-            else if (hd == 64) SCORES(64);
-            else SCORES(128);
+            switch (hd) {
+                case 16: SCORES(16); break;
+                case 32: SCORES(32); break;
+                case 48: SCORES(48); break;
+                case 64: SCORES(64); break;
+                case 80: SCORES(80); break;
+                case 96: SCORES(96); break;
+                case 112: SCORES(112); break;
+                default: SCORES(128); break;
+            }
 #undef SCORES
             CPMCU_LAUNCH_CHECK("select_scores");
             const size_t lds3 = sizeof(float) * ((size_t)sc.n_groups * G * 2 + 2 * G);
@@ -345,10 +351,16 @@ extern "C" const char* cpmcu_sparse_select(const void* q, const void* ckpool, in
                 sparse_select_mfma_kernel<HDv, 4><<<grid, 256, lds2, stream>>>(                              \
                     (const bf16_t*)q, (const bf16_t*)ckpool, pv, positions, tok_slot, sp, sel_blocks, sel_count); \
         } while (0)
-        if (hd == 16) LAUNCH(16);
-        else if (hd == 32) LAUNCH(32);
-        else if (hd == 64) LAUNCH(64);
-        else LAUNCH(128);
+        switch (hd) {
+            case 16: LAUNCH(16); break;
+            case 32: LAUNCH(32); break;
+            case 48: LAUNCH(48); break;
+            case 64: LAUNCH(64); break;
+            case 80: LAUNCH(80); break;
+            case 96: LAUNCH(96); break;
+            case 112: LAUNCH(112); break;
+            default: LAUNCH(128); break;
+        }
 #undef LAUNCH
         CPMCU_LAUNCH_CHECK("sparse_select_mfma");
         return nullptr;

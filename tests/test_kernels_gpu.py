@@ -588,7 +588,7 @@ def test_compressed_keys_are_means_written_when_their_last_key_arrives(ks, st, d
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("nh,nkv,hd", [(6, 2, 16), (32, 2, 128), (20, 1, 32)])
+@pytest.mark.parametrize("nh,nkv,hd", [(6, 2, 16), (32, 2, 128), (20, 1, 32), (8, 2, 48), (3, 1, 96)])
 @pytest.mark.parametrize("ks,st,bs,init,topk,window,dense_len", [(8, 4, 16, 1, 4, 32, 64), (32, 16, 64, 1, 3, 128, 0),
                                                               (8, 8, 32, 2, 2, 32, 100), (16, 4, 16, 0, 5, 16, 0)])
 def test_block_selection_equals_the_plain_selection(dtype, nh, nkv, hd, ks, st, bs, init, topk, window, dense_len):
