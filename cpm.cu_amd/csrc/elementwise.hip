@@ -129,6 +129,28 @@ __global__ __launch_bounds__(1024) void add_rms_norm_vec4_kernel(float* __restri
         if (c < H4) emit(c, v, 1.0f / sqrtf(ss / (float)H + eps));
         return;
     }
+    if (H4 <= 4 * (int)blockDim.x) {
+        // up to 4 vectors a thread stay in registers as well (many rows: blocks of 256 threads, rows of 4,096)
+        float4 v[4];
+        float ss = 0.f;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int c = threadIdx.x + k * blockDim.x;
+            v[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (c < H4) {
+                v[k] = summed(c);
+                if (branch && !rows) *(float4*)(xr + 4 * c) = v[k];
+            }
+            ss += v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w;
+        }
+        const float rs = 1.0f / sqrtf(block_sum(ss, red) / (float)H + eps);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int c = threadIdx.x + k * blockDim.x;
+            if (c < H4) emit(c, v[k], rs);
+        }
+        return;
+    }
     float ss = 0.f;
     for (int c = threadIdx.x; c < H4; c += blockDim.x) {
         const float4 v = summed(c);
