@@ -405,6 +405,16 @@ __global__ void attention_combine_kernel(const float* __restrict__ part_o, const
     __shared__ float wgt[64];
     const long row = blockIdx.x;             // token * nh + head
     const float2* ml = part_ml + row * n_splits;
+    const float* po = part_o + row * n_splits * hd;
+    // Up to 16 shares and one feature a thread: the shares' outputs are asked for before anything waits for
+    // the (max, sum) pairs, so that both come back in one trip to memory instead of two.
+    const bool held = n_splits <= 16 && hd <= (int)blockDim.x;
+    float held_o[16];
+    if (held) {
+        const int d = min((int)threadIdx.x, hd - 1);
+#pragma unroll
+        for (int s = 0; s < 16; ++s) held_o[s] = po[(long)min(s, n_splits - 1) * hd + d];
+    }
     float m = -INFINITY;
     for (int s = 0; s < n_splits; ++s) {
         const float2 v = ml[s];
@@ -419,7 +429,14 @@ __global__ void attention_combine_kernel(const float* __restrict__ part_o, const
     }
     __syncthreads();
     const float inv = 1.0f / denom;
-    const float* po = part_o + row * n_splits * hd;
+    if (held) {
+        float a = 0.f;
+#pragma unroll
+        for (int s = 0; s < 16; ++s)
+            if (s < n_splits) a += wgt[s] * held_o[s];
+        if ((int)threadIdx.x < hd) out[row * hd + threadIdx.x] = f32_to_bf16(a * inv);
+        return;
+    }
     for (int d = threadIdx.x; d < hd; d += blockDim.x) {
         float a = 0.f;
 #pragma unroll 8
@@ -479,7 +496,7 @@ extern "C" const char* cpmcu_attention_mfma(const void* q, void* out, float* par
 #undef LAUNCH
     CPMCU_LAUNCH_CHECK("attention_mfma");
     if (n_splits > 1) {
-        attention_combine_kernel<<<(unsigned)((long)n * nh), hd >= 64 ? 64 : hd, 0, stream>>>(
+        attention_combine_kernel<<<(unsigned)((long)n * nh), hd > 64 ? 128 : 64, 0, stream>>>(
             part_o, (const float2*)part_ml, (bf16_t*)out, hd, n_splits);
         CPMCU_LAUNCH_CHECK("attention_combine");
     }
