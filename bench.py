@@ -161,7 +161,8 @@ def main():
     step_bytes = weight_bytes_per_step(cfg, esize) + args.batch * (args.context + args.steps // 2) * kv_bytes_per_token(cfg, esize)
     achieved = step_bytes / (ms_step * 1e-3) / 1e9
     rec = {
-        "metric": "MiniCPM4-8B decode tok/s @ batch 8, context 4096 (bf16, random weights)",
+        "metric": f"MiniCPM4-8B decode tok/s @ batch {args.batch}, context {args.context} "
+                  f"({'bf16' if args.dtype == 'bfloat16' else 'fp32'}, random weights)",
         "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
