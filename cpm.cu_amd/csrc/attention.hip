@@ -613,70 +613,91 @@ __global__ __launch_bounds__(NW * 64) void attention_prefill_mfma_kernel(
         load_k(pchunk, kf);
         load_v(pchunk, vf);
     }
+    // the three stages of a tile's work on a chunk of keys
+    auto scores = [&](int r, afloatx4_t (&st)[2]) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            st[u] = afloatx4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks)
+                st[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][ks], qf[r][ks], st[u], 0, 0, 0);
+        }
+    };
+    auto weights = [&](int r, int key0, const afloatx4_t (&st)[2]) {
+        // raw scores; only a chunk that reaches past a row's position needs the causal mask
+        float sc[8];
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sc[u * 4 + i] = st[u][i];
+        if (key0 + 31 > tile_first_pos[r]) {
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (key0 + 8 * g + 4 * u + i > row_pos[r]) sc[u * 4 + i] = -INFINITY;
+        }
+        float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
+                         fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+        mx = rows_max(mx);
+        // running maximum in units of scaled scores (scale > 0); a row whose position lies before
+        // this chunk sees none of its keys: nothing changes for it
+        // the reference follows the maximum only past a move of more than 8 (see attention_mfma_kernel)
+        const float m_top = fmaxf(m[r], mx * scale_log2e);
+        const bool moved = __builtin_amdgcn_ballot_w64(m_top > m[r] + 8.0f) != 0;
+        const float m_new = moved ? m_top : m[r];
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        const float corr = fast_exp2(m[r] - m_use);
+        float rs = 0.f;
+        abf16x8_t pb;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float p = fast_exp2(fmaf(sc[j], scale_log2e, -m_use));
+            rs += p;
+            pb[j] = (__bf16)p;
+        }
+        rs = rows_sum(rs);
+        l[r] = l[r] * corr + rs;
+        if (moved) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[r][dt][i] *= corr;
+        }
+        m[r] = m_new;
+        return pb;
+    };
+    auto values = [&](int r, abf16x8_t pb) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+            acc[r][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pb, acc[r][dt], 0, 0, 0);
+    };
     for (int c = wave; c < total_chunks; c += NW) {
         const int key0 = c * 32;
         const bool more = c + NW < total_chunks;
         int pchunkn = 0;
         if (more) pchunkn = next_pchunk();
+        if constexpr (R == 2) {
+            // The matrix instructions of one tile are issued before the vector work of the other, so that each
+            // runs in the other's shadow (a wavefront issues in order, and a matrix instruction holds only its
+            // own pipe).  A tile that does not see this chunk (the first tile at the last chunk of the second, an
+            // unused tile) is computed all the same: the mask leaves it weights of 0.
+            afloatx4_t s0[2], s1[2];
+            scores(0, s0);
+            scores(1, s1);
+            if (more) load_k(pchunkn, kf);
+            const abf16x8_t p0 = weights(0, key0, s0);
+            values(0, p0);
+            const abf16x8_t p1 = weights(1, key0, s1);
+            values(1, p1);
+        } else {
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const bool active = r < n_tiles_used && key0 <= tile_last_pos[r];
-            afloatx4_t st[2];
-            if (active) {
-#pragma unroll
-                for (int u = 0; u < 2; ++u) {
-                    st[u] = afloatx4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int ks = 0; ks < KSTEPS; ++ks)
-                        st[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][ks], qf[r][ks], st[u], 0, 0, 0);
-                }
-            }
-            if (r == R - 1 && more) load_k(pchunkn, kf);      // the last tile's scores are issued: keys are free
-            if (active) {
-                // raw scores; only a chunk that reaches past a row's position needs the causal mask
-                float sc[8];
-#pragma unroll
-                for (int u = 0; u < 2; ++u)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) sc[u * 4 + i] = st[u][i];
-                if (key0 + 31 > tile_first_pos[r]) {
-#pragma unroll
-                    for (int u = 0; u < 2; ++u)
-#pragma unroll
-                        for (int i = 0; i < 4; ++i)
-                            if (key0 + 8 * g + 4 * u + i > row_pos[r]) sc[u * 4 + i] = -INFINITY;
-                }
-                float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
-                                 fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
-                mx = rows_max(mx);
-                // running maximum in units of scaled scores (scale > 0); a row whose position lies before
-                // this chunk sees none of its keys: nothing changes for it
-                // the reference follows the maximum only past a move of more than 8 (see attention_mfma_kernel)
-                const float m_top = fmaxf(m[r], mx * scale_log2e);
-                const bool moved = __builtin_amdgcn_ballot_w64(m_top > m[r] + 8.0f) != 0;
-                const float m_new = moved ? m_top : m[r];
-                const float m_use = m_new == -INFINITY ? 0.f : m_new;
-                const float corr = fast_exp2(m[r] - m_use);
-                float rs = 0.f;
-                abf16x8_t pb;
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const float p = fast_exp2(fmaf(sc[j], scale_log2e, -m_use));
-                    rs += p;
-                    pb[j] = (__bf16)p;
-                }
-                rs = rows_sum(rs);
-                l[r] = l[r] * corr + rs;
-                if (moved) {
-#pragma unroll
-                    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) acc[r][dt][i] *= corr;
-                }
-                m[r] = m_new;
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-                    acc[r][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pb, acc[r][dt], 0, 0, 0);
+            for (int r = 0; r < R; ++r) {
+                const bool active = r < n_tiles_used && key0 <= tile_last_pos[r];
+                afloatx4_t st[2];
+                if (active) scores(r, st);
+                if (r == R - 1 && more) load_k(pchunkn, kf);      // the last tile's scores are issued: keys are free
+                if (active) values(r, weights(r, key0, st));
             }
         }
         if (more) load_v(pchunkn, vf);
