@@ -450,7 +450,8 @@ extern "C" const char* cpmcu_attention_mfma(const void* q, void* out, float* par
                                             const int* page_table, int table_width, int page_size,
                                             const int* positions, const int* tok_slot, const int* sel_blocks,
                                             const int* sel_count, int max_sel, int block_size, int n_splits,
-                                            int waves_per_group, int last_blocks_first, hipStream_t stream) {
+                                            int waves_per_group, int last_blocks_first, int merge,
+                                            hipStream_t stream) {
     CPMCU_REQUIRE(n > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_mfma: bad shape n=%d heads=%d kv_heads=%d", n, nh, nkv);
     CPMCU_REQUIRE(hd >= 16 && hd <= 128 && hd % 16 == 0,
                   "attention_mfma: head_dim %d has no matrix-core kernel (16, 32, ... 128 have; the plain kernel takes the rest)", hd);
@@ -495,7 +496,9 @@ extern "C" const char* cpmcu_attention_mfma(const void* q, void* out, float* par
 #undef BY_NW
 #undef LAUNCH
     CPMCU_LAUNCH_CHECK("attention_mfma");
-    if (n_splits > 1) {
+    // merge == 0 leaves the shares (part_o, part_ml) for a consumer that merges them itself
+    // (gemm.hip: cpmcu_gemm_skinny_shares); `out` is then not written
+    if (n_splits > 1 && merge) {
         attention_combine_kernel<<<(unsigned)((long)n * nh), hd > 64 ? 128 : 64, 0, stream>>>(
             part_o, (const float2*)part_ml, (bf16_t*)out, hd, n_splits);
         CPMCU_LAUNCH_CHECK("attention_combine");

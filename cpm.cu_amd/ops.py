@@ -248,7 +248,7 @@ def attention_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hd: in
                    positions: torch.Tensor, tok_slot: torch.Tensor, n_splits: int = 1,
                    part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None,
                    sel_blocks: Optional[torch.Tensor] = None, sel_count: Optional[torch.Tensor] = None,
-                   block_size: int = 0, waves_per_group: int = 0, last_blocks_first: int = 0):
+                   block_size: int = 0, waves_per_group: int = 0, last_blocks_first: int = 0, merge: bool = True):
     """bf16 attention on the matrix cores (head_dim 16, 32, ... 128; pages and key blocks multiples of 32).
     With n_splits > 1 every token's keys are shared among n_splits wavefronts and merged afterwards;
     part_o float32 [n, nh, n_splits, hd] and part_ml float32 [n, nh, n_splits, 2] are its scratch.
@@ -274,7 +274,7 @@ def attention_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hd: in
         _p(q), _p(out), _p(part_o), _p(part_ml), c_int(n), c_int(nh), c_int(nkv), c_int(hd), c_float(scale),
         _p(kpool), _p(vpool), _p(page_table), c_int(page_table.shape[1]), c_int(page_size), _p(positions),
         _p(tok_slot), _p(sel_blocks), _p(sel_count), c_int(max_sel), c_int(block_size), c_int(n_splits),
-        c_int(waves_per_group), c_int(last_blocks_first), _stream()))
+        c_int(waves_per_group), c_int(last_blocks_first), c_int(1 if merge else 0), _stream()))
 
 
 def attention_prefill_tokens_per_wave(nh: int, nkv: int, tiles_per_wave: int = 4) -> int:
@@ -536,6 +536,31 @@ def gemm_skinny(x: torch.Tensor, w, out: torch.Tensor, alpha: float = 1.0, mode:
                                             c_float(row_scale.eps if row_scale is not None else 0.0), _stream()))
 
 
+def gemm_skinny_shares(part_o: torch.Tensor, part_ml: torch.Tensor, w: "TiledWeight", out: torch.Tensor,
+                       alpha: float = 1.0, mode: str = "plain"):
+    """The skinny product whose x is the merged output of a split-KV attention, given as its shares: part_o
+    float32 [m, heads, shares, hd], part_ml float32 [m, heads, shares, 2] (attention_mfma with merge=False);
+    x[m, head*hd + d] = merged, rounded to bfloat16 as the merge kernel would.  w tiled [N, heads*hd]; out float32
+    [m, N] ('plain') or [S, m, N] ('partial')."""
+    _need(part_o, "attention shares", torch.float32, (None, None, None, None))
+    M, nh, S, hd = part_o.shape
+    _need(part_ml, "attention share stats", torch.float32, (M, nh, S, 2))
+    if not isinstance(w, TiledWeight) or w.K != nh * hd:
+        raise KernelError(f"gemm_skinny_shares: the weight must be tiled for K = {nh * hd}")
+    N = w.N
+    if mode == "plain":
+        _need(out, "gemm out", torch.float32, (M, N))
+        ksplit, omode = 1, 0
+    elif mode == "partial":
+        _need(out, "gemm partial sums", torch.float32, (None, M, N))
+        ksplit, omode = out.shape[0], 1
+    else:
+        raise KernelError(f"gemm_skinny_shares: unknown mode '{mode}'")
+    _check(_fn("gemm", "cpmcu_gemm_skinny_shares")(_p(part_o), _p(part_ml), c_int(S), c_int(nh), c_int(hd), _p(w.data),
+                                                   _p(out), c_long(N), c_int(omode), c_int(M), c_int(N),
+                                                   c_int(ksplit), c_float(alpha), _stream()))
+
+
 SKINNY_MAX_ROWS = 64
 
 
@@ -584,9 +609,18 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, alpha: float = 1
     gemm_nt_plain(x, w, out, alpha)
 
 
+# rows up to which the output projection merges the shares of a split-KV attention itself (the shares are
+# n_splits times the size of the merged rows and every workgroup of the product reads them: beyond two rows
+# that costs more than the merge kernel it saves; MI355X, 8B shape, one sequence at 4,096 keys: 3.47 against
+# 3.57 ms a step)
+ATTENTION_SHARES_MAX_ROWS = 2
+
+
 def attention(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, ctx,
-              sel_blocks=None, sel_count=None, block_size=0, window_blocks=0):
-    """Attention of the step's queries over the cache, with the kernel that suits the step."""
+              sel_blocks=None, sel_count=None, block_size=0, window_blocks=0, leave_shares=False):
+    """Attention of the step's queries over the cache, with the kernel that suits the step.
+    With ``leave_shares`` a split-KV attention of few rows is not merged: (part_o, part_ml) are returned for
+    gemm_skinny_shares, and ``out`` is not written; otherwise, and always when None is returned, out is."""
     if sel_count is None and not ctx.single_token and attention_mfma_ok(q, hd, page_size):
         r, nw = attention_prefill_shape(q.shape[0], nh, nkv, hd)
         tpw = attention_prefill_tokens_per_wave(nh, nkv, r)
@@ -603,12 +637,19 @@ def attention(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, c
         if sel_count is not None:
             keys = min(keys, sel_blocks.shape[2] * block_size)
         splits = attention_splits(n, nkv, nh // nkv, keys)
+        # up to 8,192 keys 8 shares serve as well as 16; beyond, more shares and the merge kernel win
+        # (one sequence at 16,384 keys: 4.03 ms a step with 8 shares merged by the product, 3.91 with 16)
+        want_shares = leave_shares and n <= ATTENTION_SHARES_MAX_ROWS and hd % 8 == 0 and keys <= 8192
+        if want_shares:
+            splits = min(splits, 8)          # what the product that merges them takes
         part_o = part_ml = None
         if splits > 1:
             part_o = ctx.ws.get("attn.part_o", (n, nh, splits, hd), torch.float32)
             part_ml = ctx.ws.get("attn.part_ml", (n, nh, splits, 2), torch.float32)
+        leave = want_shares and splits > 1
         attention_mfma(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, ctx.positions, ctx.tok_slot,
-                       splits, part_o, part_ml, sel_blocks, sel_count, block_size, last_blocks_first=window_blocks)
-        return
+                       splits, part_o, part_ml, sel_blocks, sel_count, block_size, last_blocks_first=window_blocks,
+                       merge=not leave)
+        return (part_o, part_ml) if leave else None
     attention_plain(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, ctx.positions, ctx.tok_slot,
                     sel_blocks, sel_count, block_size)

@@ -104,11 +104,22 @@ class GQAAttention(Mixer):
                       cache.page_table, cache.page_size, ctx, sel_blocks, sel_count, bs, window_blocks)
         return out
 
+    def attend_and_project(self, q, ctx: StepContext, cache: CacheView, sel=None) -> torch.Tensor:
+        """attend, then the output projection; for steps of one or two tokens the projection merges the shares
+        of the split-KV attention itself (one kernel of the chain less)."""
+        sel_blocks, sel_count, bs, window_blocks = sel if sel is not None else (None, None, 0, 0)
+        out = ctx.ws.get("attn.out", tuple(q.shape), q.dtype)
+        shares = ops.attention(q, out, self.nh, self.nkv, self.hd, self.scale, cache.streams["k"],
+                               cache.streams["v"], cache.page_table, cache.page_size, ctx, sel_blocks, sel_count, bs,
+                               window_blocks, leave_shares=self.o.takes_attention_shares())
+        if shares is not None:
+            return self.o.forward_shares(shares[0], shares[1], ctx, "attn.o")
+        return self.o.forward(out, ctx, "attn.o", out_dtype=torch.float32, partials=True)
+
     def forward(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool = True, row_scale=None
                 ) -> torch.Tensor:
         q = self.project_and_store(h, ctx, cache, writes_cache, row_scale)
-        a = self.attend(q, ctx, cache)
-        return self.o.forward(a, ctx, "attn.o", out_dtype=torch.float32, partials=True)
+        return self.attend_and_project(q, ctx, cache)
 
 
 @MIXERS.register("infllm_v2_attention")
@@ -154,5 +165,4 @@ class InfLLMv2Attention(GQAAttention):
                               self.init_blocks, self.topk, self.window_blocks, self.dense_len, ctx.max_pos,
                               sel_blocks, sel_count, scratch=scratch)
             sel = (sel_blocks, sel_count, self.bs, self.window_blocks)
-        a = self.attend(q, ctx, cache, sel)
-        return self.o.forward(a, ctx, "attn.o", out_dtype=torch.float32, partials=True)
+        return self.attend_and_project(q, ctx, cache, sel)
