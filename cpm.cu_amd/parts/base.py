@@ -177,7 +177,8 @@ class Mixer(Part):
         raise NotImplementedError
 
     def takes_row_scale(self, n: int, ctx: StepContext, cache: Optional[CacheView], writes_cache: bool) -> bool:
-        """True if forward, for this step of n tokens, accepts ``row_scale=`` (Norm.forward_unscaled) beside h."""
+        """True if forward, for this step of n tokens, accepts ``row_scale=`` (Norm.forward_unscaled) beside h.
+        A subclass that overrides forward of a mixer that says yes takes the argument too, or says no here."""
         return False
 
 
