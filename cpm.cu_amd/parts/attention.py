@@ -97,16 +97,10 @@ class GQAAttention(Mixer):
                        cache.page_table if writes_cache else None, cache.page_size, writes_cache)
         return q
 
-    def attend(self, q, ctx: StepContext, cache: CacheView, sel=None) -> torch.Tensor:
-        out = ctx.ws.get("attn.out", tuple(q.shape), q.dtype)
-        sel_blocks, sel_count, bs, window_blocks = sel if sel is not None else (None, None, 0, 0)
-        ops.attention(q, out, self.nh, self.nkv, self.hd, self.scale, cache.streams["k"], cache.streams["v"],
-                      cache.page_table, cache.page_size, ctx, sel_blocks, sel_count, bs, window_blocks)
-        return out
-
     def attend_and_project(self, q, ctx: StepContext, cache: CacheView, sel=None) -> torch.Tensor:
-        """attend, then the output projection; for steps of one or two tokens the projection merges the shares
-        of the split-KV attention itself (one kernel of the chain less)."""
+        """Attention of q over the cache (all keys up to each query, or the blocks listed in ``sel``), then the
+        output projection; for steps of one or two tokens the projection merges the shares of the split-KV
+        attention itself (one kernel of the chain less)."""
         sel_blocks, sel_count, bs, window_blocks = sel if sel is not None else (None, None, 0, 0)
         out = ctx.ws.get("attn.out", tuple(q.shape), q.dtype)
         shares = ops.attention(q, out, self.nh, self.nkv, self.hd, self.scale, cache.streams["k"],
