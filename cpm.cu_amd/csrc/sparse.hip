@@ -421,6 +421,7 @@ __global__ __launch_bounds__(NW * 64) void sparse_select_mfma_kernel(
     const int q_block = p / sp.bs;
     const int n_cand = max(q_block - sp.window_blocks + 1, 0);
     const int rows_per_page = pv.page_size / sp.st;
+    const unsigned rpp_magic = (unsigned)(((1ull << 32) + rows_per_page - 1) / (unsigned)rows_per_page);
     const float scale_log2e = sp.scale * 1.4426950408889634f;
     const int n_tiles = (n_vis + 15) / 16;
 
@@ -441,11 +442,16 @@ __global__ __launch_bounds__(NW * 64) void sparse_select_mfma_kernel(
         // The wavefront's tiles of 16 compressed keys in turn, f(tile, scores).  B operand: lane (key n, g) holds
         // CK[key][32*ks + 8g .. +8].  A tile's page is looked up two tiles ahead and its keys are asked for one
         // tile ahead, so that neither latency stands between two tiles' arithmetic.
-        auto page_of = [&](int tile) { return ptab[min(tile * 16 + n, n_vis - 1) / rows_per_page]; };
-        auto load_b = [&](int tile, int page, sbf16x8_t (&b)[KSTEPS]) {
+        // (a division by rows_per_page for every tile and lane would be a third of this kernel's vector
+        // instructions: floor(j / r) = umulhi(j, ceil(2^32 / r)) for j < 2^32 / r)
+        auto locate = [&](int tile, int& page, int& row) {
             const int j = min(tile * 16 + n, n_vis - 1);
-            const bf16_t* ck = ckpool + ck_index(page, j % rows_per_page, kvh, sp.nkv, HD, rows_per_page) +
-                               g * rows_per_page * 8;
+            const int pg = rows_per_page == 1 ? j : (int)__umulhi((unsigned)j, rpp_magic);
+            row = j - pg * rows_per_page;
+            page = ptab[pg];
+        };
+        auto load_b = [&](int page, int row, sbf16x8_t (&b)[KSTEPS]) {
+            const bf16_t* ck = ckpool + ck_index(page, row, kvh, sp.nkv, HD, rows_per_page) + g * rows_per_page * 8;
 #pragma unroll
             for (int ks = 0; ks < KSTEPS; ++ks) {
                 sbf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -456,11 +462,14 @@ __global__ __launch_bounds__(NW * 64) void sparse_select_mfma_kernel(
         auto for_tiles = [&](auto f) {
             if (wave >= n_tiles) return;
             sbf16x8_t b[KSTEPS], bn[KSTEPS];
-            load_b(wave, page_of(wave), b);
-            int page_next = page_of(wave + NW);               // (tiles beyond the last repeat the last key)
+            int page, row, page_next, row_next;
+            locate(wave, page, row);
+            load_b(page, row, b);
+            locate(wave + NW, page_next, row_next);           // (tiles beyond the last repeat the last key)
             for (int tile = wave; tile < n_tiles; tile += NW) {
-                const int page_after = page_of(tile + 2 * NW);
-                load_b(tile + NW, page_next, bn);
+                int page_after, row_after;
+                locate(tile + 2 * NW, page_after, row_after);
+                load_b(page_next, row_next, bn);
                 sfloatx4_t st = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int ks = 0; ks < KSTEPS; ++ks) st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ks], b[ks], st, 0, 0, 0);
@@ -468,6 +477,7 @@ __global__ __launch_bounds__(NW * 64) void sparse_select_mfma_kernel(
 #pragma unroll
                 for (int ks = 0; ks < KSTEPS; ++ks) b[ks] = bn[ks];
                 page_next = page_after;
+                row_next = row_after;
             }
         };
         // pass 1: running max and sum per head, per lane
