@@ -331,15 +331,16 @@ def prefill_tiles(q_lens: Sequence[int], tokens_per_wave: int, device) -> torch.
 
 def attention_splits(n_tokens: int, nkv: int, group: int, max_keys: int) -> int:
     """Shares of a token's keys for steps of few tokens.  Measured on the MI355X (head size 128, 2 kv heads,
-    workgroups of 4 wavefronts, graph replay, attention + merge): 8 sequences at 4,096 keys 60/36/24/17/18/25 us
-    for 1/2/4/8/16/32 shares; 64 sequences 68/46/50/51/59 us; 8 sequences at 32,768 keys 124/68/50/60 us for
-    4/8/16/32; one sequence at 16,384 keys 25/16/14/16/25 us for 4/8/16/32/64, at 65,536 keys 46/31/26/33 us for
-    8/16/32/64 (the merge reads every share).  So: about 256 workgroups in all, a share of at least 512 keys,
-    and at most 16 shares (32 from 64k keys on)."""
+    workgroups of 4 wavefronts, graph replay, attention + merge, in us for 1/2/4/8/16/32 shares):
+      8 sequences at 4,096 keys 22/17/13/11/12/18, at 16,384 keys 72/42/30/26/28/32, at 32,768 149/84/55/48/48/53;
+      16 sequences at 4,096 keys 25/18/17/17/20/27; 32 sequences 28/25/26/28/31/37; 64 sequences 47/46/48/50/52/68;
+      one sequence at 16,384 keys 71/39/25/16/14/16, at 65,536 keys 296/154/83/46/31/26.
+    So: about 128 workgroups in all but at least 2 shares, a share of at least 512 keys, and at most 16 shares
+    (32 from 64k keys on: the merge reads every share)."""
     if n_tokens > 256:
         return 1
     groups = n_tokens * nkv * -(-group // 16)
-    return max(1, min(256 // max(groups, 1), max_keys // 512, 16 if max_keys < 65536 else 32))
+    return max(1, min(max(128 // max(groups, 1), 2), max_keys // 512, 16 if max_keys < 65536 else 32))
 
 
 def compress_keys(kpool: torch.Tensor, ckpool: torch.Tensor, nkv: int, page_table: torch.Tensor, page_size: int,
