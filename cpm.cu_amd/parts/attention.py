@@ -59,7 +59,7 @@ class GQAAttention(Mixer):
         plain_rotation = self.position is None or self.position.rotary_params() is not None
         return (writes_cache and cache is not None and plain_rotation and n <= ops.QKV_ROPE_MAX_ROWS
                 and dtype == torch.bfloat16 and self.qkv.tiled is not None and self.hd % 16 == 0
-                and cache.page_size % 32 == 0)
+                and self.hidden_size % 8 == 0 and cache.page_size % 32 == 0)
 
     def takes_row_scale(self, n: int, ctx: StepContext, cache, writes_cache: bool) -> bool:
         return self._fused_projection(n, self.rt.dtype, cache, writes_cache)
