@@ -246,6 +246,10 @@ ODD = {
     "mha80": dict(num_hidden_layers=1, hidden_size=72, num_attention_heads=6, num_key_value_heads=6, head_dim=80,
                   intermediate_size=100, vocab_size=1001, rms_norm_eps=1e-5, rope_theta=10000.0,
                   max_position_embeddings=192, scale_emb=1, dim_model_base=72, scale_depth=1.0, tie_word_embeddings=True),
+    # a width that is a multiple of 4 only: the bfloat16 decode kernels that want 8 must step aside
+    "w100": dict(num_hidden_layers=2, hidden_size=100, num_attention_heads=4, num_key_value_heads=2, head_dim=32,
+                 intermediate_size=88, vocab_size=97, rms_norm_eps=1e-5, rope_theta=10000.0, max_position_embeddings=192,
+                 scale_emb=4, dim_model_base=50, scale_depth=1.4, tie_word_embeddings=True),
     # block-sparse attention with 5 query heads on one kv head and blocks of 32
     "sparse5": dict(num_hidden_layers=2, hidden_size=160, num_attention_heads=5, num_key_value_heads=1, head_dim=32,
                     intermediate_size=208, vocab_size=300, rms_norm_eps=1e-6, rope_theta=20000.0,
