@@ -31,6 +31,33 @@ __global__ void compress_keys_kernel(const T* __restrict__ kpool, T* __restrict_
     const int first = st * j;
     const int page = pv.page_table[(long)slot * pv.table_width + first / pv.page_size];
     const int rpp = pv.page_size / st;
+    if constexpr (sizeof(T) == 2) {
+        // bf16: a thread takes 8 neighbouring features, which lie in one 16-byte piece of every key and of
+        // the compressed key (head sizes are multiples of 16); the sums run over the keys in the same order
+        // as below, feature by feature
+        for (int e = threadIdx.x; e < width / 8; e += blockDim.x) {
+            const int kvh = (e * 8) / hd, d = e * 8 - kvh * hd;
+            float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+            for (int r = 0; r < ks; ++r) {
+                const uint4 u = *(const uint4*)(kpool + key_index(paged_row(pv, slot, first + r), kvh, nkv, hd) +
+                                                key_d_offset(d));
+                const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    acc[2 * j] += __uint_as_float(w[j] << 16);
+                    acc[2 * j + 1] += __uint_as_float(w[j] & 0xffff0000u);
+                }
+            }
+            uint32_t o[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                o[j] = (uint32_t)f32_to_bf16(acc[2 * j] / (float)ks).v | ((uint32_t)f32_to_bf16(acc[2 * j + 1] / (float)ks).v << 16);
+            *(uint4*)(ckpool + ck_index(page, (first % pv.page_size) / st, kvh, nkv, hd, rpp) + ck_d_offset(d, rpp)) =
+                make_uint4(o[0], o[1], o[2], o[3]);
+        }
+        return;
+    }
     for (int e = threadIdx.x; e < width; e += blockDim.x) {
         float s = 0.f;
         const int kvh = e / hd, d = e - kvh * hd;
