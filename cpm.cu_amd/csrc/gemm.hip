@@ -118,8 +118,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
                                                              const bf16_t* __restrict__ W, long ldw,
                                                              OT* __restrict__ Y, long ldy, int M, int N, int K, int KS,
                                                              float alpha, int I, long part_stride,
-                                                             const float* __restrict__ row_ss, float eps,
-                                                             XShares xsh) {
+                                                             const float* __restrict__ row_ss, int ss_slices,
+                                                             float eps, XShares xsh) {
     static_assert(MODE != 2 || SPW == 2, "gated output pairs a gate strip with an up strip");
     constexpr int NT = NW * 64;
     constexpr int XV = MT * 16 * 64 / NT;     // 16-byte vectors of X a thread stages per chunk
@@ -242,7 +242,7 @@ if (TILED) {
     // X may be x * w of a norm whose row factor is still to come (common.h: row_scales); the loop's first
     // barrier makes rs_s visible
     __shared__ float rs_s[MT * 16];
-    if (row_ss) row_scales<NT, MT * 16>(row_ss, (K + NORM_SLICE - 1) / NORM_SLICE, M, 1.0f / (float)K, eps, rs_s);
+    if (row_ss) row_scales<NT, MT * 16>(row_ss, ss_slices, M, 1.0f / (float)K, eps, rs_s);
     const int nchunk = (nkb + 3) / 4;
     for (int c = 0; c < nchunk; ++c) {
         __syncthreads();
@@ -296,12 +296,13 @@ if (TILED) {
 
 // out_mode: 0 = Y[m,N] in out_dtype; 1 = float partial sums Y[ksplit][m][N]; 2 = gated (N = 2*I rows of W, Y[m,I] bf16)
 // variant (gated output only): 0 = 4 waves a workgroup, 1 = 2 waves
-// row_ss (or null): X is x * w of add_norm_columns, whose sums of squares [M][ceil(K/64)] these are; the
-// output is multiplied by rsqrt(sum / K + eps) row by row
+// row_ss (or null): X is x * w of a norm cut by columns, whose sums of squares [M][ss_slices] these are (a
+// slice for every 64 columns after add_norm_columns, for every 16 after proj_add_norm); the output is multiplied
+// by rsqrt(sum of the row's slices / K + eps) row by row
 extern "C" const char* cpmcu_gemm_skinny_v(const void* X, long ldx, const void* W, long ldw, void* Y, long ldy,
                                            int out_dtype, int out_mode, int M, int N, int K, int ksplit, float alpha,
-                                           int variant, int tiled, const float* row_ss, float eps,
-                                           hipStream_t stream) {
+                                           int variant, int tiled, const float* row_ss, int ss_slices,
+                                           float eps, hipStream_t stream) {
     CPMCU_REQUIRE(M > 0 && M <= 64, "gemm_skinny: %d rows (1..64 are taken; more rows belong to the tiled product)", M);
     CPMCU_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "gemm_skinny: K=%d must be a positive multiple of 8 (N=%d)", K, N);
     CPMCU_REQUIRE(ldx % 8 == 0 && ldx >= K && (tiled || (ldw % 8 == 0 && ldw >= K)),
@@ -325,11 +326,11 @@ extern "C" const char* cpmcu_gemm_skinny_v(const void* X, long ldx, const void* 
         if (tiled)                                                                                                \
             gemm_skinny_kernel<MTv, MODEv, OT, SPW, NW, true><<<grid, NW * 64, 0, stream>>>(                      \
                 (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (OT*)Y, ldy, M, N, K, KS, alpha, I, part_stride,    \
-                row_ss, eps, XShares{});                                                                          \
+                row_ss, ss_slices, eps, XShares{});                                                               \
         else                                                                                                      \
             gemm_skinny_kernel<MTv, MODEv, OT, SPW, NW, false><<<grid, NW * 64, 0, stream>>>(                     \
                 (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (OT*)Y, ldy, M, N, K, KS, alpha, I, part_stride,    \
-                row_ss, eps, XShares{});                                                                          \
+                row_ss, ss_slices, eps, XShares{});                                                               \
     } while (0)
 // shapes that measured best: one strip a wave in workgroups of 4 waves; gated output in workgroups of
 // 2 waves up to 16 rows of X (variant 1), of 4 waves above (variant 0)
@@ -362,10 +363,10 @@ extern "C" const char* cpmcu_gemm_skinny_v(const void* X, long ldx, const void* 
 // workgroups balance better over 256 CUs); gated output with 2 waves a workgroup up to 16 rows.
 extern "C" const char* cpmcu_gemm_skinny(const void* X, long ldx, const void* W, long ldw, void* Y, long ldy,
                                          int out_dtype, int out_mode, int M, int N, int K, int ksplit, float alpha,
-                                         int tiled, const float* row_ss, float eps, hipStream_t stream) {
+                                         int tiled, const float* row_ss, int ss_slices, float eps, hipStream_t stream) {
     const int variant = out_mode == 2 ? (M <= 16 ? 1 : 0) : 2;
     return cpmcu_gemm_skinny_v(X, ldx, W, ldw, Y, ldy, out_dtype, out_mode, M, N, K, ksplit, alpha, variant, tiled,
-                               row_ss, eps, stream);
+                               row_ss, ss_slices, eps, stream);
 }
 
 // The same product with X given as attention shares (see XShares): rows = tokens (at most 16), K = nh * hd,
@@ -388,10 +389,10 @@ extern "C" const char* cpmcu_gemm_skinny_shares(const float* part_o, const float
     dim3 grid((N + 63) / 64, ksplit);
     if (out_mode == 0)
         gemm_skinny_kernel<1, 0, float, 1, 4, true, true><<<grid, 256, 0, stream>>>(
-            nullptr, K, (const bf16_t*)W, K, (float*)Y, ldy, M, N, K, KS, alpha, N / 2, (long)M * ldy, nullptr, 0.f, xsh);
+            nullptr, K, (const bf16_t*)W, K, (float*)Y, ldy, M, N, K, KS, alpha, N / 2, (long)M * ldy, nullptr, 0, 0.f, xsh);
     else
         gemm_skinny_kernel<1, 1, float, 1, 4, true, true><<<grid, 256, 0, stream>>>(
-            nullptr, K, (const bf16_t*)W, K, (float*)Y, ldy, M, N, K, KS, alpha, N / 2, (long)M * ldy, nullptr, 0.f, xsh);
+            nullptr, K, (const bf16_t*)W, K, (float*)Y, ldy, M, N, K, KS, alpha, N / 2, (long)M * ldy, nullptr, 0, 0.f, xsh);
     CPMCU_LAUNCH_CHECK("gemm_skinny_shares");
     return nullptr;
 }

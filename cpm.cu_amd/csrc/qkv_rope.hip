@@ -26,8 +26,8 @@ __global__ __launch_bounds__(NW * 64) void qkv_rope_kernel(
     const bf16_t* __restrict__ X, long ldx, const bf16_t* __restrict__ W, int M, int K, bf16_t* __restrict__ q_out,
     int nh, int nkv, int hd, const int* __restrict__ positions, const int* __restrict__ tok_slot,
     const float* __restrict__ inv_freq, float mscale, bf16_t* __restrict__ kpool, bf16_t* __restrict__ vpool,
-    PagedView pv, const float* __restrict__ row_ss, float eps, bf16_t* __restrict__ ckpool, int ck_size,
-    int ck_stride) {
+    PagedView pv, const float* __restrict__ row_ss, int ss_slices, float eps, bf16_t* __restrict__ ckpool,
+    int ck_size, int ck_stride) {
     __shared__ float red[NW - 1][MT][4][64];
     __shared__ float rs_s[MT * 16];            // the norm's row factors (common.h: row_scales), if x lacks them
     const int strip = blockIdx.x;
@@ -67,7 +67,7 @@ __global__ __launch_bounds__(NW * 64) void qkv_rope_kernel(
     };
 #pragma unroll
     for (int j = 0; j < PF; ++j) load_block(kb0 + j, a[j], bx[j]);
-    if (row_ss) row_scales<NW * 64, MT * 16>(row_ss, (K + NORM_SLICE - 1) / NORM_SLICE, M, 1.0f / (float)K, eps, rs_s);
+    if (row_ss) row_scales<NW * 64, MT * 16>(row_ss, ss_slices, M, 1.0f / (float)K, eps, rs_s);
     int kb = kb0;
     for (; kb + 2 * PF <= kb1; kb += PF) {           // every block and every block asked for exists
 #pragma unroll
@@ -204,7 +204,7 @@ extern "C" const char* cpmcu_qkv_rope(const void* X, long ldx, const void* W, in
                                       int nkv, int hd, const int* positions, const int* tok_slot,
                                       const float* inv_freq, float mscale, void* kpool, void* vpool,
                                       const int* page_table, int table_width, int page_size, const float* row_ss,
-                                      float eps, void* ckpool, int ck_size, int ck_stride, hipStream_t stream) {
+                                      int ss_slices, float eps, void* ckpool, int ck_size, int ck_stride, hipStream_t stream) {
     CPMCU_REQUIRE(M > 0 && M <= 32, "qkv_rope: %d tokens (1..32 are taken; more go through the split product and the rotary kernel)", M);
     CPMCU_REQUIRE(nh > 0 && nkv > 0 && hd > 0 && hd % 16 == 0, "qkv_rope: bad shape heads=%d kv_heads=%d head_dim=%d", nh, nkv, hd);
     CPMCU_REQUIRE(K > 0 && K % 8 == 0 && ldx % 8 == 0 && ldx >= K, "qkv_rope: K=%d, row stride %ld must be multiples of 8", K, ldx);
@@ -219,7 +219,7 @@ extern "C" const char* cpmcu_qkv_rope(const void* X, long ldx, const void* W, in
 #define LAUNCH(MTv)                                                                                              \
     qkv_rope_kernel<4, 4, MTv><<<strips, 256, 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, M, K, (bf16_t*)q_out, \
                                                            nh, nkv, hd, positions, tok_slot, inv_freq, mscale,       \
-                                                           (bf16_t*)kpool, (bf16_t*)vpool, pv, row_ss, eps,      \
+                                                           (bf16_t*)kpool, (bf16_t*)vpool, pv, row_ss, ss_slices, eps, \
                                                            (bf16_t*)ckpool, ck_size, ck_stride)
     if (M <= 16) LAUNCH(1);
     else LAUNCH(2);

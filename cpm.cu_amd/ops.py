@@ -117,9 +117,10 @@ NORM_COLUMNS_MAX_ROWS = 16
 
 
 class RowScale:
-    """What a product needs to finish a norm that add_norm_columns began: the rows' sums of squares by slices
-    of NORM_SLICE columns, float32 [n, ceil(H / NORM_SLICE)], and eps.  The product multiplies its rows by
-    rsqrt(sum / H + eps), H being its own input width."""
+    """What a product needs to finish a norm cut by columns: the rows' sums of squares by slices of columns,
+    float32 [n, slices] (a slice for every NORM_SLICE columns after add_norm_columns, for every 16 after
+    proj_add_norm), and eps.  The product multiplies its rows by rsqrt(sum of the row's slices / H + eps), H
+    being its own input width."""
     __slots__ = ("sums", "eps")
 
     def __init__(self, sums: torch.Tensor, eps: float):
@@ -472,7 +473,7 @@ def qkv_rope(x: torch.Tensor, w: TiledWeight, q_out: torch.Tensor, nh: int, nkv:
     _need(x, "qkv x", torch.bfloat16, (None, w.K))
     n = x.shape[0]
     if row_scale is not None:
-        _need(row_scale.sums, "qkv row sums", torch.float32, (n, norm_slices(w.K)))
+        _need(row_scale.sums, "qkv row sums", torch.float32, (n, None))
     ckpool, ks, st = compress if compress is not None else (None, 0, 0)
     if ckpool is not None:
         # (compressed key pool, kernel_size, kernel_stride): the step's tokens also complete their compressed keys
@@ -494,8 +495,33 @@ def qkv_rope(x: torch.Tensor, w: TiledWeight, q_out: torch.Tensor, nh: int, nkv:
                                         c_float(mscale), _p(kpool), _p(vpool), _p(page_table),
                                         c_int(page_table.shape[1]), c_int(page_size),
                                         _p(row_scale.sums if row_scale is not None else None),
+                                        c_int(row_scale.sums.shape[1] if row_scale is not None else 0),
                                         c_float(row_scale.eps if row_scale is not None else 0.0),
                                         _p(ckpool), c_int(ks), c_int(st), _stream()))
+
+
+PROJ_NORM_MAX_ROWS = 16
+
+
+def proj_add_norm(a: torch.Tensor, w: "TiledWeight", alpha: float, x: torch.Tensor, weight: torch.Tensor,
+                  out: torch.Tensor, sums: torch.Tensor):
+    """A branch's last product fused with the residual add and the column part of the norm that follows, for a
+    step of at most 32 tokens: x += alpha * (a . w^T) in place (x float32 [n, N], a bfloat16 [n, K], w tiled
+    [N, K]); out = bfloat16(x * weight); sums[r, s] = sum of x[r]^2 over the 16 columns of strip s (float32
+    [n, ceil(N / 16)]).  As after add_norm_columns, the product that reads `out` applies the row factor."""
+    _need(a, "proj a", torch.bfloat16, (None, None))
+    n, K = a.shape
+    if not isinstance(w, TiledWeight) or w.K != K:
+        raise KernelError(f"proj_add_norm: the weight must be tiled for K = {K}")
+    N = w.N
+    if N % 4 or K % 8:
+        raise KernelError(f"proj_add_norm: N={N} must be a multiple of 4 and K={K} of 8")
+    _need(x, "proj residual", torch.float32, (n, N))
+    _need(weight, "proj norm weight", torch.float32, (N,))
+    _need(out, "proj out", torch.bfloat16, (n, N))
+    _need(sums, "proj row sums", torch.float32, (n, -(-N // 16)))
+    _check(_fn("qkv", "cpmcu_proj_add_norm")(_p(a), c_long(K), _p(w.data), c_int(n), c_int(N), c_int(K),
+                                             c_float(alpha), _p(x), _p(weight), _p(out), _p(sums), _stream()))
 
 
 def gemm_skinny(x: torch.Tensor, w, out: torch.Tensor, alpha: float = 1.0, mode: str = "plain",
@@ -509,7 +535,7 @@ def gemm_skinny(x: torch.Tensor, w, out: torch.Tensor, alpha: float = 1.0, mode:
     _need(x, "gemm x", torch.bfloat16, (None, None))
     M, K = x.shape
     if row_scale is not None:
-        _need(row_scale.sums, "gemm row sums", torch.float32, (M, norm_slices(K)))
+        _need(row_scale.sums, "gemm row sums", torch.float32, (M, None))
     tiled = isinstance(w, TiledWeight)
     if tiled:
         if w.K != K:
@@ -534,6 +560,7 @@ def gemm_skinny(x: torch.Tensor, w, out: torch.Tensor, alpha: float = 1.0, mode:
                                             c_int(_code(out)), c_int(omode), c_int(M), c_int(N), c_int(K),
                                             c_int(ksplit), c_float(alpha), c_int(1 if tiled else 0),
                                             _p(row_scale.sums if row_scale is not None else None),
+                                            c_int(row_scale.sums.shape[1] if row_scale is not None else 0),
                                             c_float(row_scale.eps if row_scale is not None else 0.0), _stream()))
 
 

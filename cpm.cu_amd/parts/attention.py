@@ -23,7 +23,7 @@ import torch
 
 from .. import ops
 from ..cache.paged import CacheNeeds, CacheView, StreamSpec
-from .base import MIXERS, Mixer, Part, PositionEncoding, Runtime, StepContext
+from .base import MIXERS, DeferredBranch, Mixer, Part, PositionEncoding, Runtime, StepContext
 from .linear import Linear
 
 
@@ -97,7 +97,9 @@ class GQAAttention(Mixer):
                        cache.page_table if writes_cache else None, cache.page_size, writes_cache)
         return q
 
-    def attend_and_project(self, q, ctx: StepContext, cache: CacheView, sel=None) -> torch.Tensor:
+    can_defer_last = True
+
+    def attend_and_project(self, q, ctx: StepContext, cache: CacheView, sel=None, defer_last: bool = False):
         """Attention of q over the cache (all keys up to each query, or the blocks listed in ``sel``), then the
         output projection; for steps of one or two tokens the projection merges the shares of the split-KV
         attention itself (one kernel of the chain less)."""
@@ -108,12 +110,16 @@ class GQAAttention(Mixer):
                                window_blocks, leave_shares=self.o.takes_attention_shares())
         if shares is not None:
             return self.o.forward_shares(shares[0], shares[1], ctx, "attn.o")
+        if defer_last and self.o.defers(out):
+            # steps of more tokens (measured for one token: the product that merges the shares and a norm
+            # kernel, 296 tokens/s, against a merge kernel and the product that does the norm's work, 290)
+            return DeferredBranch(self.o, out, ctx, "attn.o")
         return self.o.forward(out, ctx, "attn.o", out_dtype=torch.float32, partials=True)
 
-    def forward(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool = True, row_scale=None
-                ) -> torch.Tensor:
+    def forward(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool = True, row_scale=None,
+                defer_last: bool = False):
         q = self.project_and_store(h, ctx, cache, writes_cache, row_scale)
-        return self.attend_and_project(q, ctx, cache)
+        return self.attend_and_project(q, ctx, cache, defer_last=defer_last)
 
 
 @MIXERS.register("infllm_v2_attention")
@@ -134,8 +140,8 @@ class InfLLMv2Attention(GQAAttention):
         w = self.nkv * self.hd
         return CacheNeeds(streams=(("k", StreamSpec(w)), ("v", StreamSpec(w)), ("ck", StreamSpec(w, every=self.st))))
 
-    def forward(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool = True, row_scale=None
-                ) -> torch.Tensor:
+    def forward(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool = True, row_scale=None,
+                defer_last: bool = False):
         # decode steps: the projection kernel completes the compressed keys itself (one kernel of the chain less)
         fused = self._fused_projection(h.shape[0], h.dtype, cache, writes_cache)
         q = self.project_and_store(h, ctx, cache, writes_cache, row_scale,
@@ -159,4 +165,4 @@ class InfLLMv2Attention(GQAAttention):
                               self.init_blocks, self.topk, self.window_blocks, self.dense_len, ctx.max_pos,
                               sel_blocks, sel_count, scratch=scratch)
             sel = (sel_blocks, sel_count, self.bs, self.window_blocks)
-        return self.attend_and_project(q, ctx, cache, sel)
+        return self.attend_and_project(q, ctx, cache, sel, defer_last=defer_last)

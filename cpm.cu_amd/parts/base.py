@@ -16,6 +16,11 @@ Kinds of parts and what each must provide:
 * ``Block``:     forward(stream, ctx, cache, writes_cache): the arrangement of the above
                  around the residual stream
 
+Two optional protocols let neighbouring parts share a kernel without knowing each other: a norm may leave
+its row factor to the product that follows (``forward_unscaled`` / ``takes_row_scale``), and a part may leave
+its last product to the norm that follows (``DeferredBranch``: ``can_defer_last`` /
+``takes_deferred_branch``).  A part that implements neither is handed plain tensors.
+
 Branches may come back as float partial sums ``[P, n, H]`` of a split matrix
 product; whoever adds them to the residual sums them.
 """
@@ -107,12 +112,47 @@ class StepContext:
     perf: Optional[object] = None                 # label-keyed timers (utils.perf.PerfTimers) when switched on
 
 
-@dataclass
+class DeferredBranch:
+    """A branch whose last linear layer has not run yet: branch = ``linear``(``a``).  A part that is asked to
+    (``forward(..., defer_last=True)``) may hand this back instead of a tensor; a norm that knows a kernel which
+    runs that product together with the residual add takes it as it is (``Norm.takes_deferred_branch``), for
+    everybody else ``evaluate()`` runs the product as the part would have and gives the tensor."""
+
+    def __init__(self, linear, a: torch.Tensor, ctx: "StepContext", tag: str):
+        self.linear, self.a, self.ctx, self.tag = linear, a, ctx, tag
+        self._value: Optional[torch.Tensor] = None
+
+    def evaluate(self) -> torch.Tensor:
+        if self._value is None:
+            self._value = self.linear.forward(self.a, self.ctx, self.tag, out_dtype=torch.float32, partials=True)
+        return self._value
+
+
+def branch_tensor(branch):
+    """The branch as a tensor (or None), whatever form it was handed over in."""
+    return branch.evaluate() if isinstance(branch, DeferredBranch) else branch
+
+
 class ResidualStream:
-    """The float residual ``x`` [n, H] and a branch not yet added to it."""
-    x: torch.Tensor
-    pending: Optional[torch.Tensor] = None
-    pending_scale: float = 1.0
+    """The float residual ``x`` [n, H] and a branch not yet added to it.  ``pending`` reads as a tensor;
+    ``take_pending()`` gives it in the form it was left in, which may be a DeferredBranch."""
+
+    def __init__(self, x: torch.Tensor, pending=None, pending_scale: float = 1.0):
+        self.x = x
+        self._pending = pending
+        self.pending_scale = pending_scale
+
+    @property
+    def pending(self) -> Optional[torch.Tensor]:
+        self._pending = branch_tensor(self._pending)
+        return self._pending
+
+    @pending.setter
+    def pending(self, value):
+        self._pending = value
+
+    def take_pending(self):
+        return self._pending
 
 
 # ---------------------------------------------------------------------------
@@ -155,6 +195,9 @@ class Norm(Part):
         consumer's takes_row_scale() said yes."""
         return None
 
+    # True if forward and forward_unscaled accept a DeferredBranch as ``branch``
+    takes_deferred_branch = False
+
 
 class PositionEncoding(Part):
     def rotary_params(self) -> Optional[Tuple[torch.Tensor, float]]:
@@ -181,6 +224,9 @@ class Mixer(Part):
         A subclass that overrides forward of a mixer that says yes takes the argument too, or says no here."""
         return False
 
+    # True if forward accepts ``defer_last=True`` and may then return a DeferredBranch
+    can_defer_last = False
+
 
 class FeedForward(Part):
     def forward(self, h: torch.Tensor, ctx: StepContext) -> torch.Tensor:
@@ -189,6 +235,9 @@ class FeedForward(Part):
     def takes_row_scale(self, n: int, ctx: StepContext) -> bool:
         """True if forward, for this step of n tokens, accepts ``row_scale=`` (Norm.forward_unscaled) beside h."""
         return False
+
+    # True if forward accepts ``defer_last=True`` and may then return a DeferredBranch
+    can_defer_last = False
 
 
 class Block(Part):

@@ -8,10 +8,18 @@ model's final norm).
 """
 from __future__ import annotations
 
+import inspect
 from typing import List, Optional
 
 from ..cache.paged import CacheView
-from .base import BLOCKS, Block, FeedForward, Mixer, Norm, Part, ResidualStream, StepContext
+from .base import BLOCKS, Block, FeedForward, Mixer, Norm, Part, ResidualStream, StepContext, branch_tensor
+
+
+def _accepts(fn, name: str) -> bool:
+    try:
+        return name in inspect.signature(fn).parameters
+    except (TypeError, ValueError):
+        return False
 
 
 @BLOCKS.register("pre_norm")
@@ -23,6 +31,10 @@ class PreNormBlock(Block):
         self.ff_norm = ff_norm
         self.feed_forward = feed_forward
         self.residual_scale = float(residual_scale)
+        # a part that can leave its last product to the norm after it is asked to (a subclass whose forward
+        # does not know the argument is not)
+        self._mixer_defers = mixer.can_defer_last and _accepts(mixer.forward, "defer_last")
+        self._ff_defers = feed_forward.can_defer_last and _accepts(feed_forward.forward, "defer_last")
 
     def parts(self) -> List[Part]:
         return [self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward]
@@ -31,6 +43,8 @@ class PreNormBlock(Block):
     def _normed(norm: Norm, deferred: bool, x, branch, branch_scale, ctx):
         """The normed rows and None, or (if the consumer finishes the norm itself) the rows without the norm's
         row factor and that factor's ingredients."""
+        if not norm.takes_deferred_branch:
+            branch = branch_tensor(branch)
         if deferred:
             hs = norm.forward_unscaled(x, branch, branch_scale, ctx, tag="block.h")
             if hs is not None:
@@ -40,18 +54,20 @@ class PreNormBlock(Block):
     def _mix(self, stream, ctx, cache, writes_cache):
         n = stream.x.shape[0]
         h, rs = self._normed(self.mixer_norm, self.mixer.takes_row_scale(n, ctx, cache, writes_cache),
-                             stream.x, stream.pending, stream.pending_scale, ctx)
-        if rs is None:
-            return self.mixer.forward(h, ctx, cache, writes_cache)
-        return self.mixer.forward(h, ctx, cache, writes_cache, row_scale=rs)
+                             stream.x, stream.take_pending(), stream.pending_scale, ctx)
+        kw = {"defer_last": True} if self._mixer_defers else {}
+        if rs is not None:
+            kw["row_scale"] = rs
+        return self.mixer.forward(h, ctx, cache, writes_cache, **kw)
 
     def _feed(self, stream, a, ctx):
         n = stream.x.shape[0]
         h, rs = self._normed(self.ff_norm, self.feed_forward.takes_row_scale(n, ctx),
                              stream.x, a, self.residual_scale, ctx)
-        if rs is None:
-            return self.feed_forward.forward(h, ctx)
-        return self.feed_forward.forward(h, ctx, row_scale=rs)
+        kw = {"defer_last": True} if self._ff_defers else {}
+        if rs is not None:
+            kw["row_scale"] = rs
+        return self.feed_forward.forward(h, ctx, **kw)
 
     def forward(self, stream: ResidualStream, ctx: StepContext, cache: Optional[CacheView], writes_cache: bool = True):
         if ctx.perf is not None and ctx.perf.enabled:

@@ -10,7 +10,7 @@ from typing import List
 import torch
 
 from .. import ops
-from .base import FEED_FORWARDS, FeedForward, Part, StepContext
+from .base import FEED_FORWARDS, DeferredBranch, FeedForward, Part, StepContext
 from .linear import Linear
 
 
@@ -29,6 +29,10 @@ class GatedFFN(FeedForward):
     def takes_row_scale(self, n: int, ctx: StepContext) -> bool:
         return self.gate_up.gated_takes_row_scale(n)
 
-    def forward(self, h: torch.Tensor, ctx: StepContext, row_scale=None) -> torch.Tensor:
+    can_defer_last = True
+
+    def forward(self, h: torch.Tensor, ctx: StepContext, row_scale=None, defer_last: bool = False):
         act = self.gate_up.forward_gated(h, ctx, "ffn.gate_up", row_scale=row_scale)
+        if defer_last and self.down.defers(act):
+            return DeferredBranch(self.down, act, ctx, "ffn.down")
         return self.down.forward(act, ctx, "ffn.down", out_dtype=torch.float32, partials=True)

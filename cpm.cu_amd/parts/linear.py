@@ -55,6 +55,12 @@ class Linear(Part):
         ops.linear(x, w, out, alpha, w_tiled=wt)
         return out
 
+    def defers(self, x: torch.Tensor) -> bool:
+        """Whether, for these rows, a norm could run this product itself (ops.proj_add_norm): only then is it
+        worth handing the product over instead of running it."""
+        return (self.tiled is not None and x.dtype == torch.bfloat16 and x.shape[0] <= ops.PROJ_NORM_MAX_ROWS
+                and self.in_features % 8 == 0 and self.out_features % 4 == 0)
+
     def takes_attention_shares(self) -> bool:
         """Whether forward_shares exists for this layer (bf16 engine with the decode product's weight layout)."""
         return self.tiled is not None

@@ -11,7 +11,7 @@ from typing import List, Mapping, Optional
 import torch
 
 from .. import ops
-from .base import NORMS, Norm, Runtime, StepContext, WeightSpec
+from .base import NORMS, DeferredBranch, Norm, Runtime, StepContext, WeightSpec, branch_tensor
 
 
 @NORMS.register("rms_norm")
@@ -28,7 +28,10 @@ class RMSNorm(Norm):
         self.weight = tensors[self.name].to(torch.float32).contiguous()
         self.rt = rt
 
+    takes_deferred_branch = True
+
     def forward(self, x, branch, branch_scale, ctx: StepContext, rows=None, tag="norm"):
+        branch = branch_tensor(branch)
         n_out = x.shape[0] if rows is None else rows.shape[0]
         out = ctx.ws.get(tag, (n_out, self.hidden_size), self.rt.dtype)
         ops.add_rms_norm(x, branch, branch_scale, self.weight, self.eps, out, rows)
@@ -41,6 +44,16 @@ class RMSNorm(Norm):
         if self.rt.dtype != torch.bfloat16 or n > ops.NORM_COLUMNS_MAX_ROWS or self.hidden_size % 4:
             return None
         out = ctx.ws.get(tag, (n, self.hidden_size), torch.bfloat16)
+        if isinstance(branch, DeferredBranch):
+            # the branch's last product, the residual add and this norm's column work in one kernel: a workgroup
+            # of that product owns 16 columns over all of K and finishes them itself
+            lin = branch.linear
+            if (lin.tiled is not None and n <= ops.PROJ_NORM_MAX_ROWS and lin.in_features % 8 == 0
+                    and lin.out_features == self.hidden_size and branch.a.dtype == torch.bfloat16):
+                sums = ctx.ws.get(tag + ".sums16", (n, -(-self.hidden_size // 16)), torch.float32)
+                ops.proj_add_norm(branch.a, lin.tiled, branch_scale, x, self.weight, out, sums)
+                return out, ops.RowScale(sums, self.eps)
+            branch = branch.evaluate()
         sums = ctx.ws.get(tag + ".sums", (n, ops.norm_slices(self.hidden_size)), torch.float32)
         ops.add_norm_columns(x, branch, branch_scale, self.weight, out, sums)
         return out, ops.RowScale(sums, self.eps)

@@ -187,6 +187,57 @@ def test_norm_cut_by_columns_and_finished_by_the_product(H, n, bdtype, parts):
         assert float((act.double() - ref).abs().max()) <= 2 ** -7 * max(1.0, float(ref.abs().max()))
 
 
+@pytest.mark.parametrize("n,N,K", [(1, 64, 128), (5, 100, 72), (16, 4096 + 16, 264), (17, 36, 1032), (32, 328, 520)])
+def test_product_that_adds_into_the_residual_and_does_the_norms_column_work(n, N, K):
+    """proj_add_norm: x += alpha * (a . W^T); x * w in bfloat16; sums of x^2 by strips of 16 columns; a product
+    that reads them finishes the norm.  Against float64, and against the pair of kernels it replaces."""
+    from cpmcu_amd import ops
+    eps, alpha = 2e-5, 0.6
+    a = rnd(n, K, seed=1, dtype=torch.bfloat16)
+    wm = rnd(N, K, seed=2, dtype=torch.bfloat16, scale=K ** -0.5)
+    x0, w = rnd(n, N, seed=3), rnd(N, seed=4) + 1.0
+    x = x0.clone()
+    xw = torch.full((n, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    sums = torch.full((n, -(-N // 16)), float("nan"), device=DEV)
+    ops.proj_add_norm(a, ops.TiledWeight(wm), alpha, x, w, xw, sums)
+    xs = x0.double() + alpha * (a.double() @ wm.double().T)
+    assert float((x.double() - xs).abs().max()) <= 1e-5 * max(1.0, float(xs.abs().max()))
+    ref = xs * w.double()
+    assert float((xw.double() - ref).abs().max()) <= 2 ** -8 * float(ref.abs().max())
+    ss = (xs * xs).sum(1)
+    assert float((sums.double().sum(1) - ss).abs().max()) <= 1e-5 * float(ss.max())
+    assert float((sums[:, 1].double() - (xs[:, 16:32] ** 2).sum(1)).abs().max()) <= 1e-5 * float(ss.max())
+    # the same through the split product and add_norm_columns
+    if n <= 16:
+        x2 = x0.clone()
+        y = torch.empty(n, N, device=DEV)
+        ops.gemm_skinny(a, wm, y)
+        xw2 = torch.empty_like(xw)
+        sums2 = torch.empty(n, ops.norm_slices(N), device=DEV)
+        ops.add_norm_columns(x2, y, alpha, w, xw2, sums2)
+        assert float((x - x2).abs().max()) <= 1e-5 * max(1.0, float(xs.abs().max()))
+    # a product that reads x * w and the strips' sums finishes the norm
+    if N % 8 == 0:
+        N2 = 48
+        w2 = rnd(N2, N, seed=5, dtype=torch.bfloat16, scale=N ** -0.5)
+        out = torch.empty(n, N2, device=DEV)
+        ops.gemm_skinny(xw, ops.TiledWeight(w2), out, 1.0, row_scale=ops.RowScale(sums, eps))
+        yr = (xw.double() @ w2.double().T) * torch.rsqrt(ss / N + eps)[:, None]
+        assert float((out.double() - yr).abs().max()) <= 1e-4 * float(yr.abs().max())
+
+
+def test_product_with_norm_refuses_what_it_does_not_take():
+    from cpmcu_amd import ops
+    a = rnd(33, 64, dtype=torch.bfloat16)
+    tw = ops.TiledWeight(rnd(32, 64, dtype=torch.bfloat16))
+    x, w = rnd(33, 32), rnd(32)
+    with pytest.raises(ops.KernelError):          # too many rows
+        ops.proj_add_norm(a, tw, 1.0, x, w, torch.empty(33, 32, dtype=torch.bfloat16, device=DEV), torch.empty(33, 2, device=DEV))
+    with pytest.raises(ops.KernelError):          # a weight that is not tiled for these columns
+        ops.proj_add_norm(a[:4, :32].contiguous(), tw, 1.0, x[:4].contiguous(), w,
+                          torch.empty(4, 32, dtype=torch.bfloat16, device=DEV), torch.empty(4, 2, device=DEV))
+
+
 @pytest.mark.parametrize("I", [77, 160, 1000])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_silu_mul(dtype, I):
