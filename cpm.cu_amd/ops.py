@@ -524,6 +524,31 @@ def proj_add_norm(a: torch.Tensor, w: "TiledWeight", alpha: float, x: torch.Tens
                                              c_float(alpha), _p(x), _p(weight), _p(out), _p(sums), _stream()))
 
 
+PROJ_NORM_SHARE_ROWS = 2        # tokens, shares and columns proj_add_norm_shares takes
+PROJ_NORM_SHARE_SPLITS = 8
+PROJ_NORM_SHARE_K = 8192
+
+
+def proj_add_norm_shares(part_o: torch.Tensor, part_ml: torch.Tensor, w: "TiledWeight", alpha: float,
+                         x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, sums: torch.Tensor):
+    """proj_add_norm whose a is the merged output of a split-KV attention, given as its shares (part_o float32
+    [m, heads, shares, hd], part_ml float32 [m, heads, shares, 2]; see gemm_skinny_shares): one or two tokens,
+    at most 8 shares, heads * hd at most 8,192."""
+    _need(part_o, "attention shares", torch.float32, (None, None, None, None))
+    n, nh, S, hd = part_o.shape
+    _need(part_ml, "attention share stats", torch.float32, (n, nh, S, 2))
+    if not isinstance(w, TiledWeight) or w.K != nh * hd:
+        raise KernelError(f"proj_add_norm_shares: the weight must be tiled for K = {nh * hd}")
+    N = w.N
+    _need(x, "proj residual", torch.float32, (n, N))
+    _need(weight, "proj norm weight", torch.float32, (N,))
+    _need(out, "proj out", torch.bfloat16, (n, N))
+    _need(sums, "proj row sums", torch.float32, (n, -(-N // 16)))
+    _check(_fn("qkv", "cpmcu_proj_add_norm_shares")(_p(part_o), _p(part_ml), c_int(S), c_int(nh), c_int(hd), _p(w.data),
+                                                    c_int(n), c_int(N), c_float(alpha), _p(x), _p(weight), _p(out),
+                                                    _p(sums), _stream()))
+
+
 def gemm_skinny(x: torch.Tensor, w, out: torch.Tensor, alpha: float = 1.0, mode: str = "plain",
                 row_scale: Optional[RowScale] = None):
     """bf16 product for at most 64 rows of x on the matrix cores, streaming w once; w is [N, K] as in the

@@ -109,10 +109,10 @@ class GQAAttention(Mixer):
                                cache.streams["v"], cache.page_table, cache.page_size, ctx, sel_blocks, sel_count, bs,
                                window_blocks, leave_shares=self.o.takes_attention_shares())
         if shares is not None:
+            if defer_last and self.o.defers_shares(shares[0]):
+                return DeferredBranch(self.o, None, ctx, "attn.o", shares=shares)
             return self.o.forward_shares(shares[0], shares[1], ctx, "attn.o")
         if defer_last and self.o.defers(out):
-            # steps of more tokens (measured for one token: the product that merges the shares and a norm
-            # kernel, 296 tokens/s, against a merge kernel and the product that does the norm's work, 290)
             return DeferredBranch(self.o, out, ctx, "attn.o")
         return self.o.forward(out, ctx, "attn.o", out_dtype=torch.float32, partials=True)
 

@@ -61,6 +61,12 @@ class Linear(Part):
         return (self.tiled is not None and x.dtype == torch.bfloat16 and x.shape[0] <= ops.PROJ_NORM_MAX_ROWS
                 and self.in_features % 8 == 0 and self.out_features % 4 == 0)
 
+    def defers_shares(self, part_o: torch.Tensor) -> bool:
+        """The same for an input given as attention shares [n, heads, shares, hd] (ops.proj_add_norm_shares)."""
+        n, _, S, _ = part_o.shape
+        return (self.tiled is not None and n <= ops.PROJ_NORM_SHARE_ROWS and S <= ops.PROJ_NORM_SHARE_SPLITS
+                and self.in_features <= ops.PROJ_NORM_SHARE_K and self.out_features % 4 == 0)
+
     def takes_attention_shares(self) -> bool:
         """Whether forward_shares exists for this layer (bf16 engine with the decode product's weight layout)."""
         return self.tiled is not None

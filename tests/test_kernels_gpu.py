@@ -399,6 +399,20 @@ def test_output_projection_merges_attention_shares(nh, nkv, hd, n):
         got_p = torch.full((2, n, N), float("nan"), device=DEV)
         ops.gemm_skinny_shares(po, pm, w, got_p, 1.0, mode="partial")
         assert torch.equal(got_p, want_p)
+    # the product that also adds into the residual and does the norm's column work takes the shares too
+    xr, wn = rnd(n, N, seed=5), rnd(N, seed=6) + 1.0
+    outs = []
+    for shares in (False, True):
+        x = xr.clone()
+        xw = torch.full((n, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+        sums = torch.full((n, -(-N // 16)), float("nan"), device=DEV)
+        if shares:
+            ops.proj_add_norm_shares(po, pm, w, 0.5, x, wn, xw, sums)
+        else:
+            ops.proj_add_norm(merged, w, 0.5, x, wn, xw, sums)
+        outs.append((x, xw, sums))
+    assert all(torch.equal(u, v) for u, v in zip(*outs))
+    assert float((outs[0][0] - (xr + want)).abs().max()) <= 1e-5 * float(want.abs().max() + 1)
 
 
 @pytest.mark.parametrize("nh,nkv,hd", [(16, 1, 64), (8, 1, 32), (4, 2, 128), (5, 5, 16), (40, 2, 32), (6, 2, 48), (2, 1, 96)])
