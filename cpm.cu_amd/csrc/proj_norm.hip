@@ -1,5 +1,5 @@
 // A branch's last product fused with the residual add and the column part of the norm that follows it
-// (bf16, decode steps of at most 32 tokens):
+// (bf16, decode steps of at most 64 tokens):
 //     x += alpha * (a . W^T);   out = bf16(x * w_norm);   row_ss[row][strip] = sum of x^2 over the strip
 // A decode step is a chain of small kernels, each of which costs a few microseconds whatever it does.  The
 // split-K product leaves partial sums that a second kernel (elementwise.hip: add_norm_columns) adds into the
@@ -183,10 +183,10 @@ __global__ __launch_bounds__(NW * 64) void proj_add_norm_kernel(
 }
 
 // x [M, N] float32 (in place), a [M, K] bf16, W tiled [N, K], w_norm [N] float32, out [M, N] bf16,
-// row_ss [M, ceil(N / 16)] float32.  N must be a multiple of 4, K of 8; at most 32 rows.
+// row_ss [M, ceil(N / 16)] float32.  N must be a multiple of 4, K of 8; at most 64 rows.
 extern "C" const char* cpmcu_proj_add_norm(const void* A, long lda, const void* W, int M, int N, int K, float alpha,
                                            float* x, const float* w_norm, void* out, float* row_ss, hipStream_t stream) {
-    CPMCU_REQUIRE(M > 0 && M <= 32, "proj_add_norm: %d tokens (1..32 are taken; more go through the split product and the norm kernel)", M);
+    CPMCU_REQUIRE(M > 0 && M <= 64, "proj_add_norm: %d tokens (1..64 are taken; more go through the split product and the norm kernel)", M);
     CPMCU_REQUIRE(N > 0 && N % 4 == 0 && K > 0 && K % 8 == 0 && lda % 8 == 0 && lda >= K,
                   "proj_add_norm: N=%d must be a multiple of 4, K=%d and the row stride %ld multiples of 8", N, K, lda);
     CPMCU_REQUIRE(A && W && x && w_norm && out && row_ss, "proj_add_norm: null pointer");
@@ -198,8 +198,10 @@ extern "C" const char* cpmcu_proj_add_norm(const void* A, long lda, const void* 
                                                                         K, alpha, x, w_norm, (bf16_t*)out, row_ss, strips, \
                                                                         AShares{})
     // 4 blocks in flight in each of 4 wavefronts measured best (8 wavefronts: the same; 8 blocks: slower)
+    // (more tokens hold more of a in registers for every block in flight: fewer blocks then)
     if (M <= 16) LAUNCH(4, 4, 1);
-    else LAUNCH(4, 4, 2);
+    else if (M <= 32) LAUNCH(4, 4, 2);
+    else LAUNCH(2, 4, 4);
 #undef LAUNCH
     CPMCU_LAUNCH_CHECK("proj_add_norm");
     return nullptr;

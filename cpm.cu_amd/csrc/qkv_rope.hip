@@ -1,4 +1,4 @@
-// q, k, v projection of a decode step fused with the rotation and the cache write (bf16, at most 32 tokens).
+// q, k, v projection of a decode step fused with the rotation and the cache write (bf16, at most 64 tokens).
 //
 // A decode step is a chain of small kernels, each of which costs a few microseconds whatever it does; this one
 // replaces the split-K product + the kernel that summed its partial sums, rotated and stored.
@@ -205,7 +205,7 @@ extern "C" const char* cpmcu_qkv_rope(const void* X, long ldx, const void* W, in
                                       const float* inv_freq, float mscale, void* kpool, void* vpool,
                                       const int* page_table, int table_width, int page_size, const float* row_ss,
                                       int ss_slices, float eps, void* ckpool, int ck_size, int ck_stride, hipStream_t stream) {
-    CPMCU_REQUIRE(M > 0 && M <= 32, "qkv_rope: %d tokens (1..32 are taken; more go through the split product and the rotary kernel)", M);
+    CPMCU_REQUIRE(M > 0 && M <= 64, "qkv_rope: %d tokens (1..64 are taken; more go through the split product and the rotary kernel)", M);
     CPMCU_REQUIRE(nh > 0 && nkv > 0 && hd > 0 && hd % 16 == 0, "qkv_rope: bad shape heads=%d kv_heads=%d head_dim=%d", nh, nkv, hd);
     CPMCU_REQUIRE(K > 0 && K % 8 == 0 && ldx % 8 == 0 && ldx >= K, "qkv_rope: K=%d, row stride %ld must be multiples of 8", K, ldx);
     CPMCU_REQUIRE(((uintptr_t)X % 16 == 0) && ((uintptr_t)W % 16 == 0), "qkv_rope: operands must be 16-byte aligned");
@@ -216,13 +216,15 @@ extern "C" const char* cpmcu_qkv_rope(const void* X, long ldx, const void* W, in
                   page_size, ck_size);
     PagedView pv{page_table, table_width, page_size};
     const int strips = (nh + 2 * nkv) * (hd / 16);
-#define LAUNCH(MTv)                                                                                              \
-    qkv_rope_kernel<4, 4, MTv><<<strips, 256, 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, M, K, (bf16_t*)q_out, \
+#define LAUNCH(PFv, MTv)                                                                                         \
+    qkv_rope_kernel<PFv, 4, MTv><<<strips, 256, 0, stream>>>((const bf16_t*)X, ldx, (const bf16_t*)W, M, K, (bf16_t*)q_out, \
                                                            nh, nkv, hd, positions, tok_slot, inv_freq, mscale,       \
                                                            (bf16_t*)kpool, (bf16_t*)vpool, pv, row_ss, ss_slices, eps, \
                                                            (bf16_t*)ckpool, ck_size, ck_stride)
-    if (M <= 16) LAUNCH(1);
-    else LAUNCH(2);
+    // more tokens hold more of x in registers for every block in flight: fewer blocks then
+    if (M <= 16) LAUNCH(4, 1);
+    else if (M <= 32) LAUNCH(4, 2);
+    else LAUNCH(2, 4);
 #undef LAUNCH
     CPMCU_LAUNCH_CHECK("qkv_rope");
     return nullptr;

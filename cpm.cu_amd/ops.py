@@ -111,9 +111,24 @@ def add_rms_norm(x: torch.Tensor, branch: Optional[torch.Tensor], branch_scale: 
 
 
 NORM_SLICE = 64        # columns a slice of add_norm_columns (common.h)
-# rows up to which the norm cut by columns wins (MI355X, 4,096 columns, after a product's partial sums: 4.7
-# against 6.6 us at 8 rows; at 64 rows 4.8 against 5.0 us, and the gated product that finishes it 58.4 against 57 us)
-NORM_COLUMNS_MAX_ROWS = 16
+
+# The kernels of decode steps that own a strip of output columns over all of K (qkv_rope, proj_add_norm) and
+# the norm cut by columns (add_norm_columns) save kernels of the chain, but every workgroup reads all of x.
+# Up to 16 rows they win at every width measured (MI355X, 4,096 columns: norm 4.7 against 6.6 us at 8 rows,
+# q/k/v + rotary 12.3 against 16.8 us at 8 rows and 15.1 against 18.0 at 16).  With more rows qkv_rope loses
+# (4,096 columns: 24.4 against 21.3 us at 32 rows; 1,024 columns: 16.8 + 4.7 against 8.9 + 5.1 + 4.2 us at 64),
+# and proj_add_norm wins only while a workgroup's copy of x stays small (1,024 columns, 64 rows: 8.6 against
+# 8.9 + 4.2 us).
+STRIP_ROWS = 16
+STRIP_MAX_ROWS = 64
+STRIP_X_BYTES = 160 * 1024
+QKV_ROPE_MAX_ROWS = STRIP_ROWS
+
+
+def strip_kernels_ok(n: int, K: int) -> bool:
+    """Whether proj_add_norm (and the norm cut by columns) take a step of n rows of K columns."""
+    return n <= STRIP_ROWS or (n <= STRIP_MAX_ROWS and n * K * 2 <= STRIP_X_BYTES)
+
 
 
 class RowScale:
@@ -442,9 +457,6 @@ class TiledWeight:
         self.N, self.K = N, K
 
 
-# qkv_rope takes up to 32 tokens; it wins up to 16 (MI355X, 8B shape: 12.3 against 16.8 us for the split product
-# and the rotary kernel at 8 tokens, 15.1 against 18.0 at 16, 24.4 against 21.3 at 32)
-QKV_ROPE_MAX_ROWS = 16
 
 
 def qkv_rope_weight(w: torch.Tensor, nh: int, nkv: int, hd: int) -> TiledWeight:
@@ -465,7 +477,7 @@ def qkv_rope(x: torch.Tensor, w: TiledWeight, q_out: torch.Tensor, nh: int, nkv:
              positions: torch.Tensor, tok_slot: torch.Tensor, inv_freq: Optional[torch.Tensor], mscale: float,
              kpool: torch.Tensor, vpool: torch.Tensor, page_table: torch.Tensor, page_size: int,
              row_scale: Optional[RowScale] = None, compress: Optional[Tuple[torch.Tensor, int, int]] = None):
-    """q, k, v = x . w^T for a step of at most 32 tokens, rotated (inv_freq None: not) and written: q to q_out
+    """q, k, v = x . w^T for a step of at most 64 tokens, rotated (inv_freq None: not) and written: q to q_out
     [n, nh*hd], k and v into the paged cache.  w from qkv_rope_weight.  With row_scale, x is the x * w of
     add_norm_columns and the rows of the product are multiplied by the norm's factor before the rotation.
     With compress = (compressed key pool, kernel_size, kernel_stride) the compressed keys that the step's tokens
@@ -500,13 +512,10 @@ def qkv_rope(x: torch.Tensor, w: TiledWeight, q_out: torch.Tensor, nh: int, nkv:
                                         _p(ckpool), c_int(ks), c_int(st), _stream()))
 
 
-PROJ_NORM_MAX_ROWS = 16
-
-
 def proj_add_norm(a: torch.Tensor, w: "TiledWeight", alpha: float, x: torch.Tensor, weight: torch.Tensor,
                   out: torch.Tensor, sums: torch.Tensor):
     """A branch's last product fused with the residual add and the column part of the norm that follows, for a
-    step of at most 32 tokens: x += alpha * (a . w^T) in place (x float32 [n, N], a bfloat16 [n, K], w tiled
+    step of at most 64 tokens: x += alpha * (a . w^T) in place (x float32 [n, N], a bfloat16 [n, K], w tiled
     [N, K]); out = bfloat16(x * weight); sums[r, s] = sum of x[r]^2 over the 16 columns of strip s (float32
     [n, ceil(N / 16)]).  As after add_norm_columns, the product that reads `out` applies the row factor."""
     _need(a, "proj a", torch.bfloat16, (None, None))

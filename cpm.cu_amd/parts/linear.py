@@ -58,7 +58,7 @@ class Linear(Part):
     def defers(self, x: torch.Tensor) -> bool:
         """Whether, for these rows, a norm could run this product itself (ops.proj_add_norm): only then is it
         worth handing the product over instead of running it."""
-        return (self.tiled is not None and x.dtype == torch.bfloat16 and x.shape[0] <= ops.PROJ_NORM_MAX_ROWS
+        return (self.tiled is not None and x.dtype == torch.bfloat16 and ops.strip_kernels_ok(x.shape[0], self.in_features)
                 and self.in_features % 8 == 0 and self.out_features % 4 == 0)
 
     def defers_shares(self, part_o: torch.Tensor) -> bool:

@@ -41,7 +41,7 @@ class RMSNorm(Norm):
         # decode steps: a row a workgroup leaves most of the chip idle, so the work is cut by columns and the
         # row factor rsqrt(mean(x^2) + eps) is left to the product that follows
         n = x.shape[0]
-        if self.rt.dtype != torch.bfloat16 or n > ops.NORM_COLUMNS_MAX_ROWS or self.hidden_size % 4:
+        if self.rt.dtype != torch.bfloat16 or not ops.strip_kernels_ok(n, self.hidden_size) or self.hidden_size % 4:
             return None
         out = ctx.ws.get(tag, (n, self.hidden_size), torch.bfloat16)
         if isinstance(branch, DeferredBranch):

@@ -187,7 +187,8 @@ def test_norm_cut_by_columns_and_finished_by_the_product(H, n, bdtype, parts):
         assert float((act.double() - ref).abs().max()) <= 2 ** -7 * max(1.0, float(ref.abs().max()))
 
 
-@pytest.mark.parametrize("n,N,K", [(1, 64, 128), (5, 100, 72), (16, 4096 + 16, 264), (17, 36, 1032), (32, 328, 520)])
+@pytest.mark.parametrize("n,N,K", [(1, 64, 128), (5, 100, 72), (16, 4096 + 16, 264), (17, 36, 1032), (32, 328, 520),
+                                   (33, 68, 136), (64, 1024 + 4, 1160)])
 def test_product_that_adds_into_the_residual_and_does_the_norms_column_work(n, N, K):
     """proj_add_norm: x += alpha * (a . W^T); x * w in bfloat16; sums of x^2 by strips of 16 columns; a product
     that reads them finishes the norm.  Against float64, and against the pair of kernels it replaces."""
@@ -228,11 +229,11 @@ def test_product_that_adds_into_the_residual_and_does_the_norms_column_work(n, N
 
 def test_product_with_norm_refuses_what_it_does_not_take():
     from cpmcu_amd import ops
-    a = rnd(33, 64, dtype=torch.bfloat16)
+    a = rnd(65, 64, dtype=torch.bfloat16)
     tw = ops.TiledWeight(rnd(32, 64, dtype=torch.bfloat16))
-    x, w = rnd(33, 32), rnd(32)
+    x, w = rnd(65, 32), rnd(32)
     with pytest.raises(ops.KernelError):          # too many rows
-        ops.proj_add_norm(a, tw, 1.0, x, w, torch.empty(33, 32, dtype=torch.bfloat16, device=DEV), torch.empty(33, 2, device=DEV))
+        ops.proj_add_norm(a, tw, 1.0, x, w, torch.empty(65, 32, dtype=torch.bfloat16, device=DEV), torch.empty(65, 2, device=DEV))
     with pytest.raises(ops.KernelError):          # a weight that is not tiled for these columns
         ops.proj_add_norm(a[:4, :32].contiguous(), tw, 1.0, x[:4].contiguous(), w,
                           torch.empty(4, 32, dtype=torch.bfloat16, device=DEV), torch.empty(4, 2, device=DEV))
@@ -583,7 +584,8 @@ def read_cache_rows(pool, table, page, nkv, hd, slot, positions, tiles):
 
 @pytest.mark.parametrize("n,nh,nkv,hd,H,rotate", [(1, 4, 2, 16, 64, True), (8, 32, 2, 128, 512, True), (16, 3, 1, 32, 96, True),
                                                   (5, 6, 3, 64, 200, False), (13, 2, 2, 48, 264, True),
-                                                  (17, 4, 2, 32, 136, True), (24, 2, 1, 64, 1160, True), (32, 6, 2, 16, 72, True)])
+                                                  (17, 4, 2, 32, 136, True), (24, 2, 1, 64, 1160, True), (32, 6, 2, 16, 72, True),
+                                                  (33, 2, 1, 32, 392, True), (64, 5, 1, 16, 1032, True)])
 @pytest.mark.parametrize("scaled", [False, True])
 def test_fused_projection_rotation_and_cache_write(n, nh, nkv, hd, H, rotate, scaled):
     """q, k, v of a decode step in one kernel: against the float64 product, rotation (pairs c, c + hd/2) and the
@@ -628,7 +630,7 @@ def test_fused_projection_rotation_and_cache_write(n, nh, nkv, hd, H, rotate, sc
     assert int((kpool != 0).sum()) <= n * nkv * hd and int((vpool != 0).sum()) <= n * nkv * hd
 
 
-@pytest.mark.parametrize("n,ks,st", [(16, 8, 4), (5, 32, 16), (32, 12, 4), (1, 32, 16)])
+@pytest.mark.parametrize("n,ks,st", [(16, 8, 4), (5, 32, 16), (32, 12, 4), (1, 32, 16), (50, 8, 4)])
 def test_fused_projection_completes_compressed_keys(n, ks, st):
     """The projection kernel of decode steps also writes the compressed keys that its tokens complete: bit for
     bit what compress_keys writes after it, from keys of earlier steps and of this step (two sequences, each
