@@ -29,7 +29,7 @@ MODULES: Dict[str, List[str]] = {
     "gemm": ["gemm.hip"],
     "attention": ["attention.hip"],
     "sparse": ["sparse.hip"],
-    "qkv": ["qkv_rope.hip", "proj_norm.hip"],
+    "qkv": ["qkv_rope.hip", "strip.hip"],
 }
 HEADERS = ["common.h"]
 

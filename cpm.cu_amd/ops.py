@@ -533,6 +533,22 @@ def proj_add_norm(a: torch.Tensor, w: "TiledWeight", alpha: float, x: torch.Tens
                                              c_float(alpha), _p(x), _p(weight), _p(out), _p(sums), _stream()))
 
 
+def gated_strip(x: torch.Tensor, w: "TiledWeight", out: torch.Tensor, row_scale: Optional[RowScale] = None):
+    """out = silu(x . Wg^T) * (x . Wu^T) for a step of at most 16 tokens, w tiled with the gate rows first (a
+    multiple of 16 of them); out bfloat16 [n, N/2].  With row_scale as in gemm_skinny."""
+    _need(x, "gated x", torch.bfloat16, (None, None))
+    n, K = x.shape
+    if not isinstance(w, TiledWeight) or w.K != K or w.N % 32:
+        raise KernelError(f"gated_strip: the weight must be tiled for K = {K} with a multiple of 16 gate rows")
+    _need(out, "gated out", torch.bfloat16, (n, w.N // 2))
+    if row_scale is not None:
+        _need(row_scale.sums, "gated row sums", torch.float32, (n, None))
+    _check(_fn("qkv", "cpmcu_gated_strip")(_p(x), c_long(K), _p(w.data), c_int(n), c_int(w.N // 2), c_int(K), _p(out),
+                                           _p(row_scale.sums if row_scale is not None else None),
+                                           c_int(row_scale.sums.shape[1] if row_scale is not None else 0),
+                                           c_float(row_scale.eps if row_scale is not None else 0.0), _stream()))
+
+
 PROJ_NORM_SHARE_ROWS = 2        # tokens, shares and columns proj_add_norm_shares takes
 PROJ_NORM_SHARE_SPLITS = 8
 PROJ_NORM_SHARE_K = 8192

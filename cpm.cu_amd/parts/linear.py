@@ -97,7 +97,10 @@ class Linear(Part):
         """For a weight of gate rows stacked on up rows: silu(x Wg^T) * (x Wu^T), [n, out/2]."""
         n, half = x.shape[0], self.out_features // 2
         act = ctx.ws.get(tag + ".act", (n, half), x.dtype)
-        if self._gated_skinny(n, x.dtype):
+        if (n <= ops.STRIP_ROWS and x.dtype == torch.bfloat16 and self.tiled is not None and half % 16 == 0
+                and self.in_features % 8 == 0):
+            ops.gated_strip(x, self.tiled, act, row_scale=row_scale)      # a strip of columns a workgroup
+        elif self._gated_skinny(n, x.dtype):
             ops.gemm_skinny(x, self.tiled if self.tiled is not None else self.weight, act, mode="gated",
                             row_scale=row_scale)
         else:

@@ -227,6 +227,39 @@ def test_product_that_adds_into_the_residual_and_does_the_norms_column_work(n, N
         assert float((out.double() - yr).abs().max()) <= 1e-4 * float(yr.abs().max())
 
 
+@pytest.mark.parametrize("n,I,K", [(1, 16, 72), (7, 48, 264), (16, 1008, 1032), (8, 4096, 128)])
+@pytest.mark.parametrize("scaled", [False, True])
+def test_gated_product_by_strips(n, I, K, scaled):
+    """gated_strip: silu(x Wg^T) * (x Wu^T) with a workgroup a strip of gate rows and their up rows, with and
+    without the row factor of a norm cut by columns; against float64 and against the skinny product."""
+    from cpmcu_amd import ops
+    x = rnd(n, K, seed=1, dtype=torch.bfloat16)
+    w = rnd(2 * I, K, seed=2, dtype=torch.bfloat16, scale=2.0 * K ** -0.5)
+    tw = ops.TiledWeight(w)
+    rs, r = None, 1.0
+    if scaled:
+        sums = torch.rand(n, 5, generator=torch.Generator().manual_seed(n)) + 0.1
+        rs = ops.RowScale(sums.to(DEV), 1e-3)
+        r = torch.rsqrt(sums.double().sum(1) / K + 1e-3).view(n, 1).to(DEV)
+    out = torch.full((n, I), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.gated_strip(x, tw, out, row_scale=rs)
+    y = (x.double() @ w.double().T) * r
+    ref = F.silu(y[:, :I]) * y[:, I:]
+    assert float((out.double() - ref).abs().max()) <= 2 ** -7 * max(1.0, float(ref.abs().max()))
+    other = torch.empty_like(out)
+    ops.gemm_skinny(x, tw, other, mode="gated", row_scale=rs)
+    assert float((out.double() - other.double()).abs().max()) <= 2 ** -6 * max(1.0, float(ref.abs().max()))
+    with pytest.raises(ops.KernelError):          # 17 rows
+        ops.gated_strip(rnd(17, K, dtype=torch.bfloat16), tw, torch.empty(17, I, dtype=torch.bfloat16, device=DEV))
+
+
+def test_gated_product_by_strips_refuses_gate_rows_that_are_no_multiple_of_16():
+    from cpmcu_amd import ops
+    tw = ops.TiledWeight(rnd(2 * 24, 64, dtype=torch.bfloat16))
+    with pytest.raises(ops.KernelError):
+        ops.gated_strip(rnd(2, 64, dtype=torch.bfloat16), tw, torch.empty(2, 24, dtype=torch.bfloat16, device=DEV))
+
+
 def test_product_with_norm_refuses_what_it_does_not_take():
     from cpmcu_amd import ops
     a = rnd(65, 64, dtype=torch.bfloat16)
