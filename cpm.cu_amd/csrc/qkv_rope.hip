@@ -59,6 +59,24 @@ __global__ __launch_bounds__(NW * 64) void qkv_rope_kernel(
     qfloatx4_t acc[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[t] = qfloatx4_t{0.f, 0.f, 0.f, 0.f};
+    // what the end needs (positions, the tokens' cache rows through two dependent lookups, the pairs'
+    // frequencies) is asked for first: it is there when the products are, instead of costing three trips to
+    // memory after them
+    const int spt = hd / 16;                       // strips a head
+    const int head = strip / spt, s = strip - head * spt;
+    int tok_pos[MT];
+    long tok_row[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        const int tok = min(t * 16 + r, M - 1);
+        tok_pos[t] = positions[tok];
+        tok_row[t] = head >= nh ? paged_row(pv, tok_slot[tok], tok_pos[t]) : 0;
+    }
+    float freq[4] = {0.f, 0.f, 0.f, 0.f};
+    if (inv_freq && head < nh + nkv) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) freq[i] = inv_freq[8 * s + 4 * (g & 1) + i];
+    }
     auto multiply = [&](qbf16x8_t (&wd)[4], qbf16x8_t (&xd)[MT][4]) {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
@@ -106,16 +124,12 @@ __global__ __launch_bounds__(NW * 64) void qkv_rope_kernel(
         }
     }
 
-    const int spt = hd / 16;                       // strips a head
-    const int head = strip / spt, s = strip - head * spt;
     float own[MT][4];                              // a key head's values as the cache holds them
-    int tok_pos[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
         const int tok = t * 16 + r;
         const bool tok_ok = tok < M;
-        const int pos = positions[min(tok, M - 1)];
-        tok_pos[t] = pos;
+        const int pos = tok_pos[t];
         if (head < nh + nkv) {
             // rows 0..7 of the strip are d = 8s .. 8s+7, rows 8..15 their partners d + hd/2: lanes g and g+2 hold
             // a pair; after the swap every lane has both (the first half of the wavefront's value, then the second's)
@@ -132,14 +146,14 @@ __global__ __launch_bounds__(NW * 64) void qkv_rope_kernel(
             bf16_t* dst = nullptr;
             if (tok_ok) {
                 if (is_q) dst = q_out + ((long)tok * nh + head) * hd;
-                else dst = kpool + key_index(paged_row(pv, tok_slot[tok], pos), head - nh, nkv, hd);
+                else dst = kpool + key_index(tok_row[t], head - nh, nkv, hd);
             }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int c = 8 * s + 4 * (g & 1) + i;             // index of the pair
                 float cs = 1.f, sn = 0.f;
                 if (inv_freq) {
-                    const float ang = (float)pos * inv_freq[c];
+                    const float ang = (float)pos * freq[i];
                     cs = cosf(ang) * mscale;
                     sn = sinf(ang) * mscale;
                 }
@@ -150,7 +164,7 @@ __global__ __launch_bounds__(NW * 64) void qkv_rope_kernel(
                 if (tok_ok) dst[is_q ? d : key_d_offset(d)] = vb;
             }
         } else if (tok_ok) {
-            bf16_t* dst = vpool + value_index(paged_row(pv, tok_slot[tok], pos), head - nh - nkv, nkv, hd);
+            bf16_t* dst = vpool + value_index(tok_row[t], head - nh - nkv, nkv, hd);
 #pragma unroll
             for (int i = 0; i < 4; ++i) dst[value_d_offset(16 * s + 4 * g + i)] = f32_to_bf16(acc[t][i]);
         }

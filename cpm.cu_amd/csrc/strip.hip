@@ -76,6 +76,14 @@ __global__ __launch_bounds__(NW * 64) void proj_add_norm_kernel(
     pfloatx4_t acc[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[t] = pfloatx4_t{0.f, 0.f, 0.f, 0.f};
+    // what the end needs (the residual's 4 columns of this lane's tokens, the norm's weights) is asked for
+    // first: it is there when the products are, instead of costing a trip to memory after them
+    const int col = strip * 16 + 4 * g;
+    const bool col_ok = col < N;                                  // N is a multiple of 4
+    const float4 wn = *(const float4*)(w_norm + min(col, N - 4));
+    float4 xin[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) xin[t] = *(const float4*)(x + (long)min(t * 16 + r, M - 1) * N + min(col, N - 4));
     const bf16_t* as_row = as + min(r, M - 1) * K + g * 8;        // SHARES: this lane's row of a in LDS
     auto multiply = [&](int kb, pbf16x8_t (&wd)[4], pbf16x8_t (&ad)[SHARES ? 1 : MT][SHARES ? 1 : 4]) {
 #pragma unroll
@@ -157,9 +165,6 @@ __global__ __launch_bounds__(NW * 64) void proj_add_norm_kernel(
     }
     __syncthreads();
     if (wave > 0) return;
-    const int col = strip * 16 + 4 * g;
-    const bool col_ok = col < N;                                  // N is a multiple of 4
-    const float4 wn = *(const float4*)(w_norm + min(col, N - 4));
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
 #pragma unroll
@@ -169,7 +174,7 @@ __global__ __launch_bounds__(NW * 64) void proj_add_norm_kernel(
         const int tok = t * 16 + r;
         const bool ok = tok < M && col_ok;
         const long off = (long)min(tok, M - 1) * N + min(col, N - 4);
-        float4 v = *(const float4*)(x + off);
+        float4 v = xin[t];
         v.x += alpha * acc[t][0]; v.y += alpha * acc[t][1]; v.z += alpha * acc[t][2]; v.w += alpha * acc[t][3];
         float ss = 0.f;
         if (ok) {
