@@ -292,7 +292,7 @@ __global__ void select_scores_kernel(const bf16_t* __restrict__ q, const bf16_t*
                                      SelectParams sp, SelectScratch sc);
 __global__ void select_normalise_kernel(const int* __restrict__ positions, SelectParams sp, SelectScratch sc);
 __global__ void select_blocks_kernel(const int* __restrict__ positions, SelectParams sp, SelectScratch sc,
-                                     int* __restrict__ sel_blocks, int* __restrict__ sel_count);
+                                     int* __restrict__ sel_blocks, int* __restrict__ sel_count, int stats_off);
 template <int HD, int NW>
 __global__ void sparse_select_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ ckpool, PagedView pv,
                                           const int* __restrict__ positions, const int* __restrict__ tok_slot,
@@ -325,7 +325,9 @@ extern "C" const char* cpmcu_sparse_select(const void* q, const void* ckpool, in
                   max_pos + 1, lds);
     dim3 grid(n, nkv);
     PagedView pv{page_table, table_width, page_size};
-    if (dtype == CPMCU_BF16 && !force_plain && hd >= 16 && hd <= 128 && hd % 16 == 0) {
+    // force_plain: 1 = the plain kernel whatever the type; 2 = matrix cores, but steps of few tokens with the
+    // kernel that normalises the scores kept apart (as for contexts whose statistics do not fit into LDS)
+    if (dtype == CPMCU_BF16 && force_plain != 1 && hd >= 16 && hd <= 128 && hd % 16 == 0) {
         const size_t lds2 = sizeof(float) * ((size_t)sp.max_ck + 4 + select_work_floats(sp.max_blocks));
         CPMCU_REQUIRE(lds2 <= 60 * 1024,
                       "sparse_select: a context of %d tokens needs %zu bytes of LDS for its block scores (limit 61440)",
@@ -362,9 +364,18 @@ extern "C" const char* cpmcu_sparse_select(const void* q, const void* ckpool, in
             CPMCU_LAUNCH_CHECK("select_scores");
             const size_t lds3 = sizeof(float) * ((size_t)sc.n_groups * G * 2 + 2 * G);
             CPMCU_REQUIRE(lds3 <= 60 * 1024, "sparse_select: %d groups of compressed keys x %d heads exceed LDS", sc.n_groups, G);
+            const size_t lds2e = (lds2 + 7) / 8 * 8;
+            if (lds2e + lds3 <= 60 * 1024 && force_plain != 2) {
+                // the last kernel normalises the scores itself (the same sums in the same order): one kernel
+                // of the chain less
+                select_blocks_kernel<<<grid, 1024, lds2e + lds3, stream>>>(positions, sp, sc, sel_blocks, sel_count,
+                                                                         (int)(lds2e / sizeof(float)));
+                CPMCU_LAUNCH_CHECK("select_blocks");
+                return nullptr;
+            }
             select_normalise_kernel<<<dim3(n, nkv, (sp.max_ck + 255) / 256), 256, lds3, stream>>>(positions, sp, sc);
             CPMCU_LAUNCH_CHECK("select_normalise");
-            select_blocks_kernel<<<grid, 1024, lds2, stream>>>(positions, sp, sc, sel_blocks, sel_count);
+            select_blocks_kernel<<<grid, 1024, lds2, stream>>>(positions, sp, sc, sel_blocks, sel_count, 0);
             CPMCU_LAUNCH_CHECK("select_blocks");
             return nullptr;
         }
@@ -697,9 +708,11 @@ __global__ __launch_bounds__(256) void select_normalise_kernel(const int* __rest
     }
 }
 
+// stats_off (in floats, or 0): where in LDS the groups' (max, sum) pairs go when this kernel does the work of
+// select_normalise_kernel itself; 0: the scores come ready in sc.score
 __global__ __launch_bounds__(1024) void select_blocks_kernel(const int* __restrict__ positions, SelectParams sp,
                                                              SelectScratch sc, int* __restrict__ sel_blocks,
-                                                             int* __restrict__ sel_count) {
+                                                             int* __restrict__ sel_count, int stats_off) {
     constexpr int NW = 16;
     extern __shared__ float lds[];
     __shared__ int wave_tot[NW];
@@ -715,7 +728,37 @@ __global__ __launch_bounds__(1024) void select_blocks_kernel(const int* __restri
     const int n_vis = p < sp.ks ? 0 : (p - sp.ks) / sp.st + 1;
     const int q_block = p / sp.bs;
     const int n_cand = max(q_block - sp.window_blocks + 1, 0);
-    for (int j = tid; j < n_vis; j += NW * 64) score[j] = sc.score[out_idx * sp.max_ck + j];
+    if (stats_off) {
+        const int G = sp.nh / sp.nkv;
+        const int groups = (n_vis + 63) / 64;
+        float2* gst = (float2*)(lds + stats_off);
+        float* ms = (float*)(gst + (long)sc.n_groups * G);
+        float* inv = ms + G;
+        const float2* st = (const float2*)(sc.stats + out_idx * sc.n_groups * G * 2);
+        for (int i = tid; i < groups * G; i += NW * 64) gst[i] = st[i];
+        __syncthreads();
+        if (tid < G) {
+            float mm = -INFINITY;
+            for (int gi = 0; gi < groups; ++gi) mm = fmaxf(mm, gst[gi * G + tid].x);
+            float ll = 0.f;
+            for (int gi = 0; gi < groups; ++gi) {
+                const float2 v = gst[gi * G + tid];
+                ll += v.y * exp2f(v.x - mm);
+            }
+            ms[tid] = mm;
+            inv[tid] = ll > 0.f ? 1.0f / ll : 0.f;
+        }
+        __syncthreads();
+        for (int j = tid; j < n_vis; j += NW * 64) {
+            const float* s = sc.sraw + out_idx * G * sp.max_ck + j;
+            float a = 0.f;
+#pragma unroll 16
+            for (int h = 0; h < G; ++h) a += exp2f(s[(long)h * sp.max_ck] - ms[h]) * inv[h];
+            score[j] = a;
+        }
+    } else {
+        for (int j = tid; j < n_vis; j += NW * 64) score[j] = sc.score[out_idx * sp.max_ck + j];
+    }
     __syncthreads();
     blocks_from_scores<NW>(score, work, wave_tot, sp, n_vis, q_block, n_cand, out_idx, sel_blocks, sel_count);
 }

@@ -395,9 +395,11 @@ def sparse_select(q: torch.Tensor, ckpool: torch.Tensor, nh: int, nkv: int, hd: 
                   page_table: torch.Tensor, page_size: int, positions: torch.Tensor, tok_slot: torch.Tensor,
                   kernel_size: int, kernel_stride: int, block_size: int, init_blocks: int, topk: int,
                   window_blocks: int, dense_len: int, max_pos: int, sel_blocks: torch.Tensor, sel_count: torch.Tensor,
-                  force_plain: bool = False, scratch: Optional[torch.Tensor] = None):
+                  force_plain=False, scratch: Optional[torch.Tensor] = None):
     """Block list per (token, kv head): sel_count -1 = dense, else the ascending blocks to attend to.
-    scratch: float32 of at least sparse_select_scratch(...) elements (bf16 steps of few tokens use it)."""
+    scratch: float32 of at least sparse_select_scratch(...) elements (bf16 steps of few tokens use it).
+    force_plain: True = the plain kernel; 2 = steps of few tokens with the normalising kernel kept apart, as for
+    contexts too long for the fused form (for tests)."""
     _need(q, "select q", shape=(None, nh * hd))
     n = q.shape[0]
     _need(ckpool, "select compressed keys", q.dtype, (None, page_size // max(kernel_stride, 1), nkv * hd))
@@ -413,7 +415,7 @@ def sparse_select(q: torch.Tensor, ckpool: torch.Tensor, nh: int, nkv: int, hd: 
         _p(page_table), c_int(page_table.shape[1]), c_int(page_size), _p(positions), _p(tok_slot),
         c_int(kernel_size), c_int(kernel_stride), c_int(block_size), c_int(init_blocks), c_int(topk),
         c_int(window_blocks), c_int(dense_len), c_int(max_pos), _p(sel_blocks), _p(sel_count),
-        c_int(sel_blocks.shape[2]), c_int(1 if force_plain else 0), _p(scratch),
+        c_int(sel_blocks.shape[2]), c_int(int(force_plain)), _p(scratch),
         c_long(scratch.numel() if scratch is not None else 0), _stream()))
 
 

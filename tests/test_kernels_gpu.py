@@ -749,9 +749,10 @@ def test_block_selection_equals_the_plain_selection(dtype, nh, nkv, hd, ks, st, 
     sel_count = torch.full((n, nkv), -7, dtype=torch.int32, device=DEV)
     # plain selection from the same (rounded) keys; compressed keys in the cache's own precision
     ck_ref = plain.compressed_keys(kseq[0], ks, st).to(dtype).double()
-    # the matrix-core kernel, its two-kernel form for steps of few tokens, and the plain twin
+    # the matrix-core kernel, its forms for steps of few tokens (two kernels, or three when the last does not
+    # normalise the scores itself), and the plain twin
     scratch = torch.full((ops.sparse_select_scratch(n, nh, nkv, max(positions), ks, st),), float("nan"), device=DEV)
-    for force_plain, scr in (((False, None), (False, scratch), (True, None)) if dtype == torch.bfloat16
+    for force_plain, scr in (((False, None), (False, scratch), (2, scratch), (True, None)) if dtype == torch.bfloat16
                              else ((True, None),)):
         sel_blocks.fill_(-7)
         sel_count.fill_(-7)
