@@ -85,6 +85,20 @@ __global__ __launch_bounds__(NW * 64) void qkv_rope_kernel(
     };
 #pragma unroll
     for (int j = 0; j < PF; ++j) load_block(kb0 + j, a[j], bx[j]);
+    // the pairs' cosines and sines are formed while the first blocks are on their way
+    float rot_cs[MT][4], rot_sn[MT][4];
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            rot_cs[t][i] = 1.f;
+            rot_sn[t][i] = 0.f;
+            if (inv_freq && head < nh + nkv) {
+                const float ang = (float)tok_pos[t] * freq[i];
+                rot_cs[t][i] = cosf(ang) * mscale;
+                rot_sn[t][i] = sinf(ang) * mscale;
+            }
+        }
     if (row_ss) row_scales<NW * 64, MT * 16>(row_ss, ss_slices, M, 1.0f / (float)K, eps, rs_s);
     int kb = kb0;
     for (; kb + 2 * PF <= kb1; kb += PF) {           // every block and every block asked for exists
@@ -151,12 +165,7 @@ __global__ __launch_bounds__(NW * 64) void qkv_rope_kernel(
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int c = 8 * s + 4 * (g & 1) + i;             // index of the pair
-                float cs = 1.f, sn = 0.f;
-                if (inv_freq) {
-                    const float ang = (float)pos * freq[i];
-                    cs = cosf(ang) * mscale;
-                    sn = sinf(ang) * mscale;
-                }
+                const float cs = rot_cs[t][i], sn = rot_sn[t][i];
                 const float v = second ? lo[i] * sn + hi[i] * cs : lo[i] * cs - hi[i] * sn;
                 const int d = second ? c + hd / 2 : c;
                 const bf16_t vb = f32_to_bf16(v);
