@@ -87,6 +87,19 @@ def test_unequal_batches_one_after_another(model_dirs, references, name, dtype):
 
 
 @pytest.mark.parametrize("name", ["A", "B"])
+def test_engine_without_the_second_copy_of_the_weights(model_dirs, references, name):
+    """tiled_weights=False: the bfloat16 engine keeps the checkpoint's layout only, so decode steps go through the
+    split products and the norm kernels instead of the kernels that own strips of the re-laid weights."""
+    cfg, w, reqs, refs = references[name]
+    eng = engine_for(model_dirs, name, "bfloat16", tiled_weights=False)
+    check(schedules.tail(eng, reqs, 32), refs, "bfloat16", "tail-32, checkpoint layout only")
+    got = schedules.batched(eng, reqs, WORK[name]["prompt"], BATCHES[:2])
+    check(got, refs, "bfloat16", "batched, checkpoint layout only")
+    eng.cache.check()
+    assert not eng.cache.live
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
 def test_cutting_changes_nothing_beyond_rounding(model_dirs, references, name):
     """32-bit: whole, token by token and batched agree far below the tolerance against the plain implementation."""
     cfg, w, reqs, refs = references[name]
