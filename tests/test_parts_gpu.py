@@ -242,6 +242,68 @@ def test_block_arrangement(dtype):
     assert float((got_pend.double().cpu() - pend).abs().max()) < tol_for(dtype, pend)
 
 
+def test_a_branch_left_to_the_next_norm_equals_the_branch_run_by_its_part():
+    """Decode steps in bfloat16: the attention and the feed-forward leave their last product to the norm that
+    follows (DeferredBranch), which runs it fused with the residual add.  Two blocks in a row, once with the
+    package's norm, once with a norm defined here that knows nothing of that hand-over and must be given
+    tensors: the same residual stream and the same pending branch, beyond rounding."""
+    from cpmcu_amd import ops
+    from cpmcu_amd.parts import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, ResidualStream
+    from cpmcu_amd.parts.base import DeferredBranch, Norm, WeightSpec
+
+    class PlainNorm(Norm):                      # no takes_deferred_branch, no forward_unscaled
+        def __init__(self, name, hidden_size, eps):
+            self.name, self.hidden_size, self.eps = name, hidden_size, eps
+
+        def weight_specs(self):
+            return [WeightSpec(self.name, (self.hidden_size,), "norm")]
+
+        def bind(self, tensors, rt):
+            self.weight, self.rt = tensors[self.name].float().contiguous(), rt
+
+        def forward(self, x, branch, branch_scale, ctx, rows=None, tag="norm"):
+            assert branch is None or isinstance(branch, torch.Tensor)
+            out = ctx.ws.get(tag, (x.shape[0], self.hidden_size), self.rt.dtype)
+            ops.add_rms_norm(x, branch, branch_scale, self.weight, self.eps, out, rows)
+            return out
+
+    H, nh, nkv, hd, I, n_seq = 64, 4, 2, 16, 96, 5
+    results = []
+    for norm_ctor in (lambda name: NORMS.build("rms_norm", name=name, hidden_size=H, eps=1e-5),
+                      lambda name: PlainNorm(name, H, 1e-5)):
+        blocks = [BLOCKS.build(
+            "pre_norm", mixer_norm=norm_ctor(f"{i}.n1"),
+            mixer=MIXERS.build("gqa_attention", prefix=f"{i}.a.", hidden_size=H, num_heads=nh, num_kv_heads=nkv,
+                               head_dim=hd, position=POSITION_ENCODINGS.build("rope", head_dim=hd, theta=100.0)),
+            ff_norm=norm_ctor(f"{i}.n2"),
+            feed_forward=FEED_FORWARDS.build("gated_silu", prefix=f"{i}.m.", hidden_size=H, intermediate_size=I),
+            residual_scale=0.7) for i in range(2)]
+        rt = runtime(torch.bfloat16)
+        for i, blk in enumerate(blocks):
+            shapes = {s.name: s.shape for s in blk.all_weight_specs()}
+            w = {k: (rnd(*v, seed=31 * i + j, scale=0.2) + (1.0 if len(v) == 1 else 0.0)).bfloat16().to(DEV)
+                 for j, (k, v) in enumerate(shapes.items())}
+            blk.bind_all(w, rt)
+        # one token each of five sequences that already hold some tokens: a decode step
+        ctx = make_ctx([b.mixer.cache_needs() for b in blocks], [[0]] * n_seq, torch.bfloat16, max_slots=8,
+                       start=[3, 70, 1, 64, 20])
+        for grp in ctx.cache.groups:
+            for st in grp.storage.values():
+                for t in st.values():
+                    t.copy_(rnd(*t.shape, seed=5, scale=0.5))
+        stream = ResidualStream(rnd(n_seq, H, seed=9).to(DEV))
+        kinds = []
+        for i, blk in enumerate(blocks):
+            blk.forward(stream, ctx, ctx.cache.view(i))
+            kinds.append(type(stream.take_pending()))
+        pend = stream.pending
+        results.append((stream.x.clone(), (pend.sum(0) if pend.dim() == 3 else pend).clone(), kinds))
+    (xa, pa, ka), (xb, pb, kb) = results
+    assert ka == [DeferredBranch, DeferredBranch] and kb == ka      # the parts hand over either way
+    assert float((xa - xb).abs().max()) <= 2 ** -7 * float(xb.abs().max())
+    assert float((pa - pb).abs().max()) <= 2 ** -6 * float(pb.abs().max())
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_block_sparse_attention_part_alone(dtype):
     """The InfLLM-v2 mixer against the plain layer, whole prompt and then token by token across block edges;
