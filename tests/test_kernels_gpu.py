@@ -615,6 +615,50 @@ def read_cache_rows(pool, table, page, nkv, hd, slot, positions, tiles):
     return torch.stack(out)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,nh,nkv,hd,parts,rotate,write_kv", [
+    (1, 4, 2, 16, 0, True, True), (7, 5, 1, 48, 3, True, True), (70, 6, 2, 32, 0, True, True),
+    (130, 32, 2, 128, 0, True, True), (67, 3, 3, 64, 0, False, True), (9, 2, 1, 80, 2, True, False),
+    (100, 4, 1, 112, 0, True, False)])
+def test_rotary_and_cache_write(dtype, n, nh, nkv, hd, parts, rotate, write_kv):
+    """rope_store alone (the kernel of few tokens, which also sums a split product's partial sums, and the kernel
+    of prompt chunks in bfloat16): q rotated into q_out, k rotated and v as they are into the pages, read back
+    through the pages' layout; pairs (c, c + hd/2), angle = position * inv_freq[c], cos and sin times the
+    magnitude; tokens of several slots at scattered positions."""
+    from cpmcu_amd import ops
+    page = 64
+    width = (nh + 2 * nkv) * hd
+    g = torch.Generator().manual_seed(n * 7 + hd)
+    src = torch.randn((parts, n, width) if parts else (n, width), generator=g)
+    src = src.to(dtype if not parts else torch.float32)              # partial sums are float32
+    slots = torch.randint(0, 3, (n,), generator=g)
+    positions = torch.randperm(190, generator=g)[:n]                 # distinct, so no two tokens share a cache row
+    table = torch.randperm(12, generator=g)[:9].view(3, 3).to(torch.int32)
+    inv_freq = (torch.rand(hd // 2, generator=g) * 0.5 + 0.01) if rotate else None
+    mscale = 1.25 if rotate else 1.0
+    kpool = torch.zeros(12, page, nkv * hd, dtype=dtype, device=DEV)
+    vpool = torch.zeros_like(kpool)
+    q_out = torch.full((n, nh * hd), float("nan"), dtype=dtype, device=DEV)
+    ops.rope_store(src.to(DEV), q_out, nh, nkv, hd, positions.to(torch.int32).to(DEV), slots.to(torch.int32).to(DEV),
+                   inv_freq.to(DEV) if rotate else None, mscale, kpool if write_kv else None,
+                   vpool if write_kv else None, table.to(DEV) if write_kv else None, page, write_kv)
+    y = (src.double().sum(0) if parts else src.double()).view(n, nh + 2 * nkv, hd).clone()
+    if rotate:
+        ang = positions.double()[:, None] * inv_freq.float().double()[None, :]
+        cs, sn = (torch.cos(ang) * mscale)[:, None, :], (torch.sin(ang) * mscale)[:, None, :]
+        a, b = y[:, :nh + nkv, :hd // 2].clone(), y[:, :nh + nkv, hd // 2:].clone()
+        y[:, :nh + nkv] = torch.cat([a * cs - b * sn, a * sn + b * cs], dim=-1)
+    tol = (1e-5 if dtype == torch.float32 else 2 ** -7) * max(1.0, float(y.abs().max()))
+    assert float((q_out.double().cpu().view(n, nh, hd) - y[:, :nh]).abs().max()) <= tol
+    if write_kv:
+        for t in range(n):
+            k_row = read_cache_rows(kpool, table, page, nkv, hd, int(slots[t]), [int(positions[t])], key_tiles)[0]
+            v_row = read_cache_rows(vpool, table, page, nkv, hd, int(slots[t]), [int(positions[t])], value_tiles)[0]
+            assert float((k_row.double() - y[t, nh:nh + nkv]).abs().max()) <= tol, t
+            assert float((v_row.double() - y[t, nh + nkv:]).abs().max()) <= tol, t
+        assert int((kpool != 0).sum()) <= n * nkv * hd and int((vpool != 0).sum()) <= n * nkv * hd
+
+
 @pytest.mark.parametrize("n,nh,nkv,hd,H,rotate", [(1, 4, 2, 16, 64, True), (8, 32, 2, 128, 512, True), (16, 3, 1, 32, 96, True),
                                                   (5, 6, 3, 64, 200, False), (13, 2, 2, 48, 264, True),
                                                   (17, 4, 2, 32, 136, True), (24, 2, 1, 64, 1160, True), (32, 6, 2, 16, 72, True),
