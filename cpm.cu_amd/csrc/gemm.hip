@@ -113,18 +113,28 @@ struct XShares {
     int n_splits, nh, hd;
 };
 
-template <int MT, int MODE, typename OT, int SPW, int NW, bool TILED, bool SHARES = false>
-__global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ X, long ldx,
+// KW (1 or 2): groups of NW wavefronts a workgroup.  With 2, both groups own the same strips and share the
+// staged X; of every chunk of 4 K-blocks the first group multiplies blocks 0, 1 and the second blocks 2, 3, and
+// the second hands its sums to the first through LDS at the end.  With 48 and more rows a wavefront is busy
+// issuing (4 tiles of rows an operand load) rather than waiting, and one wavefront a SIMD cannot hide that:
+// twice the wavefronts on the same X traffic.
+template <int MT, int MODE, typename OT, int SPW, int NW, bool TILED, bool SHARES = false, int KW = 1>
+__global__ __launch_bounds__(NW * KW * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ X, long ldx,
                                                              const bf16_t* __restrict__ W, long ldw,
                                                              OT* __restrict__ Y, long ldy, int M, int N, int K, int KS,
                                                              float alpha, int I, long part_stride,
                                                              const float* __restrict__ row_ss, int ss_slices,
                                                              float eps, XShares xsh) {
     static_assert(MODE != 2 || SPW == 2, "gated output pairs a gate strip with an up strip");
-    constexpr int NT = NW * 64;
+    static_assert(KW == 1 || (KW == 2 && !SHARES), "one or two groups of wavefronts");
+    constexpr int NT = NW * KW * 64;
     constexpr int XV = MT * 16 * 64 / NT;     // 16-byte vectors of X a thread stages per chunk
+    constexpr int BPW = 4 / KW;               // K-blocks of a chunk a wavefront multiplies
     __shared__ __attribute__((aligned(16))) bf16_t xs[MT * 16 * SK_XS];
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave_wg = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int kw = KW > 1 ? wave_wg / NW : 0;              // which blocks of a chunk
+    const int wave = KW > 1 ? wave_wg - kw * NW : wave_wg; // which strips
     const int r = lane & 15, g = lane >> 4;
     const int k_begin = blockIdx.y * KS;
     const int k_end = min(K, k_begin + KS);
@@ -157,7 +167,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
         }
     }
 
-    bf16x8_t a[4][SPW][4];
+    bf16x8_t a[KW][BPW][SPW][4];              // [chunk parity][block of the wavefront]
     auto load_w = [&](int kb, bf16x8_t (&dst)[SPW][4]) {
         const int k = k_begin + kb * 128 + g * 8;
 #pragma unroll
@@ -237,33 +247,65 @@ if (TILED) {
         for (int t = 0; t < MT; ++t) acc[s][t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
 #pragma unroll
-    for (int j = 0; j < 4; ++j) load_w(j, a[j]);
+    for (int p = 0; p < KW; ++p)
+#pragma unroll
+        for (int jj = 0; jj < BPW; ++jj) load_w(p * 4 + kw * BPW + jj, a[p][jj]);
     load_x(0);
     // X may be x * w of a norm whose row factor is still to come (common.h: row_scales); the loop's first
     // barrier makes rs_s visible
     __shared__ float rs_s[MT * 16];
     if (row_ss) row_scales<NT, MT * 16>(row_ss, ss_slices, M, 1.0f / (float)K, eps, rs_s);
     const int nchunk = (nkb + 3) / 4;
-    for (int c = 0; c < nchunk; ++c) {
-        __syncthreads();
-        store_x();
-        __syncthreads();
-        if (c + 1 < nchunk) load_x(c + 1);
+    // a wavefront's weight blocks are asked for KW chunks (4 blocks of its own) ahead; the chunk's parity picks
+    // the registers, so the loop advances KW chunks a turn
+    for (int c0 = 0; c0 < nchunk; c0 += KW) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            // consecutive matrix instructions go to different accumulators (tiles of rows, then strips)
+        for (int p = 0; p < KW; ++p) {
+            const int c = c0 + p;
+            if (c >= nchunk) break;
+            __syncthreads();
+            store_x();
+            __syncthreads();
+            if (c + 1 < nchunk) load_x(c + 1);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
+            for (int jj = 0; jj < BPW; ++jj) {
+                const int j = kw * BPW + jj;
+                // consecutive matrix instructions go to different accumulators (tiles of rows, then strips)
 #pragma unroll
-                for (int t = 0; t < MT; ++t) {
-                    const bf16x8_t b = *(const bf16x8_t*)(xs + (t * 16 + r) * SK_XS + j * 128 + g * 8 + i * 32);
+                for (int i = 0; i < 4; ++i) {
 #pragma unroll
-                    for (int s = 0; s < SPW; ++s)
-                        acc[s][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j][s][i], b, acc[s][t], 0, 0, 0);
+                    for (int t = 0; t < MT; ++t) {
+                        const bf16x8_t b = *(const bf16x8_t*)(xs + (t * 16 + r) * SK_XS + j * 128 + g * 8 + i * 32);
+#pragma unroll
+                        for (int s = 0; s < SPW; ++s)
+                            acc[s][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[p][jj][s][i], b, acc[s][t], 0, 0, 0);
+                    }
                 }
+                load_w((c + KW) * 4 + j, a[p][jj]);
             }
-            load_w(c * 4 + j + 4, a[j]);
         }
+    }
+    if (KW > 1) {
+        // the second group's sums go to the first through LDS (the staged X is no longer needed)
+        float* red = (float*)xs;
+        static_assert(KW == 1 || NW * SPW * MT * 4 * 64 * sizeof(float) <= sizeof(xs), "sums of a group fit into the X buffer");
+        __syncthreads();
+        if (kw == 1) {
+#pragma unroll
+            for (int s = 0; s < SPW; ++s)
+#pragma unroll
+                for (int t = 0; t < MT; ++t)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) red[(((wave * SPW + s) * MT + t) * 4 + i) * 64 + lane] = acc[s][t][i];
+        }
+        __syncthreads();
+        if (kw == 1) return;
+#pragma unroll
+        for (int s = 0; s < SPW; ++s)
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[s][t][i] += red[(((wave * SPW + s) * MT + t) * 4 + i) * 64 + lane];
     }
 
     // lane (r, g) of tile t holds token t*16 + r, rows 4g .. 4g+3 of each strip
@@ -295,7 +337,7 @@ if (TILED) {
 }
 
 // out_mode: 0 = Y[m,N] in out_dtype; 1 = float partial sums Y[ksplit][m][N]; 2 = gated (N = 2*I rows of W, Y[m,I] bf16)
-// variant (gated output only): 0 = 4 waves a workgroup, 1 = 2 waves
+// variant: gated output 0 = 4 waves a workgroup, 1 = 2 waves; 4 = two groups of 4 waves (33..64 rows, any mode)
 // row_ss (or null): X is x * w of a norm cut by columns, whose sums of squares [M][ss_slices] these are (a
 // slice for every 64 columns after add_norm_columns, for every 16 after proj_add_norm); the output is multiplied
 // by rsqrt(sum of the row's slices / K + eps) row by row
@@ -319,16 +361,16 @@ extern "C" const char* cpmcu_gemm_skinny_v(const void* X, long ldx, const void* 
     const int MT = (M + 15) / 16 == 3 ? 4 : (M + 15) / 16;
     const int I = N / 2;
     const long part_stride = (long)M * ldy;
-#define LAUNCH(MTv, MODEv, OT, SPW, NW)                                                                           \
+#define LAUNCH(MTv, MODEv, OT, SPW, NW, KWv)                                                                      \
     do {                                                                                                          \
         const int rows_wg = (MODEv == 2) ? NW * 16 : NW * SPW * 16;                                               \
         dim3 grid(((MODEv == 2 ? I : N) + rows_wg - 1) / rows_wg, ksplit);                                        \
         if (tiled)                                                                                                \
-            gemm_skinny_kernel<MTv, MODEv, OT, SPW, NW, true><<<grid, NW * 64, 0, stream>>>(                      \
+            gemm_skinny_kernel<MTv, MODEv, OT, SPW, NW, true, false, KWv><<<grid, NW * KWv * 64, 0, stream>>>(    \
                 (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (OT*)Y, ldy, M, N, K, KS, alpha, I, part_stride,    \
                 row_ss, ss_slices, eps, XShares{});                                                               \
         else                                                                                                      \
-            gemm_skinny_kernel<MTv, MODEv, OT, SPW, NW, false><<<grid, NW * 64, 0, stream>>>(                     \
+            gemm_skinny_kernel<MTv, MODEv, OT, SPW, NW, false, false, KWv><<<grid, NW * KWv * 64, 0, stream>>>(   \
                 (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (OT*)Y, ldy, M, N, K, KS, alpha, I, part_stride,    \
                 row_ss, ss_slices, eps, XShares{});                                                               \
     } while (0)
@@ -337,9 +379,11 @@ extern "C" const char* cpmcu_gemm_skinny_v(const void* X, long ldx, const void* 
 #define BY_VAR(MTv, MODEv, OT)                                  \
     do {                                                        \
         if (MODEv == 2) {                                       \
-            if (variant == 1) LAUNCH(MTv, MODEv, OT, 2, 2);     \
-            else LAUNCH(MTv, MODEv, OT, 2, 4);                  \
-        } else LAUNCH(MTv, (MODEv == 2 ? 0 : MODEv), OT, 1, 4); \
+            if (variant == 1) LAUNCH(MTv, MODEv, OT, 2, 2, 1);  \
+            else if (variant == 4 && MTv == 4) LAUNCH(4, MODEv, OT, 2, 4, 2); \
+            else LAUNCH(MTv, MODEv, OT, 2, 4, 1);               \
+        } else if (variant == 4 && MTv == 4) LAUNCH(4, (MODEv == 2 ? 0 : MODEv), OT, 1, 4, 2); \
+        else LAUNCH(MTv, (MODEv == 2 ? 0 : MODEv), OT, 1, 4, 1); \
     } while (0)
 #define BY_MT(MODEv, OT)                         \
     do {                                         \
@@ -360,11 +404,13 @@ extern "C" const char* cpmcu_gemm_skinny_v(const void* X, long ldx, const void* 
 }
 
 // The variant that measured best on the MI355X for each shape: one strip a wave (more, smaller
-// workgroups balance better over 256 CUs); gated output with 2 waves a workgroup up to 16 rows.
+// workgroups balance better over 256 CUs); gated output with 2 waves a workgroup up to 16 rows, and with two
+// groups of 4 waves that share the staged X from 33 rows on (64 rows, 32,768 x 4,096: 54.4 against 59.9 us; the
+// split products gain nothing from it: down 33.1 against 34.0 us, o 15.0 against 13.8).
 extern "C" const char* cpmcu_gemm_skinny(const void* X, long ldx, const void* W, long ldw, void* Y, long ldy,
                                          int out_dtype, int out_mode, int M, int N, int K, int ksplit, float alpha,
                                          int tiled, const float* row_ss, int ss_slices, float eps, hipStream_t stream) {
-    const int variant = out_mode == 2 ? (M <= 16 ? 1 : 0) : 2;
+    const int variant = out_mode == 2 ? (M <= 16 ? 1 : (M > 32 ? 4 : 0)) : 2;
     return cpmcu_gemm_skinny_v(X, ldx, W, ldw, Y, ldy, out_dtype, out_mode, M, N, K, ksplit, alpha, variant, tiled,
                                row_ss, ss_slices, eps, stream);
 }
