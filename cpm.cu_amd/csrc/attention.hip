@@ -12,6 +12,9 @@
 // s_j = (q.k_j) * scale for keys j <= position of the query, softmax over j in
 // float, out = sum_j p_j v_j; query head h reads kv head h / (nh/nkv).
 #include "common.h"
+#include "no_alloc.h"
+
+#include <mutex>
 
 template <typename T>
 __global__ __launch_bounds__(64) void attention_paged_kernel(
@@ -445,13 +448,15 @@ __global__ void attention_combine_kernel(const float* __restrict__ part_o, const
     }
 }
 
-extern "C" const char* cpmcu_attention_mfma(const void* q, void* out, float* part_o, float* part_ml, int n, int nh,
-                                            int nkv, int hd, float scale, const void* kpool, const void* vtpool,
-                                            const int* page_table, int table_width, int page_size,
-                                            const int* positions, const int* tok_slot, const int* sel_blocks,
-                                            const int* sel_count, int max_sel, int block_size, int n_splits,
-                                            int waves_per_group, int last_blocks_first, int merge,
-                                            hipStream_t stream) {
+// Checks and launches of the matrix-core attention; part_o / part_ml are the scratch of its shares, wherever
+// the caller keeps them.
+static const char* attention_mfma_launch(const void* q, void* out, float* part_o, float* part_ml, int n, int nh,
+                                         int nkv, int hd, float scale, const void* kpool, const void* vtpool,
+                                         const int* page_table, int table_width, int page_size,
+                                         const int* positions, const int* tok_slot, const int* sel_blocks,
+                                         const int* sel_count, int max_sel, int block_size, int n_splits,
+                                         int waves_per_group, int last_blocks_first, int merge,
+                                         hipStream_t stream) {
     CPMCU_REQUIRE(n > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_mfma: bad shape n=%d heads=%d kv_heads=%d", n, nh, nkv);
     CPMCU_REQUIRE(hd >= 16 && hd <= 128 && hd % 16 == 0,
                   "attention_mfma: head_dim %d has no matrix-core kernel (16, 32, ... 128 have; the plain kernel takes the rest)", hd);
@@ -504,6 +509,84 @@ extern "C" const char* cpmcu_attention_mfma(const void* q, void* out, float* par
         CPMCU_LAUNCH_CHECK("attention_combine");
     }
     return nullptr;
+}
+
+extern "C" const char* cpmcu_attention_mfma(const void* q, void* out, float* part_o, float* part_ml, int n, int nh,
+                                            int nkv, int hd, float scale, const void* kpool, const void* vtpool,
+                                            const int* page_table, int table_width, int page_size,
+                                            const int* positions, const int* tok_slot, const int* sel_blocks,
+                                            const int* sel_count, int max_sel, int block_size, int n_splits,
+                                            int waves_per_group, int last_blocks_first, int merge,
+                                            hipStream_t stream) {
+    return attention_mfma_launch(q, out, part_o, part_ml, n, nh, nkv, hd, scale, kpool, vtpool, page_table,
+                                 table_width, page_size, positions, tok_slot, sel_blocks, sel_count, max_sel,
+                                 block_size, n_splits, waves_per_group, last_blocks_first, merge, stream);
+}
+
+// ---------------------------------------------------------------------------
+// The same attention for callers that cannot allocate (declared in no_alloc.h): the shares of a split-KV
+// run lie in an array of the library's own instead of a workspace the caller brings.
+//
+// `static_scratch` is the array; in host code that name is only a stand-in for the symbol, not a device
+// address, so the address is asked for once per device (each GPU holds its own copy at its own address) and
+// only that pointer is handed to kernels.  Every share's output and (max, sum) pair is written by the
+// attention kernel before the merge kernel reads it (a share without keys writes sum 0), so nothing has to
+// be cleared between calls.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) float static_scratch[CPMCU_STATIC_SCRATCH_FLOATS];
+
+namespace {
+constexpr int kMaxDevices = 64;
+float* g_scratch_ptr[kMaxDevices];          // per device, set at the first call on that device
+std::mutex g_scratch_mutex;
+
+const char* static_scratch_address(float** ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) CPMCU_FAIL("attention_mfma_static: hipGetDevice failed: %s", hipGetErrorString(e));
+    CPMCU_REQUIRE(dev >= 0 && dev < kMaxDevices, "attention_mfma_static: device %d (0..%d are taken)", dev,
+                  kMaxDevices - 1);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(static_scratch));
+        if (e != hipSuccess || !p)
+            CPMCU_FAIL("attention_mfma_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+        g_scratch_ptr[dev] = (float*)p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return nullptr;
+}
+}  // namespace
+
+extern "C" const char* cpmcu_attention_mfma_static(const void* q, void* out, int n, int nh, int nkv, int hd,
+                                                   float scale, const void* kpool, const void* vtpool,
+                                                   const int* page_table, int table_width, int page_size,
+                                                   const int* positions, const int* tok_slot, const int* sel_blocks,
+                                                   const int* sel_count, int max_sel, int block_size, int n_splits,
+                                                   int waves_per_group, int last_blocks_first, hipStream_t stream) {
+    CPMCU_REQUIRE(n > 0 && nh > 0 && hd > 0 && n_splits >= 1, "attention_mfma_static: bad shape n=%d heads=%d head_dim=%d shares=%d",
+                  n, nh, hd, n_splits);
+    float* part_o = nullptr;
+    float* part_ml = nullptr;
+    if (n_splits > 1) {
+        // shares' outputs [n][heads][shares][hd], then their (max, sum) pairs [n][heads][shares][2]
+        const long rows = (long)n * nh * n_splits;
+        const long need = rows * hd + rows * 2;
+        CPMCU_REQUIRE(need <= (long)CPMCU_STATIC_SCRATCH_FLOATS,
+                      "attention_mfma_static: %d tokens x %d heads x %d shares x (head_dim %d + 2) = %ld floats of "
+                      "shares exceed the library's own scratch of %ld floats (%ld MiB); use fewer shares or tokens, "
+                      "or cpmcu_attention_mfma with a workspace",
+                      n, nh, n_splits, hd, need, (long)CPMCU_STATIC_SCRATCH_FLOATS,
+                      (long)CPMCU_STATIC_SCRATCH_FLOATS * 4 / (1 << 20));
+        float* base = nullptr;
+        if (const char* err = static_scratch_address(&base)) return err;
+        part_o = base;
+        part_ml = base + rows * hd;
+    }
+    return attention_mfma_launch(q, out, part_o, part_ml, n, nh, nkv, hd, scale, kpool, vtpool, page_table,
+                                 table_width, page_size, positions, tok_slot, sel_blocks, sel_count, max_sel,
+                                 block_size, n_splits, waves_per_group, last_blocks_first, 1, stream);
 }
 
 // ===========================================================================

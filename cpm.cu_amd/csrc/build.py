@@ -31,7 +31,7 @@ MODULES: Dict[str, List[str]] = {
     "sparse": ["sparse.hip"],
     "qkv": ["qkv_rope.hip", "strip.hip"],
 }
-HEADERS = ["common.h"]
+HEADERS = ["common.h", "no_alloc.h"]
 
 # -packed-fp32-ops off: the compiler must not form packed float instructions on its own
 HIPCC_FLAGS = [
