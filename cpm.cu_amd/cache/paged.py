@@ -20,7 +20,7 @@ device sees the page tables and the pools.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Dict, List, Optional, Tuple
+from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
 
@@ -108,7 +108,10 @@ class SequenceCache:
         self.device = torch.device(device)
         self.dtype = dtype
         self.n_pages = -(-max_tokens // page_size)
-        self.table_width = min(-(-max_seq_len // page_size), self.n_pages)
+        seq_pages = -(-max_seq_len // page_size)
+        # a page table has an entry for every page number a sequence can reach: a group that keeps every token
+        # cannot hold more pages than its pool has, a group that keeps a window can (it gives old pages back)
+        self.table_width = min(seq_pages, self.n_pages)
         self.groups: List[_Group] = []
         self.entry_group: List[int] = []
         by_key: Dict[object, List[int]] = {}
@@ -116,8 +119,8 @@ class SequenceCache:
             by_key.setdefault(n.group_key(), []).append(e)
         self.entry_group = [0] * len(needs)
         for key, entries in by_key.items():
-            g = _Group(needs[entries[0]], entries, self.n_pages, max_slots, self.table_width, page_size,
-                       self.device, dtype)
+            width = seq_pages if needs[entries[0]].window is not None else self.table_width
+            g = _Group(needs[entries[0]], entries, self.n_pages, max_slots, width, page_size, self.device, dtype)
             for e in entries:
                 self.entry_group[e] = len(self.groups)
             self.groups.append(g)
@@ -156,10 +159,60 @@ class SequenceCache:
             raise CacheError(f"slot {slot} is not held by a live sequence") from None
 
     # ---- tokens ----
-    def pages_needed(self, slot: int, new_len: int) -> int:
-        """Pages a full-history group must still take for the slot to hold new_len tokens."""
-        have = -(-self.length(slot) // self.page_size)
-        return max(-(-new_len // self.page_size) - have, 0)
+    def _first_kept(self, g: _Group, old: int) -> int:
+        """The first page number a group still needs when the next query sits at position ``old``."""
+        if g.needs.window is None:
+            return 0
+        return max(old - g.needs.window + 1, 0) // self.page_size
+
+    def _group_need(self, g: _Group, slot: int, old: int, new: int) -> Tuple[int, int]:
+        """(pages the group must take, pages it gives back first) to grow the slot from old to new tokens."""
+        pages = g.pages[slot]
+        n_pg = -(-new // self.page_size)
+        if g.needs.window is None:
+            return max(n_pg - len(pages), 0), 0
+        first_kept = self._first_kept(g, old)
+        need = max(n_pg - max(len(pages), first_kept), 0)
+        need += sum(1 for pn in range(first_kept, min(len(pages), n_pg)) if pages[pn] < 0)
+        freed = 0
+        for pn in range(min(first_kept, len(pages)) - 1, -1, -1):
+            if pages[pn] < 0:
+                break
+            freed += 1
+        return need, freed
+
+    def room_for(self, extensions: Sequence[Tuple[int, int]]) -> Optional[str]:
+        """None if every group can take ``n_new`` more tokens for each (slot, n_new) at once, else the reason.
+        Each group is asked for what it really needs: a group that keeps a window counts the pages it gives
+        back.  A step that is cut into several passes never needs more than this."""
+        for gi, g in enumerate(self.groups):
+            need = freed = 0
+            for slot, n_new in extensions:
+                old = self.length(slot)
+                a, b = self._group_need(g, slot, old, old + n_new)
+                need += a
+                freed += b
+            if need > len(g.free_pages) + freed:
+                return (f"the cache is full: this step needs {need} more pages of {self.page_size} tokens"
+                        f"{'' if len(self.groups) == 1 else f' in cache group {gi}'}, "
+                        f"{len(g.free_pages) + freed} are free of {g.n_pages}")
+        return None
+
+    def pages_to_hold(self, length: int, step: int) -> List[int]:
+        """Per group, the most pages a sequence of ``length`` tokens holds at any time when it grows by at most
+        ``step`` tokens at once (what a planner reserves for it)."""
+        out = []
+        for g in self.groups:
+            full = -(-length // self.page_size)
+            if g.needs.window is None:
+                out.append(full)
+            else:
+                out.append(min(full, (step + g.needs.window - 2) // self.page_size + 2))
+        return out
+
+    def capacity(self) -> List[int]:
+        """Pages of each group's pool."""
+        return [g.n_pages for g in self.groups]
 
     def free_page_count(self) -> int:
         return min(len(g.free_pages) for g in self.groups) if self.groups else self.n_pages
@@ -176,35 +229,48 @@ class SequenceCache:
         n_pg = -(-new // self.page_size)
         # check every group before touching any, so a refused step changes nothing
         for g in self.groups:
-            first_kept = 0 if g.needs.window is None else max(old - g.needs.window + 1, 0) // self.page_size
-            need = sum(1 for pn in range(first_kept, n_pg) if pn >= len(g.pages[slot]) or g.pages[slot][pn] < 0)
-            freed = 0 if g.needs.window is None else sum(1 for p in g.pages[slot][:first_kept] if p >= 0)
+            need, freed = self._group_need(g, slot, old, new)
             if need > len(g.free_pages) + freed:
                 raise CacheError(f"the cache is full: slot {slot} needs {need} more pages of {self.page_size} tokens, "
                                  f"{len(g.free_pages) + freed} are free of {g.n_pages}")
         for g in self.groups:
             pages = g.pages[slot]
-            if g.needs.window is not None:
-                # the step's first query (position `old`) still reads back to old - window + 1
-                first_kept = max(old - g.needs.window + 1, 0) // self.page_size
-                for pn in range(min(first_kept, len(pages))):
-                    if pages[pn] >= 0:
-                        g.free_pages.append(pages[pn])
-                        pages[pn] = -1
-            else:
-                first_kept = 0
-            changed = False
+            # the step's first query (position `old`) still reads back to old - window + 1
+            first_kept = self._first_kept(g, old)
+            changed = []
+            for pn in range(min(first_kept, len(pages)) - 1, -1, -1):
+                if pages[pn] < 0:
+                    break                       # everything before an entry given back was given back earlier
+                g.free_pages.append(pages[pn])
+                pages[pn] = -1
+                changed.append(pn)
             while len(pages) < n_pg:
                 pn = len(pages)
                 pages.append(g.free_pages.pop() if pn >= first_kept else -1)
-                changed = True
-            if changed or g.needs.window is not None:
+                changed.append(pn)
+            if changed:
                 row = g.table_host[slot]
-                for pn, p in enumerate(pages):
-                    row[pn] = max(p, 0)
+                for pn in changed:
+                    row[pn] = max(pages[pn], 0)
                 g.dirty.add(slot)
         self.live[slot] = new
         return old
+
+    def truncate(self, slot: int, length: int):
+        """Forget the slot's tokens from ``length`` on (a step that failed after extend): their pages return
+        to the pools.  Pages that a windowed group gave back while the slot grew stay given back; no query at
+        or beyond ``length`` reads them."""
+        have = self.length(slot)
+        if not 0 <= length <= have:
+            raise CacheError(f"slot {slot}: cannot truncate {have} tokens to {length}")
+        n_pg = -(-length // self.page_size)
+        for g in self.groups:
+            pages = g.pages[slot]
+            while len(pages) > n_pg:
+                p = pages.pop()
+                if p >= 0:
+                    g.free_pages.append(p)
+        self.live[slot] = length
 
     def extend_one(self, slot: int) -> int:
         """extend(slot, 1) for the decode loop: nothing but the length changes while the token fits the

@@ -9,7 +9,6 @@ from --config and --seed.
 """
 from __future__ import annotations
 
-import dataclasses
 import json
 import os
 import sys
@@ -126,30 +125,20 @@ def run_generation(args):
     if not os.path.isdir(model_path):
         raise FileNotFoundError(f"model folder not found: {model_path} (there is no download: give a local folder)")
 
-    raw = read_config_json(model_path)
-    model_type = args.model_type
-    if model_type == "auto":
-        model_type = "minicpm4" if raw.get("sparse_config") else "minicpm"
+    # 'minicpm4' switches the block-sparse attention on, 'minicpm' (and 'llama') off (cpmcu/common/utils.py:123);
+    # 'auto' leaves it to the architecture, which turns it on iff its configuration describes it
+    apply_sparse = {"minicpm4": True, "auto": None}.get(args.model_type, False)
     tokenizer = load_tokenizer(model_path)
     llm = LLM(model_path, memory_limit=args.memory_limit, chunk_length=args.chunk_length, dtype=args.dtype,
-              cuda_graph=args.hip_graph, apply_sparse=(model_type == "minicpm4"),
+              cuda_graph=args.hip_graph, apply_sparse=apply_sparse,
               sink_window_size=args.sink_window_size, block_window_size=args.block_window_size,
               sparse_topk_k=args.sparse_topk_k, sparse_switch=args.sparse_switch,
               use_compress_lse=args.use_compress_lse, temperature=args.temperature, random_seed=args.random_seed,
-              max_tokens=args.max_tokens, max_seq_len=args.max_seq_len, max_batch=args.batch)
+              max_tokens=args.max_tokens, max_seq_len=args.max_seq_len, max_batch=args.batch,
+              minicpm4_yarn=args.minicpm4_yarn)
     llm.tokenizer = tokenizer
     llm.perf.enabled = bool(args.perf)
-    if args.minicpm4_yarn:
-        from .config.minicpm4_yarn import MINICPM4_YARN_FACTORS
-        from .config.minicpm import RopeScaling
-        if llm.config.head_dim != 2 * len(MINICPM4_YARN_FACTORS):
-            raise ValueError(f"--minicpm4-yarn holds factors for head_dim {2 * len(MINICPM4_YARN_FACTORS)}, "
-                             f"the model has {llm.config.head_dim}")
-        rs = llm.config.rope_scaling
-        orig = rs.original_max_position_embeddings if rs else llm.config.max_position_embeddings
-        llm.config = dataclasses.replace(llm.config, rope_scaling=RopeScaling(
-            "longrope", MINICPM4_YARN_FACTORS, MINICPM4_YARN_FACTORS, orig))
-    prompts = make_prompts(args, tokenizer, llm.config.vocab_size)
+    prompts = make_prompts(args, tokenizer, llm.config.vocabulary_size)
     log(f"Input tokens: {[len(p) for p in prompts]}")
     terminators = []
     if not args.ignore_eos:

@@ -85,6 +85,18 @@ class ModelConfig:
         """config.json content that from_dict reads back to an equal object."""
         raise NotImplementedError
 
+    # What the engine, the generation loop and the front end ask of any configuration, whatever its own
+    # keys are called:
     @property
     def stop_token_ids(self):
+        """Token ids that end a sequence."""
         return ()
+
+    @property
+    def vocabulary_size(self) -> int:  # pragma: no cover - interface
+        raise NotImplementedError
+
+    @property
+    def longest_sequence(self) -> Optional[int]:
+        """Positions the model is meant for (None: no limit of its own); the engine's default max_seq_len."""
+        return None

@@ -129,6 +129,14 @@ class MiniCPMConfig(ModelConfig):
     def stop_token_ids(self):
         return self.eos_token_ids
 
+    @property
+    def vocabulary_size(self) -> int:
+        return self.vocab_size
+
+    @property
+    def longest_sequence(self) -> Optional[int]:
+        return self.max_position_embeddings
+
     @classmethod
     def from_dict(cls, raw: Dict[str, Any]) -> "MiniCPMConfig":
         arch = raw.get("architectures") or ["MiniCPMForCausalLM"]

@@ -31,7 +31,9 @@ MODULES: Dict[str, List[str]] = {
     "sparse": ["sparse.hip"],
     "qkv": ["qkv_rope.hip", "strip.hip"],
 }
-HEADERS = ["common.h", "no_alloc.h"]
+HEADERS = ["common.h"]
+# headers of single libraries
+MODULE_HEADERS: Dict[str, List[str]] = {"attention": ["no_alloc.h"]}
 
 # -packed-fp32-ops off: the compiler must not form packed float instructions on its own
 HIPCC_FLAGS = [
@@ -68,7 +70,7 @@ def _hipcc() -> str:
 def _digest(module: str) -> str:
     h = hashlib.sha256()
     h.update(" ".join(_flags(module)).encode())
-    for name in HEADERS + MODULES[module]:
+    for name in HEADERS + MODULE_HEADERS.get(module, []) + MODULES[module]:
         with open(os.path.join(HERE, name), "rb") as f:
             h.update(name.encode())
             h.update(f.read())

@@ -101,6 +101,11 @@ struct SelectParams {
     float scale;
     int ks, st, bs, init_blocks, topk, window_blocks, dense_len;
     int max_ck, max_blocks, max_sel;
+    // Contexts whose scores and ranking arrays do not fit into LDS keep them in global scratch instead, a row
+    // of spill_stride floats for every (token, kv head): [scores ...][ranking arrays]; null: all in LDS
+    float* spill;
+    long spill_stride;
+    int score_spilled, work_spilled;
 };
 
 template <typename T>
@@ -110,15 +115,15 @@ __global__ __launch_bounds__(256) void sparse_select_kernel(const T* __restrict_
                                                            int* __restrict__ sel_blocks, int* __restrict__ sel_count) {
     extern __shared__ float lds[];
     __shared__ float red[17];
-    float* tmp = lds;
-    float* score = tmp + sp.max_ck;
-    float* pool = score + sp.max_ck;
-    int* flag = (int*)(pool + sp.max_blocks);
-    float* qs = (float*)(flag + sp.max_blocks);
-
     const int t = blockIdx.x, g = blockIdx.y, tid = threadIdx.x;
     const int p = positions[t];
     const long out_idx = (long)t * sp.nkv + g;
+    // tmp[max_ck] score[max_ck] pool[max_blocks] flag[max_blocks] in LDS, or in this row of the global scratch
+    float* tmp = sp.score_spilled ? sp.spill + out_idx * sp.spill_stride : lds;
+    float* score = tmp + sp.max_ck;
+    float* pool = score + sp.max_ck;
+    int* flag = (int*)(pool + sp.max_blocks);
+    float* qs = sp.score_spilled ? lds : (float*)(flag + sp.max_blocks);
     if (p + 1 <= sp.dense_len) {
         if (tid == 0) sel_count[out_idx] = -1;
         return;
@@ -290,13 +295,86 @@ template <int HD>
 __global__ void select_scores_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ ckpool, PagedView pv,
                                      const int* __restrict__ positions, const int* __restrict__ tok_slot,
                                      SelectParams sp, SelectScratch sc);
-__global__ void select_normalise_kernel(const int* __restrict__ positions, SelectParams sp, SelectScratch sc);
+__global__ void select_normalise_kernel(const int* __restrict__ positions, SelectParams sp, SelectScratch sc,
+                                        int stats_in_lds);
 __global__ void select_blocks_kernel(const int* __restrict__ positions, SelectParams sp, SelectScratch sc,
                                      int* __restrict__ sel_blocks, int* __restrict__ sel_count, int stats_off);
 template <int HD, int NW>
 __global__ void sparse_select_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ ckpool, PagedView pv,
                                           const int* __restrict__ positions, const int* __restrict__ tok_slot,
                                           SelectParams sp, int* __restrict__ sel_blocks, int* __restrict__ sel_count);
+
+// ---------------------------------------------------------------------------
+// Which kernels a selection runs as and where their arrays lie: decided on the host from the sizes alone, by
+// cpmcu_sparse_select and by cpmcu_sparse_select_scratch (which tells the caller how much scratch to bring).
+//   plain:        the plain kernel (float32 engine, or asked for): scores and ranking arrays in LDS, or all of
+//                 them in a row of scratch when they exceed it
+//   few tokens:   scratch = [raw scores][groups' statistics][scores] (+ [ranking arrays] when LDS cannot hold them)
+//   many tokens:  the fused matrix-core kernel; scores, then also the ranking arrays, move to scratch rows when
+//                 LDS cannot hold them
+// ---------------------------------------------------------------------------
+static constexpr size_t SELECT_LDS_LIMIT = 60 * 1024;
+
+struct SelectPlan {
+    bool mfma, few;
+    int max_ck, max_ck4, max_blocks, n_groups, G;
+    bool score_spilled, work_spilled, fused_blocks, stats_in_lds;
+    size_t lds_main, lds_stats;
+    long off_stats, off_score, off_spill, spill_stride, need;     // in floats
+};
+
+static long round4(long v) { return (v + 3) / 4 * 4; }
+
+static SelectPlan select_plan(int dtype, int n, int nh, int nkv, int hd, int ks, int st, int bs, int max_pos,
+                              int force_plain, bool have_scratch) {
+    SelectPlan pl{};
+    pl.G = nh / nkv;
+    pl.max_ck = max_pos < ks ? 1 : (max_pos - ks) / st + 1;
+    pl.max_ck4 = (int)round4(pl.max_ck);
+    pl.max_blocks = max_pos / bs + 1;
+    pl.n_groups = (pl.max_ck + 63) / 64;
+    const long rows = (long)n * nkv;
+    pl.mfma = dtype == CPMCU_BF16 && force_plain != 1 && hd >= 16 && hd <= 128 && hd % 16 == 0;
+    if (!pl.mfma) {
+        const size_t all = sizeof(float) * ((size_t)2 * pl.max_ck + 2 * pl.max_blocks + hd + 8);
+        pl.score_spilled = pl.work_spilled = all > SELECT_LDS_LIMIT;
+        pl.lds_main = pl.score_spilled ? sizeof(float) * (hd + 8) : all;
+        pl.spill_stride = round4(2L * pl.max_ck + 2L * pl.max_blocks);
+        pl.need = pl.score_spilled ? rows * pl.spill_stride : 0;
+        return pl;
+    }
+    const size_t score_b = sizeof(float) * (size_t)(pl.max_ck4 + 4);
+    const size_t work_b = sizeof(float) * (size_t)select_work_floats(pl.max_blocks);
+    pl.score_spilled = score_b + work_b > SELECT_LDS_LIMIT;
+    pl.work_spilled = work_b > SELECT_LDS_LIMIT;
+    pl.lds_main = (pl.score_spilled ? 0 : score_b) + (pl.work_spilled ? 0 : work_b);
+    if (pl.lds_main == 0) pl.lds_main = 16;
+    pl.few = rows <= 256 && (have_scratch || pl.score_spilled);
+    if (pl.few) {
+        pl.off_stats = round4(rows * pl.max_ck * pl.G);
+        pl.off_score = pl.off_stats + round4(rows * pl.n_groups * pl.G * 2);
+        pl.off_spill = pl.off_score + round4(rows * pl.max_ck);
+        pl.spill_stride = pl.work_spilled ? round4(select_work_floats(pl.max_blocks)) : 0;
+        pl.need = pl.off_spill + rows * pl.spill_stride;
+        pl.lds_stats = sizeof(float) * ((size_t)pl.n_groups * pl.G * 2 + 2 * pl.G);
+        const size_t main8 = (pl.lds_main + 7) / 8 * 8;
+        pl.fused_blocks = !pl.score_spilled && main8 + pl.lds_stats <= SELECT_LDS_LIMIT && force_plain != 2;
+        pl.stats_in_lds = pl.lds_stats <= SELECT_LDS_LIMIT;
+        if (!pl.stats_in_lds) pl.lds_stats = sizeof(float) * 2 * pl.G;
+    } else {
+        pl.spill_stride = pl.score_spilled ? pl.max_ck4 + (pl.work_spilled ? round4(select_work_floats(pl.max_blocks)) : 0) : 0;
+        pl.need = rows * pl.spill_stride;
+    }
+    return pl;
+}
+
+// Floats of scratch that cpmcu_sparse_select wants for these sizes (0: none).  bf16 steps of few tokens run
+// faster with it (three kernels of many small workgroups); contexts beyond what LDS holds need it.
+extern "C" long cpmcu_sparse_select_scratch(int dtype, int n, int nh, int nkv, int hd, int ks, int st, int bs,
+                                            int max_pos, int force_plain) {
+    if (n <= 0 || nkv <= 0 || nh <= 0 || nh % nkv || st <= 0 || bs <= 0 || ks <= 0) return 0;
+    return select_plan(dtype, n, nh, nkv, hd, ks, st, bs, max_pos, force_plain, true).need;
+}
 
 extern "C" const char* cpmcu_sparse_select(const void* q, const void* ckpool, int dtype, int n, int nh, int nkv,
                                            int hd, float scale, const int* page_table, int table_width,
@@ -312,106 +390,106 @@ extern "C" const char* cpmcu_sparse_select(const void* q, const void* ckpool, in
     CPMCU_REQUIRE(window_blocks >= 1 && max_sel >= topk + window_blocks,
                   "sparse_select: block list of %d entries cannot hold topk %d + window %d", max_sel, topk,
                   window_blocks);
+    CPMCU_REQUIRE(dtype == CPMCU_F32 || dtype == CPMCU_BF16, "sparse_select: unknown dtype %d", dtype);
+    CPMCU_REQUIRE(max_pos >= 0, "sparse_select: negative position bound");
+    const SelectPlan pl = select_plan(dtype, n, nh, nkv, hd, ks, st, bs, max_pos, force_plain, scratch != nullptr);
+    CPMCU_REQUIRE(pl.need == 0 || (scratch && scratch_floats >= pl.need),
+                  "sparse_select: %d tokens at a context of up to %d tokens need %ld floats of scratch, %ld were given",
+                  n, max_pos + 1, pl.need, scratch ? scratch_floats : 0L);
+    CPMCU_REQUIRE(((uintptr_t)scratch & 15) == 0, "sparse_select: the scratch must be aligned to 16 bytes");
     SelectParams sp;
     sp.nh = nh; sp.nkv = nkv; sp.hd = hd; sp.scale = scale;
     sp.ks = ks; sp.st = st; sp.bs = bs; sp.init_blocks = init_blocks; sp.topk = topk;
     sp.window_blocks = window_blocks; sp.dense_len = dense_len;
-    sp.max_ck = max_pos < ks ? 1 : (max_pos - ks) / st + 1;
-    sp.max_blocks = max_pos / bs + 1;
+    sp.max_ck = pl.max_ck;
+    sp.max_blocks = pl.max_blocks;
     sp.max_sel = max_sel;
-    const size_t lds = sizeof(float) * ((size_t)2 * sp.max_ck + 2 * sp.max_blocks + hd + 8);
-    CPMCU_REQUIRE(lds <= 60 * 1024,
-                  "sparse_select: a context of %d tokens needs %zu bytes of LDS for its block scores (limit 61440)",
-                  max_pos + 1, lds);
+    sp.spill = nullptr;
+    sp.spill_stride = pl.spill_stride;
+    sp.score_spilled = pl.score_spilled ? 1 : 0;
+    sp.work_spilled = pl.work_spilled ? 1 : 0;
     dim3 grid(n, nkv);
     PagedView pv{page_table, table_width, page_size};
+    if (!pl.mfma) {
+        sp.spill = pl.score_spilled ? scratch : nullptr;
+        if (dtype == CPMCU_F32)
+            sparse_select_kernel<float><<<grid, 256, pl.lds_main, stream>>>((const float*)q, (const float*)ckpool, pv,
+                                                                            positions, tok_slot, sp, sel_blocks, sel_count);
+        else
+            sparse_select_kernel<bf16_t><<<grid, 256, pl.lds_main, stream>>>((const bf16_t*)q, (const bf16_t*)ckpool, pv,
+                                                                             positions, tok_slot, sp, sel_blocks, sel_count);
+        CPMCU_LAUNCH_CHECK("sparse_select");
+        return nullptr;
+    }
     // force_plain: 1 = the plain kernel whatever the type; 2 = matrix cores, but steps of few tokens with the
     // kernel that normalises the scores kept apart (as for contexts whose statistics do not fit into LDS)
-    if (dtype == CPMCU_BF16 && force_plain != 1 && hd >= 16 && hd <= 128 && hd % 16 == 0) {
-        const size_t lds2 = sizeof(float) * ((size_t)sp.max_ck + 4 + select_work_floats(sp.max_blocks));
-        CPMCU_REQUIRE(lds2 <= 60 * 1024,
-                      "sparse_select: a context of %d tokens needs %zu bytes of LDS for its block scores (limit 61440)",
-                      max_pos + 1, lds2);
-        const int G = nh / nkv;
-        if (scratch && n * nkv <= 256) {
-            // few tokens: raw scores and their softmax by many small workgroups through `scratch`, then one
-            // workgroup a (token, kv head) for the block list
-            SelectScratch sc;
-            sc.n_groups = (sp.max_ck + 63) / 64;
-            const long rows = (long)n * nkv;
-            const long need = rows * ((long)sp.max_ck * (G + 1) + (long)sc.n_groups * G * 2);
-            CPMCU_REQUIRE(scratch_floats >= need, "sparse_select: scratch of %ld floats, %ld needed", scratch_floats, need);
-            sc.sraw = scratch;
-            sc.stats = sc.sraw + rows * sp.max_ck * G;
-            sc.score = sc.stats + rows * sc.n_groups * G * 2;
-            dim3 sgrid(n, nkv * ((G + 15) / 16), sc.n_groups);
-            CPMCU_REQUIRE(sgrid.y <= 65535 && sgrid.z <= 65535, "sparse_select: too many head tiles or compressed keys");
-            CPMCU_REQUIRE(G <= 256, "sparse_select: %d heads a kv head (256 are taken)", G);
+    if (pl.few) {
+        // few tokens: raw scores and their softmax by many small workgroups through `scratch`, then one
+        // workgroup a (token, kv head) for the block list
+        SelectScratch sc;
+        sc.n_groups = pl.n_groups;
+        sc.sraw = scratch;
+        sc.stats = scratch + pl.off_stats;
+        sc.score = scratch + pl.off_score;
+        sp.spill = scratch + pl.off_spill;
+        const int G = pl.G;
+        dim3 sgrid(n, nkv * ((G + 15) / 16), sc.n_groups);
+        CPMCU_REQUIRE(sgrid.y <= 65535 && sgrid.z <= 65535, "sparse_select: too many head tiles or compressed keys");
+        CPMCU_REQUIRE(G <= 256, "sparse_select: %d heads a kv head (256 are taken)", G);
 #define SCORES(HDv)                                                                                               \
-            select_scores_kernel<HDv><<<sgrid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)ckpool, pv, positions, \
-                                                                 tok_slot, sp, sc)
-            switch (hd) {
-                case 16: SCORES(16); break;
-                case 32: SCORES(32); break;
-                case 48: SCORES(48); break;
-                case 64: SCORES(64); break;
-                case 80: SCORES(80); break;
-                case 96: SCORES(96); break;
-                case 112: SCORES(112); break;
-                default: SCORES(128); break;
-            }
+        select_scores_kernel<HDv><<<sgrid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)ckpool, pv, positions, \
+                                                             tok_slot, sp, sc)
+        switch (hd) {
+            case 16: SCORES(16); break;
+            case 32: SCORES(32); break;
+            case 48: SCORES(48); break;
+            case 64: SCORES(64); break;
+            case 80: SCORES(80); break;
+            case 96: SCORES(96); break;
+            case 112: SCORES(112); break;
+            default: SCORES(128); break;
+        }
 #undef SCORES
-            CPMCU_LAUNCH_CHECK("select_scores");
-            const size_t lds3 = sizeof(float) * ((size_t)sc.n_groups * G * 2 + 2 * G);
-            CPMCU_REQUIRE(lds3 <= 60 * 1024, "sparse_select: %d groups of compressed keys x %d heads exceed LDS", sc.n_groups, G);
-            const size_t lds2e = (lds2 + 7) / 8 * 8;
-            if (lds2e + lds3 <= 60 * 1024 && force_plain != 2) {
-                // the last kernel normalises the scores itself (the same sums in the same order): one kernel
-                // of the chain less
-                select_blocks_kernel<<<grid, 1024, lds2e + lds3, stream>>>(positions, sp, sc, sel_blocks, sel_count,
-                                                                         (int)(lds2e / sizeof(float)));
-                CPMCU_LAUNCH_CHECK("select_blocks");
-                return nullptr;
-            }
-            select_normalise_kernel<<<dim3(n, nkv, (sp.max_ck + 255) / 256), 256, lds3, stream>>>(positions, sp, sc);
-            CPMCU_LAUNCH_CHECK("select_normalise");
-            select_blocks_kernel<<<grid, 1024, lds2, stream>>>(positions, sp, sc, sel_blocks, sel_count, 0);
+        CPMCU_LAUNCH_CHECK("select_scores");
+        if (pl.fused_blocks) {
+            // the last kernel normalises the scores itself (the same sums in the same order): one kernel
+            // of the chain less
+            const size_t main8 = (pl.lds_main + 7) / 8 * 8;
+            select_blocks_kernel<<<grid, 1024, main8 + pl.lds_stats, stream>>>(positions, sp, sc, sel_blocks, sel_count,
+                                                                              (int)(main8 / sizeof(float)));
             CPMCU_LAUNCH_CHECK("select_blocks");
             return nullptr;
         }
-        // few tokens (decode steps): 16 wavefronts share a (token, kv head)'s compressed keys; many: 4
-#define LAUNCH(HDv)                                                                                          \
-        do {                                                                                                 \
-            if (n * nkv <= 256)                                                                              \
-                sparse_select_mfma_kernel<HDv, 16><<<grid, 1024, lds2, stream>>>(                            \
-                    (const bf16_t*)q, (const bf16_t*)ckpool, pv, positions, tok_slot, sp, sel_blocks, sel_count); \
-            else                                                                                             \
-                sparse_select_mfma_kernel<HDv, 4><<<grid, 256, lds2, stream>>>(                              \
-                    (const bf16_t*)q, (const bf16_t*)ckpool, pv, positions, tok_slot, sp, sel_blocks, sel_count); \
-        } while (0)
-        switch (hd) {
-            case 16: LAUNCH(16); break;
-            case 32: LAUNCH(32); break;
-            case 48: LAUNCH(48); break;
-            case 64: LAUNCH(64); break;
-            case 80: LAUNCH(80); break;
-            case 96: LAUNCH(96); break;
-            case 112: LAUNCH(112); break;
-            default: LAUNCH(128); break;
-        }
-#undef LAUNCH
-        CPMCU_LAUNCH_CHECK("sparse_select_mfma");
+        select_normalise_kernel<<<dim3(n, nkv, (sp.max_ck + 255) / 256), 256, pl.lds_stats, stream>>>(
+            positions, sp, sc, pl.stats_in_lds ? 1 : 0);
+        CPMCU_LAUNCH_CHECK("select_normalise");
+        select_blocks_kernel<<<grid, 1024, pl.lds_main, stream>>>(positions, sp, sc, sel_blocks, sel_count, 0);
+        CPMCU_LAUNCH_CHECK("select_blocks");
         return nullptr;
     }
-    if (dtype == CPMCU_F32)
-        sparse_select_kernel<float><<<grid, 256, lds, stream>>>((const float*)q, (const float*)ckpool, pv, positions,
-                                                                tok_slot, sp, sel_blocks, sel_count);
-    else if (dtype == CPMCU_BF16)
-        sparse_select_kernel<bf16_t><<<grid, 256, lds, stream>>>((const bf16_t*)q, (const bf16_t*)ckpool, pv,
-                                                                 positions, tok_slot, sp, sel_blocks, sel_count);
-    else
-        CPMCU_FAIL("sparse_select: unknown dtype %d", dtype);
-    CPMCU_LAUNCH_CHECK("sparse_select");
+    sp.spill = pl.score_spilled ? scratch : nullptr;
+    // few tokens (decode steps): 16 wavefronts share a (token, kv head)'s compressed keys; many: 4
+#define LAUNCH(HDv)                                                                                          \
+    do {                                                                                                     \
+        if (n * nkv <= 256)                                                                                  \
+            sparse_select_mfma_kernel<HDv, 16><<<grid, 1024, pl.lds_main, stream>>>(                         \
+                (const bf16_t*)q, (const bf16_t*)ckpool, pv, positions, tok_slot, sp, sel_blocks, sel_count); \
+        else                                                                                                 \
+            sparse_select_mfma_kernel<HDv, 4><<<grid, 256, pl.lds_main, stream>>>(                           \
+                (const bf16_t*)q, (const bf16_t*)ckpool, pv, positions, tok_slot, sp, sel_blocks, sel_count); \
+    } while (0)
+    switch (hd) {
+        case 16: LAUNCH(16); break;
+        case 32: LAUNCH(32); break;
+        case 48: LAUNCH(48); break;
+        case 64: LAUNCH(64); break;
+        case 80: LAUNCH(80); break;
+        case 96: LAUNCH(96); break;
+        case 112: LAUNCH(112); break;
+        default: LAUNCH(128); break;
+    }
+#undef LAUNCH
+    CPMCU_LAUNCH_CHECK("sparse_select_mfma");
     return nullptr;
 }
 
@@ -440,14 +518,15 @@ __global__ __launch_bounds__(NW * 64) void sparse_select_mfma_kernel(
     extern __shared__ float lds[];
     __shared__ float stat_s[NW][16][2];
     __shared__ int wave_tot[NW];
-    float* score = lds;
-    float* work = score + (sp.max_ck + 3) / 4 * 4;
-
     const int t = blockIdx.x, kvh = blockIdx.y, tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63, n = lane & 15, g = lane >> 4;
     const int p = positions[t];
     const long out_idx = (long)t * sp.nkv + kvh;
+    const int max_ck4 = (sp.max_ck + 3) / 4 * 4;
+    float* row_spill = sp.spill + out_idx * sp.spill_stride;
+    float* score = sp.score_spilled ? row_spill : lds;
+    float* work = sp.work_spilled ? row_spill + max_ck4 : (sp.score_spilled ? lds : lds + max_ck4);
     if (p + 1 <= sp.dense_len) {
         if (tid == 0) sel_count[out_idx] = -1;
         return;
@@ -669,8 +748,8 @@ __global__ __launch_bounds__(256) void select_scores_kernel(
 }
 
 __global__ __launch_bounds__(256) void select_normalise_kernel(const int* __restrict__ positions, SelectParams sp,
-                                                               SelectScratch sc) {
-    extern __shared__ float2 gst[];          // [group][head] (max, sum), then ms/inv behind it
+                                                               SelectScratch sc, int stats_in_lds) {
+    extern __shared__ float2 gst[];          // [group][head] (max, sum) if they fit, then ms/inv behind them
     const int t = blockIdx.x, kvh = blockIdx.y, tid = threadIdx.x;
     const int p = positions[t];
     if (p + 1 <= sp.dense_len) return;
@@ -679,23 +758,27 @@ __global__ __launch_bounds__(256) void select_normalise_kernel(const int* __rest
     if ((int)blockIdx.z * 256 >= n_vis) return;
     const long row = (long)t * sp.nkv + kvh;
     const int groups = (n_vis + 63) / 64;
-    float* ms = (float*)(gst + (long)sc.n_groups * G);
+    float* ms = stats_in_lds ? (float*)(gst + (long)sc.n_groups * G) : (float*)gst;
     float* inv = ms + G;
     // all threads fetch the groups' (max, sum) at once; then a thread a head merges them in their order,
     // so the result does not depend on which workgroup forms it
     const float2* st = (const float2*)(sc.stats + row * sc.n_groups * G * 2);
-    for (int i = tid; i < groups * G; i += 256) gst[i] = st[i];
-    __syncthreads();
-    if (tid < G) {
+    const float2* src = st;
+    if (stats_in_lds) {
+        for (int i = tid; i < groups * G; i += 256) gst[i] = st[i];
+        __syncthreads();
+        src = gst;
+    }
+    for (int h = tid; h < G; h += 256) {
         float mm = -INFINITY;
-        for (int gi = 0; gi < groups; ++gi) mm = fmaxf(mm, gst[gi * G + tid].x);
+        for (int gi = 0; gi < groups; ++gi) mm = fmaxf(mm, src[gi * G + h].x);
         float ll = 0.f;
         for (int gi = 0; gi < groups; ++gi) {
-            const float2 v = gst[gi * G + tid];
+            const float2 v = src[gi * G + h];
             ll += v.y * exp2f(v.x - mm);
         }
-        ms[tid] = mm;
-        inv[tid] = ll > 0.f ? 1.0f / ll : 0.f;
+        ms[h] = mm;
+        inv[h] = ll > 0.f ? 1.0f / ll : 0.f;
     }
     __syncthreads();
     const int j = blockIdx.z * 256 + tid;
@@ -709,18 +792,20 @@ __global__ __launch_bounds__(256) void select_normalise_kernel(const int* __rest
 }
 
 // stats_off (in floats, or 0): where in LDS the groups' (max, sum) pairs go when this kernel does the work of
-// select_normalise_kernel itself; 0: the scores come ready in sc.score
+// select_normalise_kernel itself; 0: the scores come ready in sc.score (and are read from there, not copied
+// into LDS, when sp.score_spilled says that LDS cannot hold them)
 __global__ __launch_bounds__(1024) void select_blocks_kernel(const int* __restrict__ positions, SelectParams sp,
                                                              SelectScratch sc, int* __restrict__ sel_blocks,
                                                              int* __restrict__ sel_count, int stats_off) {
     constexpr int NW = 16;
     extern __shared__ float lds[];
     __shared__ int wave_tot[NW];
-    float* score = lds;
-    float* work = score + (sp.max_ck + 3) / 4 * 4;
     const int t = blockIdx.x, kvh = blockIdx.y, tid = threadIdx.x;
     const int p = positions[t];
     const long out_idx = (long)t * sp.nkv + kvh;
+    float* score = sp.score_spilled ? sc.score + out_idx * sp.max_ck : lds;
+    float* work = sp.work_spilled ? sp.spill + out_idx * sp.spill_stride
+                                  : (sp.score_spilled ? lds : lds + (sp.max_ck + 3) / 4 * 4);
     if (p + 1 <= sp.dense_len) {
         if (tid == 0) sel_count[out_idx] = -1;
         return;
@@ -756,7 +841,7 @@ __global__ __launch_bounds__(1024) void select_blocks_kernel(const int* __restri
             for (int h = 0; h < G; ++h) a += exp2f(s[(long)h * sp.max_ck] - ms[h]) * inv[h];
             score[j] = a;
         }
-    } else {
+    } else if (!sp.score_spilled) {
         for (int j = tid; j < n_vis; j += NW * 64) score[j] = sc.score[out_idx * sp.max_ck + j];
     }
     __syncthreads();

@@ -12,7 +12,7 @@ step function are this engine's own.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Dict, List, Optional, Sequence, Tuple
+from typing import Any, Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
@@ -34,14 +34,16 @@ class StepError(ValueError):
 class EngineOptions:
     dtype: str = "bfloat16"                 # 'bfloat16' (serving kernels) or 'float32' (everything in true 32-bit)
     max_tokens: int = 8192                  # tokens all live sequences hold together (each rounded up to a page)
-    max_seq_len: Optional[int] = None       # longest sequence; default: the model's max_position_embeddings
+    max_seq_len: Optional[int] = None       # longest sequence; default: what the configuration says the model is for
     max_slots: Optional[int] = None         # live sequences; default: one per page, at most 1024
     max_step_tokens: int = 2048             # tokens one forward pass carries (the reference's chunk_length)
     page_size: int = 64
     device: str = "cuda:0"
     hip_graph: bool = False                 # replay single-token steps from a captured graph
-    sparse: bool = True                     # honour sparse_config (False: dense attention everywhere)
     tiled_weights: bool = True              # second copy of the linear weights laid out for decode steps (bf16)
+    # options of the architecture's own (those its registry entry declares, e.g. 'sparse' for MiniCPM4)
+    model_options: Dict[str, Any] = field(default_factory=dict)
+    max_graphs: int = 32                    # captured decode steps kept (one per batch size and position bound)
 
 
 @dataclass
@@ -67,10 +69,12 @@ class Engine:
         if options.page_size <= 0 or options.page_size % 32:
             raise ValueError(f"page_size {options.page_size}: the cache kernels lay a page out in chunks of 32 tokens; "
                              f"give a positive multiple of 32")
-        max_seq_len = options.max_seq_len or getattr(config, "max_position_embeddings", None) or options.max_tokens
+        max_seq_len = options.max_seq_len or config.longest_sequence or options.max_tokens
         self.max_seq_len = int(max_seq_len)
         self.workspace = Workspace(self.device)
-        self.runtime = Runtime(self.device, self.dtype, self.workspace, self.max_seq_len, options.tiled_weights)
+        # parts check here, at bind time, what their kernels take of these sizes: an engine that was built runs
+        self.runtime = Runtime(self.device, self.dtype, self.workspace, self.max_seq_len, options.tiled_weights,
+                               options.page_size)
         with torch.cuda.device(self.device):
             model.bind_all(tensors, self.runtime)
         n_pages = -(-options.max_tokens // options.page_size)
@@ -99,10 +103,7 @@ class Engine:
         arch = get_architecture(architecture_name(raw))
         if config is None:
             config = arch.config_class.from_dict(raw)
-        tied = None
-        if arch.tie_key is not None:
-            tied = arch.tie_key not in checkpoint_names(model_dir)
-        model = arch.build(config, tied=tied, sparse=options.sparse)
+        model = arch.build_model(config, options.model_options, checkpoint_names(model_dir))
         tensors = load_tensors(
             model_dir, model.all_weight_specs(), device=options.device,
             split_fused=(lambda n, t: arch.split_fused(config, n, t)) if arch.split_fused else None,
@@ -114,8 +115,7 @@ class Engine:
                      options: Optional[EngineOptions] = None) -> "Engine":
         options = options or EngineOptions()
         arch = get_architecture(config.architecture)
-        tied = (arch.tie_key not in tensors) if arch.tie_key is not None else None
-        model = arch.build(config, tied=tied, sparse=options.sparse)
+        model = arch.build_model(config, options.model_options, tensors.keys())
         from ..weights.loader import _compare
         _compare(model.all_weight_specs(), {k: tuple(v.shape) for k, v in tensors.items()}, "the given tensors")
         dev = torch.device(options.device)
@@ -137,7 +137,6 @@ class Engine:
             raise StepError("a step needs at least one sequence")
         seen = set()
         V = self.vocab_size
-        pages = 0
         for e in entries:
             if e.slot in seen:
                 raise StepError(f"slot {e.slot} occurs twice in one step")
@@ -158,10 +157,9 @@ class Engine:
             for w in e.want:
                 if not 0 <= int(w) < n:
                     raise StepError(f"slot {e.slot}: wanted place {w} is outside the {n} tokens of this step")
-            pages += self.cache.pages_needed(e.slot, have + n)
-        if pages > self.cache.free_page_count():
-            raise StepError(f"the cache is full: this step needs {pages} more pages of {self.cache.page_size} tokens, "
-                            f"{self.cache.free_page_count()} are free (max_tokens={self.options.max_tokens})")
+        full = self.cache.room_for([(e.slot, len(e.tokens)) for e in entries])
+        if full is not None:
+            raise StepError(f"{full} (max_tokens={self.options.max_tokens})")
 
     def _chunks(self, entries: Sequence[StepEntry]):
         """Cut a step into forward passes of at most max_step_tokens tokens.  Yields lists of
@@ -244,16 +242,23 @@ class Engine:
                 raise StepError(f"slot {s}: {have} cached + 1 new tokens exceed the longest sequence this engine "
                                 f"holds ({self.max_seq_len})")
             pages += have % cache.page_size == 0
-        if pages > cache.free_page_count():
-            raise StepError(f"the cache is full: this step needs {pages} more pages of {cache.page_size} tokens, "
-                            f"{cache.free_page_count()} are free (max_tokens={self.options.max_tokens})")
+        if pages:
+            # a token that opens a page: ask the groups (one that keeps a window gives a page back for it)
+            full = cache.room_for([(s, 1) for s in slots])
+            if full is not None:
+                raise StepError(f"{full} (max_tokens={self.options.max_tokens})")
+        before = [live[s] for s in slots]
         pos = np.fromiter((cache.extend_one(s) for s in slots), dtype=np.int32, count=B)
         cache.sync()
         sl = np.asarray(slots, dtype=np.int32)
         graph = bool(self.options.hip_graph)
         rows = np.arange(B, dtype=np.int32) if graph else np.asarray(want_rows, dtype=np.int32)
         host = np.concatenate([tok.astype(np.int32), pos, sl, np.arange(B + 1, dtype=np.int32), sl, pos + 1, rows])
-        logits = self._run(host, B, B, [1] * B, int(pos.max()), True, graph, int(rows.size), device_tokens)
+        try:
+            logits = self._run(host, B, B, [1] * B, int(pos.max()), True, graph, int(rows.size), device_tokens)
+        except BaseException:
+            self._roll_back(slots, before)
+            raise
         if not want_rows:
             return None
         if graph and want_rows != list(range(B)):
@@ -308,6 +313,8 @@ class Engine:
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g):
                 captured = self.model.forward(ctx)
+            while len(self._graphs) >= max(int(self.options.max_graphs), 1):
+                self._graphs.pop(next(iter(self._graphs)))      # the oldest capture goes
             self._graphs[key] = (g, meta, captured, self.workspace.generation)
         return logits
 
@@ -327,6 +334,7 @@ class Engine:
         rows: List[int] = []
         dest: List[int] = []
         o = 0
+        before = [cache.length(entries[i].slot) for i, _, _ in chunk]
         for bi, (i, a, b) in enumerate(chunk):
             e = entries[i]
             first = cache.extend(e.slot, b - a)
@@ -347,13 +355,26 @@ class Engine:
         cache.sync()
         want_rows = np.arange(B, dtype=np.int32) if graph else np.asarray(rows, dtype=np.int32)
         host = np.concatenate([tok, pos, tslot, cu, sslot, slen, want_rows])
-        logits = self._run(host, n, B, q_lens, int(pos.max()), single, graph, int(want_rows.size))
+        try:
+            logits = self._run(host, n, B, q_lens, int(pos.max()), single, graph, int(want_rows.size))
+        except BaseException:
+            self._roll_back([entries[i].slot for i, _, _ in chunk], before)
+            raise
         if rows:
             dest_t = torch.tensor([dest, rows], dtype=torch.long).to(self.device, non_blocking=True)
             if graph:
                 result.index_copy_(0, dest_t[0], logits.index_select(0, dest_t[1]))
             else:
                 result.index_copy_(0, dest_t[0], logits)
+
+    def _roll_back(self, slots: Sequence[int], lengths: Sequence[int]):
+        """A forward pass failed after the cache had made room for its tokens (a kernel refused a size, the
+        device ran out of memory): the slots forget that pass's tokens, so that lengths and cache rows agree
+        again.  Passes of the same step that had completed before stay (a step that validation refuses, by
+        contrast, changes nothing at all)."""
+        for s, n in zip(slots, lengths):
+            if s in self.cache.live and self.cache.length(s) > n:
+                self.cache.truncate(s, n)
 
     def _upload(self, host: np.ndarray, dst: torch.Tensor):
         """Step metadata to the device through pinned memory, without waiting for the GPU."""

@@ -28,21 +28,23 @@ class Completion:
     decode_time: float = 0.0
 
 
-def plan_batches(prompt_lens: Sequence[int], max_new_tokens: int, max_batch: int, max_tokens: int,
-                 page_size: int, max_seq_len: int) -> List[List[int]]:
+def plan_batches(prompt_lens: Sequence[int], max_new_tokens: int, max_batch: int,
+                 pages_to_hold: Callable[[int], Sequence[int]], capacity: Sequence[int],
+                 max_seq_len: int) -> List[List[int]]:
     """Split request indices into batches that run one after another.
 
-    Requests keep their order.  A batch takes requests while it has a slot for each and the
-    cache can hold every one of them at its full length (prompt + max_new_tokens, rounded up
-    to whole pages)."""
+    Requests keep their order.  A batch takes requests while it has a slot for each and every group of the
+    cache can hold every one of them at its full length (prompt + max_new_tokens).  How many pages of each
+    group a sequence of a given length holds is the cache's to say (``pages_to_hold(length)``, one number a
+    group: a group that keeps a window needs fewer than one that keeps everything); ``capacity`` is the
+    groups' pools."""
     if max_new_tokens < 1:
         raise ValueError("max_new_tokens must be at least 1")
     if max_batch < 1:
         raise ValueError("max_batch must be at least 1")
-    pages_total = max_tokens // page_size if max_tokens % page_size == 0 else -(-max_tokens // page_size)
     batches: List[List[int]] = []
     cur: List[int] = []
-    cur_pages = 0
+    cur_pages = [0] * len(capacity)
     for i, n in enumerate(prompt_lens):
         if n < 1:
             raise ValueError(f"request {i}: the prompt is empty")
@@ -50,14 +52,15 @@ def plan_batches(prompt_lens: Sequence[int], max_new_tokens: int, max_batch: int
         if total > max_seq_len:
             raise ValueError(f"request {i}: prompt of {n} + {max_new_tokens} new tokens exceeds the longest sequence "
                              f"the engine holds ({max_seq_len})")
-        pages = -(-total // page_size)
-        if pages > pages_total:
-            raise ValueError(f"request {i}: {total} tokens do not fit the cache of {max_tokens} tokens")
-        if cur and (len(cur) >= max_batch or cur_pages + pages > pages_total):
+        pages = list(pages_to_hold(total))
+        if any(p > c for p, c in zip(pages, capacity)):
+            raise ValueError(f"request {i}: {total} tokens do not fit the cache ({pages} pages needed, "
+                             f"{list(capacity)} in all)")
+        if cur and (len(cur) >= max_batch or any(a + p > c for a, p, c in zip(cur_pages, pages, capacity))):
             batches.append(cur)
-            cur, cur_pages = [], 0
+            cur, cur_pages = [], [0] * len(capacity)
         cur.append(i)
-        cur_pages += pages
+        cur_pages = [a + p for a, p in zip(cur_pages, pages)]
     if cur:
         batches.append(cur)
     return batches
@@ -74,8 +77,10 @@ def generate(engine: Engine, prompts: Sequence[Sequence[int]], max_new_tokens: i
     sampler = sampler or Sampler(temperature, seed)
     max_batch = max_batch or engine.cache.max_slots
     max_batch = min(max_batch, engine.cache.max_slots)
-    batches = plan_batches([len(p) for p in prompts], max_new_tokens, max_batch, engine.options.max_tokens,
-                           engine.cache.page_size, engine.max_seq_len)
+    step = int(getattr(engine, "max_step_tokens", 0)) or engine.max_seq_len
+    batches = plan_batches([len(p) for p in prompts], max_new_tokens, max_batch,
+                           lambda length: engine.cache.pages_to_hold(length, step), engine.cache.capacity(),
+                           engine.max_seq_len)
     results: List[Optional[Completion]] = [None] * len(prompts)
     run = _run_batch_overlapped if getattr(engine, "accepts_device_tokens", False) else _run_batch
     for batch in batches:

@@ -9,14 +9,12 @@ tokenizer is optional (token ids are first-class).
 """
 from __future__ import annotations
 
-import dataclasses
 import time
 from typing import Iterable, List, Optional, Sequence, Union
 
 import torch
 
 from .config.base import architecture_name, read_config_json
-from .config.minicpm import SparseConfig
 from .engine.engine import Engine, EngineOptions, StepEntry
 from .engine.generate import Completion, generate as _generate
 from .registry import get_architecture
@@ -32,7 +30,7 @@ class LLM:
                  chunk_length: int = 1024,
                  dtype=None,
                  cuda_graph: bool = False,
-                 apply_sparse: bool = False,
+                 apply_sparse: Optional[bool] = False,
                  sink_window_size: Optional[int] = None,
                  block_window_size: Optional[int] = None,
                  sparse_topk_k: Optional[int] = None,
@@ -43,7 +41,8 @@ class LLM:
                  max_tokens: Optional[int] = None,
                  max_seq_len: Optional[int] = None,
                  max_batch: Optional[int] = None,
-                 device: str = "cuda:0"):
+                 device: str = "cuda:0",
+                 minicpm4_yarn: bool = False):
         self.path = path
         raw = read_config_json(path)
         self.arch = get_architecture(architecture_name(raw))
@@ -55,26 +54,14 @@ class LLM:
         if dtype not in _DTYPE_NAMES:
             raise ValueError(f"Unsupported dtype: {dtype}")
         self.dtype = _DTYPE_NAMES[dtype]
-        if use_compress_lse:
-            raise ValueError("use_compress_lse is not supported: block scores are normalised over the compressed "
-                             "keys they are computed from")
-        # the reference's sparse flags (cpmcu/common/args.py:72-83) override config.json's sparse_config
-        sc = getattr(self.config, "sparse_config", None)
-        if apply_sparse and sc is None:
-            raise ValueError("apply_sparse: config.json has no sparse_config (kernel_size, kernel_stride, block_size ...)")
-        if apply_sparse:
-            over = {}
-            if sink_window_size is not None:
-                over["init_blocks"] = sink_window_size
-            if block_window_size is not None:
-                over["window_size"] = block_window_size * sc.block_size
-            if sparse_topk_k is not None:
-                over["topk"] = sparse_topk_k
-            if sparse_switch is not None:
-                over["dense_len"] = sparse_switch
-            if over:
-                sc = SparseConfig.from_dict({**sc.to_dict(), **over})
-                self.config = dataclasses.replace(self.config, sparse_config=sc)
+        # The reference's model flags (cpmcu/common/args.py:38-40, 72-83) go to the architecture, which knows
+        # what they mean for its configuration and which options of its model they switch; an architecture that
+        # has no such flags refuses any that is set.
+        flags = {"apply_sparse": apply_sparse, "sink_window_size": sink_window_size,
+                 "block_window_size": block_window_size, "sparse_topk_k": sparse_topk_k,
+                 "sparse_switch": sparse_switch, "use_compress_lse": use_compress_lse or None,
+                 "minicpm4_yarn": minicpm4_yarn or None}
+        self.config, self.model_options = self.arch.with_flags(self.config, flags)
         self.apply_sparse = apply_sparse
         self.memory_limit = memory_limit
         self.chunk_length = chunk_length
@@ -101,17 +88,18 @@ class LLM:
             total = torch.cuda.get_device_properties(torch.device(self.device)).total_memory
             weight_bytes = sum(os.path.getsize(f) for f in checkpoint_files(self.path))
             weight_bytes *= 2          # float32: upcast weights; bfloat16: the second copy in the decode layout
-            model = self.arch.build(self.config, sparse=self.apply_sparse)
+            model = self.arch.build_model(self.config, self.model_options)
             esize = 4 if self.dtype == "float32" else 2
             per_token = sum(sum(s.width / s.every for _, s in n.streams) for n in model.cache_needs()) * esize
             budget = total * self.memory_limit - weight_bytes - (2 << 30)
             if budget <= per_token * 64:
                 raise MemoryError(f"memory limit exceeded: {self.memory_limit:.0%} of {total / 2**30:.1f} GiB leaves "
                                   f"no room for a cache beside {weight_bytes / 2**30:.1f} GiB of weights")
-            limit = self.max_seq_len or self.config.max_position_embeddings
+            limit = self.max_seq_len or self.config.longest_sequence
             slots = self.max_batch or 1
-            self.max_tokens = int(min(budget // per_token, limit * slots) // 64 * 64)
-        self.max_total_length = min(self.max_tokens, self.max_seq_len or self.config.max_position_embeddings)
+            fit = budget // per_token
+            self.max_tokens = int((min(fit, limit * slots) if limit else fit) // 64 * 64)
+        self.max_total_length = min(self.max_tokens, self.max_seq_len or self.config.longest_sequence or self.max_tokens)
         return self.max_total_length
 
     def load_from_hf(self):
@@ -120,9 +108,8 @@ class LLM:
             raise RuntimeError("call init_storage() before load_from_hf()")
         opts = EngineOptions(dtype=self.dtype, max_tokens=self.max_tokens, max_seq_len=self.max_seq_len,
                              max_slots=self.max_batch, max_step_tokens=self.chunk_length, device=self.device,
-                             hip_graph=self.cuda_graph, sparse=self.apply_sparse)
-        raw = read_config_json(self.path)
-        # the engine reads config.json itself; sparse overrides are handed over through the typed config
+                             hip_graph=self.cuda_graph, model_options=dict(self.model_options))
+        # the engine reads config.json itself; what the flags changed is handed over through the typed config
         self.engine = Engine.from_dir(self.path, opts, config=self.config)
         self.engine.perf = self.perf
         return self

@@ -93,6 +93,58 @@ def ignore_tensor(cfg: MiniCPMConfig, name: str) -> bool:
     return "rotary_emb.inv_freq" in name
 
 
+def checkpoint_options(cfg: MiniCPMConfig, names) -> Dict[str, object]:
+    """Embeddings are tied when config.json is silent and the checkpoint holds no head (cpmcu/llm.py:136-137)."""
+    return {"tied": "lm_head.weight" not in names}
+
+
+def apply_flags(cfg: MiniCPMConfig, flags: Dict[str, object]) -> Tuple[MiniCPMConfig, Dict[str, object]]:
+    """The reference's front-end flags for this architecture (cpmcu/common/args.py:38-40, 72-83,
+    cpmcu/llm.py:31-36): ``apply_sparse`` switches InfLLM-v2 on, the sparse flags override single values of
+    config.json's sparse_config, ``minicpm4_yarn`` installs the built-in LongRoPE factors
+    (cpmcu/common/utils.py:181-207)."""
+    import dataclasses
+
+    from ..config.minicpm import RopeScaling, SparseConfig
+    known = {"apply_sparse", "sink_window_size", "block_window_size", "sparse_topk_k", "sparse_switch",
+             "use_compress_lse", "minicpm4_yarn"}
+    unknown = sorted(set(flags) - known)
+    if unknown:
+        raise ValueError(f"{ARCHITECTURE} does not know the flags {unknown} (it knows: {sorted(known)})")
+    if flags.get("use_compress_lse"):
+        raise ValueError("use_compress_lse is not supported: block scores are normalised over the compressed "
+                         "keys they are computed from")
+    options: Dict[str, object] = {}
+    if "apply_sparse" in flags:
+        options["sparse"] = bool(flags["apply_sparse"])
+    sc = cfg.sparse_config
+    if flags.get("apply_sparse"):
+        if sc is None:
+            raise ValueError("apply_sparse: config.json has no sparse_config (kernel_size, kernel_stride, block_size ...)")
+        over = {}
+        if "sink_window_size" in flags:
+            over["init_blocks"] = flags["sink_window_size"]
+        if "block_window_size" in flags:
+            over["window_size"] = flags["block_window_size"] * sc.block_size
+        if "sparse_topk_k" in flags:
+            over["topk"] = flags["sparse_topk_k"]
+        if "sparse_switch" in flags:
+            over["dense_len"] = flags["sparse_switch"]
+        if over:
+            cfg = dataclasses.replace(cfg, sparse_config=SparseConfig.from_dict({**sc.to_dict(), **over}))
+    if flags.get("minicpm4_yarn"):
+        from ..config.minicpm4_yarn import MINICPM4_YARN_FACTORS
+        if cfg.head_dim != 2 * len(MINICPM4_YARN_FACTORS):
+            raise ValueError(f"minicpm4_yarn holds factors for head_dim {2 * len(MINICPM4_YARN_FACTORS)}, "
+                             f"the model has {cfg.head_dim}")
+        rs = cfg.rope_scaling
+        orig = rs.original_max_position_embeddings if rs else cfg.max_position_embeddings
+        cfg = dataclasses.replace(cfg, rope_scaling=RopeScaling("longrope", MINICPM4_YARN_FACTORS,
+                                                                MINICPM4_YARN_FACTORS, orig))
+    return cfg, options
+
+
 register_architecture(Architecture(
-    name=ARCHITECTURE, config_class=MiniCPMConfig, build=build, split_fused=split_fused, ignore_tensor=ignore_tensor,
-    tie_key="lm_head.weight"))
+    name=ARCHITECTURE, config_class=MiniCPMConfig, build=build, options={"tied": None, "sparse": True},
+    split_fused=split_fused, ignore_tensor=ignore_tensor, checkpoint_options=checkpoint_options,
+    apply_flags=apply_flags))

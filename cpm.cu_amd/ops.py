@@ -382,15 +382,16 @@ def compress_keys(kpool: torch.Tensor, ckpool: torch.Tensor, nkv: int, page_tabl
                                                 _stream()))
 
 
-def sparse_select_scratch(n: int, nh: int, nkv: int, max_pos: int, kernel_size: int, kernel_stride: int) -> int:
-    """Floats of scratch with which sparse_select runs a step of few tokens as three kernels (raw scores and their
-    softmax by many small workgroups, then one workgroup a (token, kv head)); 0: the step has too many tokens
-    to gain."""
-    if n * nkv > 256:
-        return 0
-    max_ck = 1 if max_pos < kernel_size else (max_pos - kernel_size) // kernel_stride + 1
-    G = nh // nkv
-    return n * nkv * (max_ck * (G + 1) + -(-max_ck // 64) * G * 2)
+def sparse_select_scratch(dtype: torch.dtype, n: int, nh: int, nkv: int, hd: int, max_pos: int, kernel_size: int,
+                          kernel_stride: int, block_size: int, force_plain=False) -> int:
+    """Floats of scratch that sparse_select wants for a step of n tokens at positions up to max_pos (0: none).
+    bf16 steps of few tokens run as three kernels of many small workgroups through it; contexts whose scores
+    and ranking arrays exceed a workgroup's LDS keep them there instead (any step, both element types)."""
+    lib = _build.load("sparse")
+    f = lib.cpmcu_sparse_select_scratch
+    f.restype = c_long
+    return int(f(c_int(_DT[dtype]), c_int(n), c_int(nh), c_int(nkv), c_int(hd), c_int(kernel_size), c_int(kernel_stride),
+                 c_int(block_size), c_int(max_pos), c_int(int(force_plain))))
 
 
 def sparse_select(q: torch.Tensor, ckpool: torch.Tensor, nh: int, nkv: int, hd: int, scale: float,
@@ -399,7 +400,7 @@ def sparse_select(q: torch.Tensor, ckpool: torch.Tensor, nh: int, nkv: int, hd: 
                   window_blocks: int, dense_len: int, max_pos: int, sel_blocks: torch.Tensor, sel_count: torch.Tensor,
                   force_plain=False, scratch: Optional[torch.Tensor] = None):
     """Block list per (token, kv head): sel_count -1 = dense, else the ascending blocks to attend to.
-    scratch: float32 of at least sparse_select_scratch(...) elements (bf16 steps of few tokens use it).
+    scratch: float32 of at least sparse_select_scratch(...) elements, if that is not 0.
     force_plain: True = the plain kernel; 2 = steps of few tokens with the normalising kernel kept apart, as for
     contexts too long for the fused form (for tests)."""
     _need(q, "select q", shape=(None, nh * hd))

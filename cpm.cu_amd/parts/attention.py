@@ -33,6 +33,12 @@ class GQAAttention(Mixer):
                  position: Optional[PositionEncoding], scale: Optional[float] = None):
         if num_heads % num_kv_heads:
             raise ValueError(f"attention: {num_heads} heads are not a multiple of {num_kv_heads} kv heads")
+        if head_dim <= 0 or head_dim % 16 or head_dim > 256:
+            # the cache lays keys and values out in pieces of 16 features (the matrix cores' operands), and the
+            # plain attention kernel holds a head in 256 features; said here so that no engine is built that
+            # would fail at its first step
+            raise ValueError(f"attention: head_dim {head_dim} is not supported: the cache and attention kernels take "
+                             f"head sizes in steps of 16 up to 256")
         self.hidden_size = hidden_size
         self.nh, self.nkv, self.hd = num_heads, num_kv_heads, head_dim
         self.position = position
@@ -136,9 +142,17 @@ class InfLLMv2Attention(GQAAttention):
         self.init_blocks, self.topk, self.dense_len = init_blocks, topk, dense_len
         self.window_blocks = window_size // block_size
 
+    def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime):
+        super().bind(tensors, rt)
+        if rt.page_size % self.st:
+            raise ValueError(f"infllm_v2: kernel_stride {self.st} must divide the cache page of {rt.page_size} tokens "
+                             f"(a compressed key's row lies in the page of its first key)")
+
     def cache_needs(self) -> CacheNeeds:
         w = self.nkv * self.hd
         return CacheNeeds(streams=(("k", StreamSpec(w)), ("v", StreamSpec(w)), ("ck", StreamSpec(w, every=self.st))))
+
+    can_defer_last = True
 
     def forward(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool = True, row_scale=None,
                 defer_last: bool = False):
@@ -155,11 +169,8 @@ class InfLLMv2Attention(GQAAttention):
             max_sel = self.topk + self.window_blocks
             sel_blocks = ctx.ws.get("attn.sel_blocks", (n, self.nkv, max_sel), torch.int32)
             sel_count = ctx.ws.get("attn.sel_count", (n, self.nkv), torch.int32)
-            scratch = None
-            if q.dtype == torch.bfloat16:
-                need = ops.sparse_select_scratch(n, self.nh, self.nkv, ctx.max_pos, self.ks, self.st)
-                if need:
-                    scratch = ctx.ws.get("attn.sel_scores", (need,), torch.float32)
+            need = ops.sparse_select_scratch(q.dtype, n, self.nh, self.nkv, self.hd, ctx.max_pos, self.ks, self.st, self.bs)
+            scratch = ctx.ws.get("attn.sel_scores", (need,), torch.float32) if need else None
             ops.sparse_select(q, cache.streams["ck"], self.nh, self.nkv, self.hd, self.scale, cache.page_table,
                               cache.page_size, ctx.positions, ctx.tok_slot, self.ks, self.st, self.bs,
                               self.init_blocks, self.topk, self.window_blocks, self.dense_len, ctx.max_pos,

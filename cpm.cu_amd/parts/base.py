@@ -39,10 +39,9 @@ from ..cache.paged import CacheNeeds, CacheView, SequenceCache
 # ---------------------------------------------------------------------------
 @dataclass(frozen=True)
 class WeightSpec:
-    """A checkpoint tensor a part needs.  ``init`` tells the random-weights
-    writer how to draw it: 'matrix' N(0, std), 'norm' 1 + N(0, norm_std),
-    'table' like 'matrix'.  ``storage`` is the dtype it is written in and kept
-    in by the loader ('bfloat16', 'float32' or 'int32')."""
+    """A checkpoint tensor a part needs.  ``init`` names the rule by which the random-weights writer draws it
+    (weights.register_init_rule; built in: 'matrix' and 'table' N(0, std), 'norm' 1 + N(0, norm_std)).
+    ``storage`` is the dtype it is written in and kept in by the loader ('bfloat16', 'float32' or 'int32')."""
     name: str
     shape: Tuple[int, ...]
     init: str = "matrix"
@@ -88,6 +87,7 @@ class Runtime:
     workspace: Workspace
     max_seq_len: int              # longest sequence the engine holds
     tiled_weights: bool = True    # keep a second copy of linear weights in the decode product's layout
+    page_size: int = 64           # tokens a cache page
 
 
 @dataclass
@@ -228,7 +228,8 @@ class Mixer(Part):
         A subclass that overrides forward of a mixer that says yes takes the argument too, or says no here."""
         return False
 
-    # True if forward accepts ``defer_last=True`` and may then return a DeferredBranch
+    # True (set in the class that defines ``forward``) if that forward accepts ``defer_last=True`` and may then
+    # return a DeferredBranch
     can_defer_last = False
 
 
@@ -242,6 +243,16 @@ class FeedForward(Part):
 
     # True if forward accepts ``defer_last=True`` and may then return a DeferredBranch
     can_defer_last = False
+
+
+def forward_declares(part: Part, flag: str) -> bool:
+    """Whether the class that defines ``part.forward`` sets the class attribute ``flag`` itself.  Optional
+    protocols that add a keyword to ``forward`` (``can_defer_last``) are declared beside the ``forward`` that
+    implements them: a subclass that overrides ``forward`` and says nothing is not handed the keyword."""
+    for cls in type(part).__mro__:
+        if "forward" in cls.__dict__:
+            return bool(cls.__dict__.get(flag, False))
+    return False
 
 
 class Block(Part):

@@ -8,18 +8,11 @@ model's final norm).
 """
 from __future__ import annotations
 
-import inspect
 from typing import List, Optional
 
 from ..cache.paged import CacheView
-from .base import BLOCKS, Block, FeedForward, Mixer, Norm, Part, ResidualStream, StepContext, branch_tensor
-
-
-def _accepts(fn, name: str) -> bool:
-    try:
-        return name in inspect.signature(fn).parameters
-    except (TypeError, ValueError):
-        return False
+from .base import (BLOCKS, Block, FeedForward, Mixer, Norm, Part, ResidualStream, StepContext, branch_tensor,
+                   forward_declares)
 
 
 @BLOCKS.register("pre_norm")
@@ -31,10 +24,11 @@ class PreNormBlock(Block):
         self.ff_norm = ff_norm
         self.feed_forward = feed_forward
         self.residual_scale = float(residual_scale)
-        # a part that can leave its last product to the norm after it is asked to (a subclass whose forward
-        # does not know the argument is not)
-        self._mixer_defers = mixer.can_defer_last and _accepts(mixer.forward, "defer_last")
-        self._ff_defers = feed_forward.can_defer_last and _accepts(feed_forward.forward, "defer_last")
+        # a part whose forward can leave its last product to the norm after it is asked to; the class that
+        # defines ``forward`` says so itself, so a subclass with a forward of its own is asked only if it
+        # declares the same
+        self._mixer_defers = forward_declares(mixer, "can_defer_last")
+        self._ff_defers = forward_declares(feed_forward, "can_defer_last")
 
     def parts(self) -> List[Part]:
         return [self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward]

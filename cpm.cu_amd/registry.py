@@ -1,24 +1,54 @@
 """One registry from an architecture's name (config.json ``architectures[0]``) to its model.
 
 An architecture brings: its typed configuration class, a function that builds the
-model (parts and schedule) from a configuration, and the checkpoint's
-peculiarities (fused tensors to split, tensors to ignore).  The reference
-chooses the model class from the same config key (cpmcu/common/utils.py:33-64).
+model (parts and schedule) from a configuration, the options that function
+understands, and the checkpoint's peculiarities (fused tensors to split, tensors
+to ignore, options that the checkpoint decides).  The reference chooses the model
+class from the same config key (cpmcu/common/utils.py:33-64).  Nothing outside
+an architecture's own file names its options or its configuration's fields.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
-from typing import Callable, Dict, List, Optional
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, Iterable, List, Mapping, Optional
 
 
 @dataclass
 class Architecture:
     name: str
     config_class: type
-    build: Callable                                  # (config, tied=None) -> model
+    build: Callable                                  # (config, **options) -> model
+    options: Dict[str, Any] = field(default_factory=dict)   # the options ``build`` understands, with their defaults
     split_fused: Optional[Callable] = None           # (config, name, tensor) -> [(name, tensor)] or None
     ignore_tensor: Optional[Callable] = None         # (config, name) -> bool
-    tie_key: Optional[str] = None                    # tensor whose absence means tied embeddings when config is silent
+    # (config, names of the checkpoint's tensors) -> options that the checkpoint decides (e.g. tied embeddings
+    # when the head's tensor is absent); explicit options win over them
+    checkpoint_options: Optional[Callable] = None
+    # (config, flags) -> (config, options): the front end's flags (the reference's command-line and ``LLM``
+    # argument names) as this architecture understands them; flags it does not know must be refused
+    apply_flags: Optional[Callable] = None
+
+    def build_model(self, config, options: Optional[Mapping[str, Any]] = None,
+                    checkpoint_names: Optional[Iterable[str]] = None):
+        """The model for ``config``: defaults, then what the checkpoint decides, then the given options."""
+        opts = dict(self.options)
+        if checkpoint_names is not None and self.checkpoint_options is not None:
+            opts.update(self.checkpoint_options(config, set(checkpoint_names)))
+        for k, v in (options or {}).items():
+            if k not in self.options:
+                raise ValueError(f"architecture '{self.name}' has no option '{k}' (it has: {sorted(self.options) or 'none'})")
+            opts[k] = v
+        return self.build(config, **opts)
+
+    def with_flags(self, config, flags: Optional[Mapping[str, Any]]):
+        """(config, options) after the front end's flags; flags that are None or absent change nothing."""
+        given = {k: v for k, v in (flags or {}).items() if v is not None}
+        if self.apply_flags is None:
+            switched_on = sorted(k for k, v in given.items() if v is not False)
+            if switched_on:
+                raise ValueError(f"architecture '{self.name}' takes no flags, got {switched_on}")
+            return config, {}
+        return self.apply_flags(config, given) if given else (config, {})
 
 
 _ARCHITECTURES: Dict[str, Architecture] = {}

@@ -1,7 +1,7 @@
 """Plain, slow MiniCPM4 (MiniCPMForCausalLM) forward pass: the oracle of the tests.
 
 Whole sequences, no cache, one function per part, written from the formulas of
-OpenBMB/CPM.cu (cited per function as path:line below /root/reference) and, where
+OpenBMB/CPM.cu (cited per function as path:line of that repository) and, where
 that engine holds one sequence or leaves a choice open, from the engine's own
 contract (block-sparse attention as a pure function of the prefix).  It shares
 no code with the product package: it only needs torch on the CPU, a raw

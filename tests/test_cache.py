@@ -108,3 +108,58 @@ def test_random_walk_never_loses_anything():
         c.release(s)
     c.check()
     assert all(len(g.free_pages) == g.n_pages for g in c.groups) and len(c.free_slots) == 6
+
+
+def test_a_windowed_sequence_may_outgrow_the_pool():
+    """A group that keeps a window holds only its window's pages: a sequence longer than the whole pool fits,
+    and its page table has an entry for every page number it reaches."""
+    c = make([WIN], max_tokens=64, max_slots=2, max_seq_len=400, page=16)        # 4 pages in all
+    s = c.acquire()
+    g = c.groups[0]
+    assert g.table.shape[1] == 25                                               # ceil(400 / 16)
+    c.extend(s, 30)
+    for _ in range(370):
+        assert c.room_for([(s, 1)]) is None
+        c.extend(s, 1)
+        assert g.held(s) <= 3
+        c.check()
+    assert c.length(s) == 400 and g.pages[s][-1] >= 0 and g.pages[s][-3] == -1
+    c.sync()
+    assert int(g.table[s, 24]) == g.pages[s][24]
+    c.release(s)
+    c.check()
+
+
+def test_room_is_asked_of_every_group_and_counts_what_a_window_gives_back():
+    c = make([FULL, WIN], max_tokens=64, max_slots=2, max_seq_len=400, page=16)
+    a, b = c.acquire(), c.acquire()
+    c.extend(a, 40)                                   # 3 of 4 pages in both groups
+    assert c.room_for([(b, 16)]) is None
+    msg = c.room_for([(b, 17)])                       # 2 pages: neither group has them
+    assert msg is not None and "cache is full" in msg
+    assert c.room_for([(a, 24)]) is None              # a's 4th page
+    msg = c.room_for([(a, 25)])                       # a 5th page: the full-history group cannot, the window could
+    assert msg is not None and "group 0" in msg
+    assert c.pages_to_hold(400, 1) == [25, 3] and c.pages_to_hold(400, 64) == [25, 7]
+    assert c.pages_to_hold(20, 64) == [2, 2] and c.capacity() == [4, 4]
+    with pytest.raises(CacheError):
+        c.extend(a, 25)
+    assert c.length(a) == 40
+    c.check()
+
+
+def test_truncate_gives_the_tail_back():
+    c = make([FULL, CK], max_tokens=128, max_slots=2, max_seq_len=128, page=16)
+    s = c.acquire()
+    c.extend(s, 20)
+    free = [len(g.free_pages) for g in c.groups]
+    c.extend(s, 50)
+    c.truncate(s, 20)
+    assert c.length(s) == 20 and [len(g.free_pages) for g in c.groups] == free
+    c.check()
+    assert c.extend(s, 3) == 20
+    with pytest.raises(CacheError):
+        c.truncate(s, 24)
+    c.truncate(s, 0)
+    assert all(len(g.free_pages) == g.n_pages for g in c.groups)
+    c.check()

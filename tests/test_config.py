@@ -100,3 +100,77 @@ def test_model_is_built_from_the_configuration_layer_by_layer():
     # sparse attention can be switched off without touching the configuration
     d = get_architecture("MiniCPMForCausalLM").build(MiniCPMConfig.from_dict(tiny.tiny_b()), sparse=False)
     assert all(type(l.mixer) is GQAAttention for l in d.layers)
+
+
+def test_options_are_declared_by_the_architecture():
+    arch = get_architecture("MiniCPMForCausalLM")
+    cfg = MiniCPMConfig.from_dict(tiny.tiny_b())
+    from cpmcu_amd.parts import GQAAttention
+    assert set(arch.options) == {"tied", "sparse"}
+    dense = arch.build_model(cfg, {"sparse": False})
+    assert all(type(l.mixer) is GQAAttention for l in dense.layers)
+    with pytest.raises(ValueError, match="no option 'window'.*sparse"):
+        arch.build_model(cfg, {"window": 3})
+    # what the checkpoint decides (no head tensor: tied) yields to an explicit option
+    raw = tiny.tiny_b()
+    del raw["tie_word_embeddings"]
+    cfg2 = MiniCPMConfig.from_dict(raw)
+    assert arch.build_model(cfg2, None, ["model.embed_tokens.weight"]).head.tied_to is not None
+    assert arch.build_model(cfg2, None, ["model.embed_tokens.weight", "lm_head.weight"]).head.tied_to is None
+    assert arch.build_model(cfg2, {"tied": False}, ["model.embed_tokens.weight"]).head.tied_to is None
+
+
+def test_head_sizes_the_kernels_do_not_take_are_refused_when_the_model_is_built():
+    raw = tiny.tiny_a()
+    raw["head_dim"] = 24
+    raw["rope_scaling"]["short_factor"] = raw["rope_scaling"]["short_factor"][:4] * 3
+    raw["rope_scaling"]["long_factor"] = raw["rope_scaling"]["long_factor"][:4] * 3
+    cfg = MiniCPMConfig.from_dict(raw)              # a valid configuration of the architecture
+    with pytest.raises(ValueError, match="head_dim 24.*steps of 16"):
+        get_architecture("MiniCPMForCausalLM").build_model(cfg)
+
+
+def test_front_end_flags_go_through_the_architecture():
+    arch = get_architecture("MiniCPMForCausalLM")
+    cfg = MiniCPMConfig.from_dict(tiny.tiny_b())
+    same, opts = arch.with_flags(cfg, {"apply_sparse": False, "sparse_topk_k": 9})
+    assert same == cfg and opts == {"sparse": False}
+    new, opts = arch.with_flags(cfg, {"apply_sparse": True, "sparse_topk_k": 9, "block_window_size": 3, "sink_window_size": 2,
+                                      "sparse_switch": 100})
+    sc = new.sparse_config
+    assert opts == {"sparse": True} and (sc.topk, sc.window_size, sc.init_blocks, sc.dense_len) == (9, 48, 2, 100)
+    with pytest.raises(ValueError, match="use_compress_lse"):
+        arch.with_flags(cfg, {"use_compress_lse": True})
+    with pytest.raises(ValueError, match="no sparse_config"):
+        arch.with_flags(MiniCPMConfig.from_dict(tiny.tiny_a()), {"apply_sparse": True})
+    with pytest.raises(ValueError, match="does not know the flags"):
+        arch.with_flags(cfg, {"draft_model": "x"})
+
+
+def test_minicpm4_yarn_installs_the_built_in_factors_for_head_size_128_only():
+    """--minicpm4-yarn overwrites both factor lists with the reference's 64 numbers
+    (cpmcu/common/utils.py:181-207): only a head size of 128 has 64 rotation pairs."""
+    from cpmcu_amd.config.minicpm4_yarn import MINICPM4_YARN_FACTORS
+    arch = get_architecture("MiniCPMForCausalLM")
+    assert len(MINICPM4_YARN_FACTORS) == 64 and MINICPM4_YARN_FACTORS[0] < 1.0 < MINICPM4_YARN_FACTORS[-1]
+    with pytest.raises(ValueError, match="head_dim 128"):
+        arch.with_flags(MiniCPMConfig.from_dict(tiny.tiny_b()), {"minicpm4_yarn": True})
+    raw = tiny.tiny_b()
+    raw.update(hidden_size=384, num_attention_heads=3, head_dim=128)
+    raw["rope_scaling"].update(short_factor=[1.5] * 64, long_factor=[2.5] * 64)
+    cfg = MiniCPMConfig.from_dict(raw)
+    new, opts = arch.with_flags(cfg, {"minicpm4_yarn": True})
+    assert opts == {}
+    rs = new.rope_scaling
+    assert rs.short_factor == tuple(MINICPM4_YARN_FACTORS) == rs.long_factor
+    assert rs.original_max_position_embeddings == cfg.rope_scaling.original_max_position_embeddings
+    # and they reach the position encoding of every layer, whichever list the engine's length selects
+    model = arch.build_model(new)
+    for layer in model.layers:
+        for max_len in (64, 4096):
+            assert tuple(layer.mixer.position.factors(max_len)) == tuple(MINICPM4_YARN_FACTORS)
+
+
+def test_neutral_properties_of_a_configuration():
+    cfg = MiniCPMConfig.from_dict(tiny.tiny_b())
+    assert cfg.vocabulary_size == 1000 and cfg.longest_sequence == 512 and tuple(cfg.stop_token_ids) == (1, 7)

@@ -8,8 +8,15 @@ from cpmcu_amd.engine.generate import generate, plan_batches
 class FakeCache:
     page_size = 16
 
-    def __init__(self, slots):
+    def __init__(self, slots, max_tokens):
         self.max_slots = slots
+        self.max_tokens = max_tokens
+
+    def pages_to_hold(self, length, step):
+        return [-(-length // self.page_size)]
+
+    def capacity(self):
+        return [self.max_tokens // self.page_size]
 
 
 class FakeEngine:
@@ -20,7 +27,7 @@ class FakeEngine:
             pass
         self.options = O()
         self.options.max_tokens = max_tokens
-        self.cache = FakeCache(slots)
+        self.cache = FakeCache(slots, max_tokens)
         self.max_seq_len = max_seq_len
         self.device = torch.device("cpu")
         self.vocab = vocab
@@ -94,17 +101,33 @@ def test_more_requests_than_slots_run_as_batches_one_after_another():
     assert s.last == ([4], [1])                                                       # request id and its step
 
 
+def full_history(page):
+    return lambda length: [-(-length // page)]
+
+
 def test_plan_batches_respects_slots_cache_and_order():
-    assert plan_batches([5, 11, 17], 8, 8, 4096, 64, 256) == [[0, 1, 2]]
-    assert plan_batches([5, 11, 17, 3], 8, 2, 4096, 64, 256) == [[0, 1], [2, 3]]
+    assert plan_batches([5, 11, 17], 8, 8, full_history(64), [64], 256) == [[0, 1, 2]]
+    assert plan_batches([5, 11, 17, 3], 8, 2, full_history(64), [64], 256) == [[0, 1], [2, 3]]
     # 100+29 tokens = 3 pages of 64 each; a cache of 320 tokens (5 pages) holds one such request at a time
-    assert plan_batches([100, 100, 10], 30, 8, 320, 64, 256) == [[0], [1, 2]]
+    assert plan_batches([100, 100, 10], 30, 8, full_history(64), [5], 256) == [[0], [1, 2]]
     with pytest.raises(ValueError, match="longest sequence"):
-        plan_batches([250], 10, 8, 4096, 64, 256)
+        plan_batches([250], 10, 8, full_history(64), [64], 256)
     with pytest.raises(ValueError, match="do not fit the cache"):
-        plan_batches([200], 10, 8, 128, 64, 256)
+        plan_batches([200], 10, 8, full_history(64), [2], 256)
     with pytest.raises(ValueError, match="empty"):
-        plan_batches([3, 0], 10, 8, 4096, 64, 256)
+        plan_batches([3, 0], 10, 8, full_history(64), [64], 256)
+
+
+def test_plan_batches_asks_every_cache_group():
+    """Two groups: one keeps every token, one a window of at most 2 pages a sequence; the fuller group decides."""
+    def two_groups(length):
+        return [-(-length // 64), min(-(-length // 64), 2)]
+    # 5 pages each in the first group: a pool of 10 holds two requests, the windowed pool of 4 as well
+    assert plan_batches([300, 300, 300], 10, 8, two_groups, [10, 4], 1000) == [[0, 1], [2]]
+    # with a windowed pool of 3 only one request fits at a time although the first group has room for two
+    assert plan_batches([300, 300, 300], 10, 8, two_groups, [10, 3], 1000) == [[0], [1], [2]]
+    # a sequence longer than the windowed group's whole pool is fine as long as its window fits
+    assert plan_batches([900], 10, 8, two_groups, [20, 2], 1000) == [[0]]
 
 
 def test_a_failing_step_gives_the_slots_back():

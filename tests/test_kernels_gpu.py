@@ -795,7 +795,7 @@ def test_block_selection_equals_the_plain_selection(dtype, nh, nkv, hd, ks, st, 
     ck_ref = plain.compressed_keys(kseq[0], ks, st).to(dtype).double()
     # the matrix-core kernel, its forms for steps of few tokens (two kernels, or three when the last does not
     # normalise the scores itself), and the plain twin
-    scratch = torch.full((ops.sparse_select_scratch(n, nh, nkv, max(positions), ks, st),), float("nan"), device=DEV)
+    scratch = torch.full((ops.sparse_select_scratch(dtype, n, nh, nkv, hd, max(positions), ks, st, bs),), float("nan"), device=DEV)
     for force_plain, scr in (((False, None), (False, scratch), (2, scratch), (True, None)) if dtype == torch.bfloat16
                              else ((True, None),)):
         sel_blocks.fill_(-7)
@@ -830,7 +830,7 @@ def test_block_selection_ties_and_forced_blocks():
         for init, topk, want in ((0, 3, [0, 1, 2, 11, 12]), (2, 2, [0, 1, 11, 12]), (1, 20, list(range(13)))):
             sb = torch.zeros(1, 1, topk + 2, dtype=torch.int32, device=DEV)
             cnt = torch.zeros(1, 1, dtype=torch.int32, device=DEV)
-            for scr in ((None, torch.zeros(ops.sparse_select_scratch(1, nh, nkv, 200, ks, st), device=DEV))
+            for scr in ((None, torch.zeros(ops.sparse_select_scratch(dtype, 1, nh, nkv, hd, 200, ks, st, bs), device=DEV))
                         if dtype == torch.bfloat16 else (None,)):
                 sb.zero_()
                 cnt.zero_()

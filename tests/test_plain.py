@@ -114,6 +114,67 @@ def test_longrope_factor_choice_and_magnitude():
     assert torch.allclose((y[..., :16] ** 2 + y[..., 16:] ** 2), m * m * (x[..., :16] ** 2 + x[..., 16:] ** 2))
 
 
+def test_longrope_factor_stretches_the_positions_of_its_pair():
+    """What the factors are for, without restating the formula: a factor f on pair c makes that pair turn f times
+    slower, so the rotation at position f * k equals the factor-free rotation (pinned to the textbook form
+    above) at position k.  A factor that multiplied the frequency, or one applied to the wrong pair, fails."""
+    raw = tiny.tiny_b()
+    hd = 32
+    fac = [1.0, 2.0, 4.0, 8.0] * 4
+    raw["rope_scaling"] = dict(raw["rope_scaling"], long_factor=fac, short_factor=[3.0] * 16)
+    raw["rope_attention_scaling"] = False
+    inv_long, m = P.rope_inv_freq(raw)                      # max_position 512 > original 128: the long list
+    plain_cfg = {k: v for k, v in raw.items() if k != "rope_scaling"}
+    inv_plain, m_plain = P.rope_inv_freq(plain_cfg)
+    assert m == 1.0 and m_plain == 1.0
+    x = rnd(1, 2, hd)
+    k = 5
+    for f in (1.0, 2.0, 4.0, 8.0):
+        stretched = P.apply_rope(x, torch.tensor([int(f) * k]), inv_long, m)
+        unstretched = P.apply_rope(x, torch.tensor([k]), inv_plain, 1.0)
+        pairs = [c for c in range(16) if fac[c] == f]
+        for c in pairs:
+            assert torch.allclose(stretched[..., c], unstretched[..., c], atol=1e-12)
+            assert torch.allclose(stretched[..., c + 16], unstretched[..., c + 16], atol=1e-12)
+        others = [c for c in range(16) if fac[c] != f]
+        assert not torch.allclose(stretched[..., others], unstretched[..., others], atol=1e-3)
+    # the short list below the original length: every pair three times slower
+    inv_short, _ = P.rope_inv_freq(raw, max_seq_len=128)
+    assert torch.allclose(P.apply_rope(x, torch.tensor([15]), inv_short, 1.0), P.apply_rope(x, torch.tensor([5]), inv_plain, 1.0),
+                          atol=1e-12)
+
+
+def test_longrope_magnitude_is_a_number_known_in_closed_form():
+    """Tiny B stretches 128 positions to 512: ln 4 / ln 128 = 2/7 exactly, so the magnitude is sqrt(9/7).
+    A natural logarithm of the wrong quantity (the factor lists, max/1, original/max) does not give this."""
+    assert P.rope_inv_freq(tiny.tiny_b())[1] == pytest.approx(1.1338934190276817, abs=1e-15)
+    raw = tiny.tiny_b()
+    raw["max_position_embeddings"] = 128 * 128          # stretched by the original length itself: sqrt(2)
+    assert P.rope_inv_freq(raw)[1] == pytest.approx(1.4142135623730951, abs=1e-15)
+
+
+def test_the_engines_position_part_equals_the_plain_frequencies():
+    """parts/rope.py bound for engines of different lengths against the plain implementation (which the tests
+    above pin): same factor list at 128 / 129 / 512 positions, same magnitude, float32 roundings only."""
+    from cpmcu_amd.config import MiniCPMConfig
+    from cpmcu_amd.models.minicpm import layer_specs
+    from cpmcu_amd.parts import POSITION_ENCODINGS
+    from cpmcu_amd.parts.base import Runtime, Workspace
+    for raw in (tiny.tiny_a(), tiny.tiny_b()):
+        cfg = MiniCPMConfig.from_dict(raw)
+        for max_seq_len in (128, 129, 256, 257, 512):
+            part = layer_specs(cfg)[0]["position"].build(POSITION_ENCODINGS)
+            part.bind({}, Runtime(torch.device("cpu"), torch.float32, Workspace("cpu"), max_seq_len))
+            inv, m = part.rotary_params()
+            want, want_m = P.rope_inv_freq(raw, max_seq_len)
+            assert inv.dtype == torch.float32 and torch.equal(inv, want.to(torch.float32))
+            assert m == pytest.approx(want_m, abs=1e-15)
+    raw = tiny.tiny_b()
+    raw["rope_attention_scaling"] = False               # what the reference does (cpmcu/llm.py:190-192)
+    part = layer_specs(MiniCPMConfig.from_dict(raw))[0]["position"].build(POSITION_ENCODINGS)
+    assert part.rotary_params()[1] == 1.0
+
+
 # ---------------------------------------------------------------------------- attention
 def test_dense_attention_is_the_library_routine():
     T, nh, nkv, hd = 13, 6, 2, 8

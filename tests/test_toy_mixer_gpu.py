@@ -57,6 +57,10 @@ def _define():
         rms_norm_eps: float = 1e-5
         max_position_embeddings: int = 128
 
+        @property
+        def longest_sequence(self):
+            return self.max_position_embeddings
+
         @classmethod
         def from_dict(cls, raw: Dict[str, Any]):
             return cls(raw["architectures"][0], field_from(raw, "vocab_size", int), field_from(raw, "hidden_size", int),
@@ -72,7 +76,7 @@ def _define():
 
     MIXERS.register("toy_decay", DecayMixer)
 
-    def build(cfg: ToyConfig, tied=None, sparse=True):
+    def build(cfg: ToyConfig):
         layers = []
         for i in range(cfg.num_hidden_layers):
             p = f"layers.{i}."

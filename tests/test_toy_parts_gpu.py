@@ -95,6 +95,10 @@ def _define():
         def num_hidden_layers(self):
             return len(self.layer_kinds)
 
+        @property
+        def longest_sequence(self):
+            return self.max_position_embeddings
+
         @classmethod
         def from_dict(cls, raw: Dict[str, Any]):
             return cls(raw["architectures"][0], field_from(raw, "vocab_size", int), field_from(raw, "hidden_size", int),
@@ -114,7 +118,7 @@ def _define():
     FEED_FORWARDS.register("toy_top1_experts", Top1Experts)
     POSITION_ENCODINGS.register("toy_interleaved_rotary", InterleavedRotary)
 
-    def build(cfg: ToyConfig, tied=None, sparse=True):
+    def build(cfg: ToyConfig):
         layers = []
         for i, kind in enumerate(cfg.layer_kinds):
             p = f"layers.{i}."

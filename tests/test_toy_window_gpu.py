@@ -63,6 +63,10 @@ def _define():
         rms_norm_eps: float = 1e-5
         max_position_embeddings: int = 512
 
+        @property
+        def longest_sequence(self):
+            return self.max_position_embeddings
+
         @classmethod
         def from_dict(cls, raw: Dict[str, Any]):
             return cls(raw["architectures"][0], *(field_from(raw, k, t) for k, t in (
@@ -79,7 +83,7 @@ def _define():
 
     MIXERS.register("toy_window_attention", WindowAttention)
 
-    def build(cfg: ToyConfig, tied=None, sparse=True):
+    def build(cfg: ToyConfig):
         layers = []
         for i, kind in enumerate(("gqa_attention", "toy_window_attention")):
             p = f"layers.{i}."

@@ -136,3 +136,25 @@ def test_tying_follows_the_checkpoint_when_the_config_is_silent(tmp_path):
     assert cfg.tie_word_embeddings is None
     assert minicpm.build(cfg, tied=True).head.tied_to is not None
     assert minicpm.build(cfg, tied=False).head.tied_to is None
+
+
+def test_a_part_brings_its_own_init_rule():
+    """Another kind of tensor (here: decay rates in (0, 1)) registers its rule; the writer needs no change."""
+    from cpmcu_amd.parts.base import WeightSpec
+    from cpmcu_amd.weights import INIT_RULES, draw, register_init_rule
+
+    def decay(spec, g, device, dtype, std, norm_std):
+        return torch.rand(spec.shape, generator=g, device=device).to(dtype)
+
+    register_init_rule("test_decay", decay)
+    try:
+        spec = WeightSpec("layer.decay", (7,), "test_decay", "float32")
+        a, b = draw(spec, 3), draw(spec, 3)
+        assert torch.equal(a, b) and a.dtype == torch.float32 and bool(((a >= 0) & (a < 1)).all())
+        assert not torch.equal(a, draw(spec, 4))
+        with pytest.raises(ValueError, match="already registered"):
+            register_init_rule("test_decay", lambda *a: None)
+    finally:
+        INIT_RULES.pop("test_decay", None)
+    with pytest.raises(ValueError, match="unknown init rule 'test_decay'.*matrix"):
+        draw(WeightSpec("layer.decay", (7,), "test_decay", "float32"), 3)
