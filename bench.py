@@ -2,10 +2,14 @@
 """Benchmark: decode tokens/s of a MiniCPM4-8B-shaped model with random weights on one MI355X.
 
 python bench.py --gpus 1 --steps K --warmup W   prints ONE JSON line.  A step is one decode step
-of the whole batch (default batch 8 at context 4,096, the sizes of BASELINE.json configs[2]).
-The same line carries the prefill of 2,048 tokens, the decode step's memory roofline and
-decode at batch 1 and 64.  Weights are random (N(0, 0.02)), token ids uniform: nothing is
-downloaded.  The engine runs on one GPU only: for --gpus > 1 it says so and exits with 2.
+of the whole batch, the next token chosen by argmax included (default: batch 8 at context 4,096,
+all 32 layers of the 8B shape).  The same line carries the prefill of 2,048 tokens, the decode
+step's memory roofline against the published peak and against what a plain read kernel and a
+large library product reach on this GPU, and decode at batch 1 and 64.  Before anything is timed,
+one decode step from the captured graph is compared with the same step run eagerly.  Weights are
+random (N(0, 0.02)), token ids uniform, the cache of the decode runs is filled with noise (what
+filled it is not timed): nothing is downloaded.  The engine runs on one GPU only: for --gpus > 1
+it says so and exits with 2.
 """
 import argparse
 import json
@@ -37,7 +41,7 @@ def config_8b(layers=None):
 
 
 def config_small():
-    """BASELINE.json configs[3]: the MiniCPM4-0.5B shape (tied embeddings)."""
+    """The MiniCPM4-0.5B shape (tied embeddings)."""
     import torch
     g = torch.Generator().manual_seed(4321)
     fac = lambda: [float(x) for x in (1.0 + 3.0 * torch.rand(32, generator=g, dtype=torch.float64))]
@@ -92,9 +96,9 @@ def main():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--hip-graph", type=int, default=1)
     ap.add_argument("--scenario", default="headline", choices=["headline", "small_batch64", "sparse32k"],
-                    help="headline: BASELINE.json configs[2] (the default, the contract's line); small_batch64: "
-                         "configs[3], 64 unequal prompts through the generation loop; sparse32k: configs[4], "
-                         "InfLLM-v2 at 32k context")
+                    help="headline: the 8B shape at batch 8, context 4,096 (the default, the contract's line); "
+                         "small_batch64: the 0.5B shape, 64 unequal prompts through the generation loop; sparse32k: "
+                         "the 8B shape with InfLLM-v2 at 32k context")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported (no multi-GPU path exists)")
@@ -140,26 +144,90 @@ def main():
                     t.normal_(0.0, 0.5)
         return slots
 
+    from cpmcu_amd import ops
+    next_tok = torch.zeros(64, dtype=torch.int32, device=dev)
+
     def decode_run(batch, context, steps, warmup):
+        """Seconds for `steps` decode steps of `batch` sequences at `context`: each step runs the model on one
+        token a sequence and chooses the next by argmax (on the device; the tokens fed are fixed beforehand so
+        that every run does the same work)."""
         slots = fill_context(batch, context)
         toks = [rand_ids(batch) for _ in range(steps + warmup)]
         for i in range(warmup):
-            eng.step([StepEntry(s, [toks[i][j]], [0]) for j, s in enumerate(slots)])
+            ops.argmax(eng.step([StepEntry(s, [toks[i][j]], [0]) for j, s in enumerate(slots)]), next_tok[:batch])
         torch.cuda.synchronize()
         t = time.perf_counter()
         for i in range(warmup, warmup + steps):
-            eng.step([StepEntry(s, [toks[i][j]], [0]) for j, s in enumerate(slots)])
+            ops.argmax(eng.step([StepEntry(s, [toks[i][j]], [0]) for j, s in enumerate(slots)]), next_tok[:batch])
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
         for s in slots:
             eng.release(s)
         return dt
 
+    def graph_check(batch, context):
+        """One decode step replayed from the captured graph against the same step run eagerly (the cache is
+        wound back one token in between): finite and equal up to the order of float sums."""
+        if not args.hip_graph:
+            return None
+        slots = fill_context(batch, context)
+        ids = rand_ids(batch)
+        entries = [StepEntry(s, [ids[j]], [0]) for j, s in enumerate(slots)]
+        eng.options.hip_graph = False
+        eager = eng.step(entries).clone()
+        eng.options.hip_graph = True
+        outs = []
+        for _ in range(2):                   # the first captures, the second replays
+            for s in slots:
+                eng.cache.truncate(s, context - 1)
+            outs.append(eng.step(entries).clone())
+        for s in slots:
+            eng.release(s)
+        if not bool(torch.isfinite(eager).all()):
+            raise SystemExit("bench.py: the decode step's logits are not finite")
+        scale = float(eager.abs().max())
+        err = max(float((o - eager).abs().max()) for o in outs)
+        if err > 1e-3 * scale:
+            raise SystemExit(f"bench.py: a decode step from the captured graph differs from the eager step by {err:.3g} "
+                             f"(logits up to {scale:.3g})")
+        return err / scale
+
+    def calibrate():
+        """What this GPU gives a kernel that only reads (GB/s) and the library's product of two large bf16
+        matrices (FLOP/s): the ceilings that memory-bound and matrix-bound work can be held against besides
+        the published peaks."""
+        buf = torch.empty(1 << 30, dtype=torch.int32, device=dev).random_()     # 4 GiB: far beyond the caches
+        out = torch.zeros(8192, dtype=torch.int32, device=dev)
+        best = 0.0
+        for _ in range(4):
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            ops.read_bandwidth(buf, out)
+            torch.cuda.synchronize()
+            best = max(best, buf.numel() * 4 / (time.perf_counter() - t) / 1e9)
+        del buf
+        a = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
+        b = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
+        c = torch.empty_like(a)
+        flops = 0.0
+        for _ in range(4):
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            for _ in range(4):
+                torch.mm(a, b.t(), out=c)
+            torch.cuda.synchronize()
+            flops = max(flops, 4 * 2 * 8192 ** 3 / (time.perf_counter() - t))
+        return best, flops
+
+    def step_bytes(batch, context, steps):
+        return weight_bytes_per_step(cfg, esize) + batch * (context + steps // 2) * kv_bytes_per_token(cfg, esize)
+
+    read_gbs, mm_flops = calibrate()
+    graph_err = graph_check(args.batch, args.context)
     dt = decode_run(args.batch, args.context, args.steps, args.warmup)
     ms_step = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
-    step_bytes = weight_bytes_per_step(cfg, esize) + args.batch * (args.context + args.steps // 2) * kv_bytes_per_token(cfg, esize)
-    achieved = step_bytes / (ms_step * 1e-3) / 1e9
+    achieved = step_bytes(args.batch, args.context, args.steps) / (ms_step * 1e-3) / 1e9
     rec = {
         "metric": f"MiniCPM4-8B decode tok/s @ batch {args.batch}, context {args.context} "
                   f"({'bf16' if args.dtype == 'bfloat16' else 'fp32'}, random weights)",
@@ -171,10 +239,14 @@ def main():
                    "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
                    "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size, "global_batch": args.batch,
                    "seq_len": args.context, "prefill_tokens": args.prefill_tokens, "parallelism": "1gpu",
-                   "page_size": 64, "hip_graph": bool(args.hip_graph)},
+                   "page_size": 64, "hip_graph": bool(args.hip_graph), "sampling": "argmax inside the timed step",
+                   "cache_fill": "noise (not timed)"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "read_kernel": round(read_gbs, 1),
+                     "frac_of_read_kernel": round(achieved / read_gbs, 4)},
     }
+    if graph_err is not None:
+        rec["graph_check"] = {"max_rel_diff_to_eager": float(f"{graph_err:.3g}")}
     if not args.no_prefill:
         n = args.prefill_tokens
         times = []
@@ -190,19 +262,24 @@ def main():
         pt = min(times[1:])
         peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
         rec["prefill"] = {"value": round(n / pt, 1), "tokens": n, "ms": round(pt * 1e3, 3),
-                          "frac": round(prefill_flops(cfg, n) / pt / peak, 4)}
+                          "frac": round(prefill_flops(cfg, n) / pt / peak, 4),
+                          "library_product": round(mm_flops / 1e12, 1), "library_product_unit": "TFLOP/s",
+                          "frac_of_library_product": round(prefill_flops(cfg, n) / pt / mm_flops, 4)}
     if not args.no_points:
         pts = {}
         for b in (1, 64):
             st = max(args.steps // 2, 8)
             d = decode_run(b, args.context, st, max(args.warmup // 2, 3))
+            gbs = step_bytes(b, args.context, st) / (d / st) / 1e9
             pts[f"decode_b{b}"] = round(b * st / d, 2)
+            pts[f"decode_b{b}_ms"] = round(d / st * 1e3, 4)
+            pts[f"decode_b{b}_frac"] = round(gbs / HBM_PEAK_GBS, 4)
         rec["points"] = pts
     print(json.dumps(rec), flush=True)
 
 
 def other_scenarios(args, dev):
-    """The two further workloads of BASELINE.json, each one JSON line of the same shape."""
+    """The two further workloads, each one JSON line of the same shape."""
     import torch
     from cpmcu_amd import Engine, EngineOptions, StepEntry
     from cpmcu_amd.config import MiniCPMConfig

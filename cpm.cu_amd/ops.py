@@ -445,6 +445,15 @@ def sample(logits: torch.Tensor, temperature: float, seed: int, request_ids: tor
                                        _p(u_out), _stream()))
 
 
+def read_bandwidth(src: torch.Tensor, out: torch.Tensor):
+    """Read all of ``src`` once with a kernel that does nothing else (out: int32 scratch of a few thousand
+    words): what measurement compares the decode products' streaming with."""
+    _need(src, "read source")
+    _need(out, "read scratch", torch.int32, (None,))
+    _check(_fn("core", "cpmcu_read_bandwidth")(_p(src), c_long(src.numel() * src.element_size()), _p(out),
+                                               c_int(out.shape[0]), _stream()))
+
+
 class TiledWeight:
     """A weight [N, K] re-laid for the skinny product: [strip of 16 rows][K-block of 128][MFMA i][lane][8],
     lane = 16*g + r holding row 16*strip + r, columns 128*block + 32*i + 8*g .. +8; zero padded."""
