@@ -473,21 +473,49 @@ class TiledWeight:
 
 
 
-def qkv_rope_weight(w: torch.Tensor, nh: int, nkv: int, hd: int) -> TiledWeight:
-    """The stacked [q heads; k heads; v heads] x hidden weight for qkv_rope: tiled, the rows of every q and k head
-    in the order (8s .. 8s+7, hd/2 + 8s .. hd/2 + 8s+7 for s = 0, 1, ...), so that a strip of 16 rows holds
-    both halves of 8 rotation pairs; v heads keep their order."""
-    _need(w, "qkv weight", torch.bfloat16, ((nh + 2 * nkv) * hd, None))
-    if hd % 16:
-        raise KernelError(f"qkv_rope: head_dim {hd} is no multiple of 16")
-    s = torch.arange(hd // 16).view(-1, 1, 1)
-    order = (8 * s + torch.tensor([0, hd // 2]).view(1, 2, 1) + torch.arange(8).view(1, 1, 8)).reshape(-1)
-    rows = torch.arange((nh + 2 * nkv) * hd).view(nh + 2 * nkv, hd)
-    rows[:nh + nkv] = rows[:nh + nkv, :1] + order
-    return TiledWeight(w[rows.reshape(-1).to(w.device)])
+class QKVRopeWeight:
+    """The stacked [q heads; k heads; v heads] x hidden weight re-laid for qkv_rope:
+    * the rows of every q and k head as rotation pairs side by side (c, c + hd/2, c + 1, c + 1 + hd/2, ...), v
+      heads in their order;
+    * cut into runs of R rows, one a workgroup (R from the kernel library: 16, or a few more where that spreads
+      the workgroups evenly over the CUs);
+    * per run and 128-column block: 16 rows as [MFMA i][lane = 16 g + row][8] (columns 32 i + 8 g ..), then the
+      other R - 16 rows as [i][g][row][8]; rows and columns zero padded."""
+
+    def __init__(self, w: torch.Tensor, nh: int, nkv: int, hd: int, rows_per_workgroup: Optional[int] = None):
+        total = (nh + 2 * nkv) * hd
+        _need(w, "qkv weight", torch.bfloat16, (total, None))
+        if hd % 16:
+            raise KernelError(f"qkv_rope: head_dim {hd} is no multiple of 16")
+        if rows_per_workgroup is None:
+            lib = _build.load("qkv")
+            lib.cpmcu_qkv_rope_rows_per_workgroup.restype = c_int
+            rows_per_workgroup = int(lib.cpmcu_qkv_rope_rows_per_workgroup(c_int(total)))
+        R = int(rows_per_workgroup)
+        if R < 16 or R > 32 or R % 2:
+            raise KernelError(f"qkv_rope: {R} rows a workgroup (an even number from 16 to 32)")
+        K = w.shape[1]
+        c = torch.arange(hd // 2)
+        order = torch.stack([c, c + hd // 2], dim=1).reshape(-1)
+        rows = torch.arange(total).view(nh + 2 * nkv, hd).clone()
+        rows[:nh + nkv] = rows[:nh + nkv, :1] + order
+        n_wg, nkb = -(-total // R), -(-K // 128)
+        padded = torch.zeros((n_wg * R, nkb * 128), dtype=w.dtype, device=w.device)
+        padded[:total, :K] = w[rows.reshape(-1).to(w.device)]
+        blk = padded.view(n_wg, R, nkb, 4, 4, 8)                 # run, row, block, i, g, element
+        first = blk[:, :16].permute(0, 2, 3, 4, 1, 5).reshape(n_wg, nkb, 2048)
+        rest = blk[:, 16:].permute(0, 2, 3, 4, 1, 5).reshape(n_wg, nkb, 128 * (R - 16))
+        self.data = torch.cat([first, rest], dim=2).contiguous()
+        self.N, self.K, self.rows_per_workgroup = total, K, R
 
 
-def qkv_rope(x: torch.Tensor, w: TiledWeight, q_out: torch.Tensor, nh: int, nkv: int, hd: int,
+def qkv_rope_weight(w: torch.Tensor, nh: int, nkv: int, hd: int, rows_per_workgroup: Optional[int] = None
+                    ) -> QKVRopeWeight:
+    """rows_per_workgroup: None lets the kernel library choose (what the engine does)."""
+    return QKVRopeWeight(w, nh, nkv, hd, rows_per_workgroup)
+
+
+def qkv_rope(x: torch.Tensor, w: QKVRopeWeight, q_out: torch.Tensor, nh: int, nkv: int, hd: int,
              positions: torch.Tensor, tok_slot: torch.Tensor, inv_freq: Optional[torch.Tensor], mscale: float,
              kpool: torch.Tensor, vpool: torch.Tensor, page_table: torch.Tensor, page_size: int,
              row_scale: Optional[RowScale] = None, compress: Optional[Tuple[torch.Tensor, int, int]] = None):
@@ -506,8 +534,8 @@ def qkv_rope(x: torch.Tensor, w: TiledWeight, q_out: torch.Tensor, nh: int, nkv:
         if st <= 0 or page_size % st:
             raise KernelError(f"qkv_rope: kernel_stride {st} must divide the cache page of {page_size} tokens")
         _need(ckpool, "qkv compressed key pool", torch.bfloat16, (kpool.shape[0], page_size // st, nkv * hd))
-    if w.N != (nh + 2 * nkv) * hd:
-        raise KernelError(f"qkv_rope: weight of {w.N} rows, {(nh + 2 * nkv) * hd} expected")
+    if not isinstance(w, QKVRopeWeight) or w.N != (nh + 2 * nkv) * hd:
+        raise KernelError(f"qkv_rope: the weight must come from qkv_rope_weight for {(nh + 2 * nkv) * hd} rows")
     _need(q_out, "qkv q_out", torch.bfloat16, (n, nh * hd))
     _need(positions, "qkv positions", torch.int32, (n,))
     _need(tok_slot, "qkv token slots", torch.int32, (n,))
@@ -516,7 +544,8 @@ def qkv_rope(x: torch.Tensor, w: TiledWeight, q_out: torch.Tensor, nh: int, nkv:
     _need(kpool, "qkv key pool", torch.bfloat16, (None, page_size, nkv * hd))
     _need(vpool, "qkv value pool", torch.bfloat16, tuple(kpool.shape))
     _need(page_table, "qkv page table", torch.int32, (None, None))
-    _check(_fn("qkv", "cpmcu_qkv_rope")(_p(x), c_long(x.stride(0)), _p(w.data), c_int(n), c_int(w.K), _p(q_out),
+    _check(_fn("qkv", "cpmcu_qkv_rope")(_p(x), c_long(x.stride(0)), _p(w.data), c_int(w.rows_per_workgroup), c_int(n),
+                                        c_int(w.K), _p(q_out),
                                         c_int(nh), c_int(nkv), c_int(hd), _p(positions), _p(tok_slot), _p(inv_freq),
                                         c_float(mscale), _p(kpool), _p(vpool), _p(page_table),
                                         c_int(page_table.shape[1]), c_int(page_size),

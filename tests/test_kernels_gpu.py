@@ -664,9 +664,12 @@ def test_rotary_and_cache_write(dtype, n, nh, nkv, hd, parts, rotate, write_kv):
                                                   (17, 4, 2, 32, 136, True), (24, 2, 1, 64, 1160, True), (32, 6, 2, 16, 72, True),
                                                   (33, 2, 1, 32, 392, True), (64, 5, 1, 16, 1032, True)])
 @pytest.mark.parametrize("scaled", [False, True])
-def test_fused_projection_rotation_and_cache_write(n, nh, nkv, hd, H, rotate, scaled):
+@pytest.mark.parametrize("R", [None, 18, 26, 32])
+def test_fused_projection_rotation_and_cache_write(n, nh, nkv, hd, H, rotate, scaled, R):
     """q, k, v of a decode step in one kernel: against the float64 product, rotation (pairs c, c + hd/2) and the
-    cache rows read back through the pages' layout; tokens of several slots at scattered positions."""
+    cache rows read back through the pages' layout; tokens of several slots at scattered positions.  R: rows of
+    the weight a workgroup owns (None: the library's choice, 16 at these sizes; more than 16 rows straddle
+    heads, and the last workgroup is not full)."""
     from cpmcu_amd import ops
     page = 64
     w = rnd((nh + 2 * nkv) * hd, H, seed=1, dtype=torch.bfloat16, scale=H ** -0.5)
@@ -680,7 +683,7 @@ def test_fused_projection_rotation_and_cache_write(n, nh, nkv, hd, H, rotate, sc
     kpool = torch.zeros(12, page, nkv * hd, dtype=torch.bfloat16, device=DEV)
     vpool = torch.zeros_like(kpool)
     q_out = torch.empty(n, nh * hd, dtype=torch.bfloat16, device=DEV)
-    wt = ops.qkv_rope_weight(w, nh, nkv, hd)
+    wt = ops.qkv_rope_weight(w, nh, nkv, hd, R)
     # with the row factor of a norm cut by columns (the sums need not belong to x: any positive numbers do)
     row_scale, r = None, 1.0
     if scaled:
@@ -708,7 +711,8 @@ def test_fused_projection_rotation_and_cache_write(n, nh, nkv, hd, H, rotate, sc
 
 
 @pytest.mark.parametrize("n,ks,st", [(16, 8, 4), (5, 32, 16), (32, 12, 4), (1, 32, 16), (50, 8, 4)])
-def test_fused_projection_completes_compressed_keys(n, ks, st):
+@pytest.mark.parametrize("R", [None, 18, 30])
+def test_fused_projection_completes_compressed_keys(n, ks, st, R):
     """The projection kernel of decode steps also writes the compressed keys that its tokens complete: bit for
     bit what compress_keys writes after it, from keys of earlier steps and of this step (two sequences, each
     with consecutive tokens in the step, at different phases of the stride)."""
@@ -723,7 +727,7 @@ def test_fused_projection_completes_compressed_keys(n, ks, st):
     slots = torch.tensor([0] * n0 + [1] * (n - n0), dtype=torch.int32)
     table = torch.randperm(8, generator=g).view(2, 4).to(torch.int32)
     inv_freq = torch.rand(hd // 2, generator=g) * 0.5 + 0.01
-    wt = ops.qkv_rope_weight(w, nh, nkv, hd)
+    wt = ops.qkv_rope_weight(w, nh, nkv, hd, R)
     results = []
     for fused in (True, False):
         kpool = rnd(8, page, nkv * hd, seed=5, dtype=torch.bfloat16)        # the keys of earlier steps
