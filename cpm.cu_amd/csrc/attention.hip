@@ -682,12 +682,12 @@ __global__ __launch_bounds__(NW * 64) void attention_prefill_mfma_kernel(
     // the wavefront's chunks in turn: page number and chunk inside the page advance without a division
     const int cpp = pv.page_size / 32;
     int pg_i = wave / cpp, in_pg = wave % cpp;
+    const int pg_step = NW / cpp, in_step = NW % cpp;      // (without a branch: the loop's code stays one stretch)
     auto next_pchunk = [&]() {
-        in_pg += NW;
-        while (in_pg >= cpp) {
-            in_pg -= cpp;
-            ++pg_i;
-        }
+        in_pg += in_step;
+        const int carry = in_pg >= cpp ? 1 : 0;
+        in_pg -= carry * cpp;
+        pg_i += pg_step + carry;
         return ptab[pg_i] * cpp + in_pg;
     };
     // one buffer each for keys and values: the next chunk's keys are asked for as soon as the last tile's
@@ -709,14 +709,17 @@ __global__ __launch_bounds__(NW * 64) void attention_prefill_mfma_kernel(
                 st[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][ks], qf[r][ks], st[u], 0, 0, 0);
         }
     };
-    auto weights = [&](int r, int key0, const afloatx4_t (&st)[2]) {
+    // MASKED false: the caller knows that every key of the chunk lies before every row of the tile.  The
+    // accumulators' rescale (rare: the maximum moved by more than 8) is the caller's: `moved` and `corr` say
+    // whether and by what.
+    auto weights_of = [&](int r, int key0, const afloatx4_t (&st)[2], bool masked, bool& moved, float& corr) {
         // raw scores; only a chunk that reaches past a row's position needs the causal mask
         float sc[8];
 #pragma unroll
         for (int u = 0; u < 2; ++u)
 #pragma unroll
             for (int i = 0; i < 4; ++i) sc[u * 4 + i] = st[u][i];
-        if (key0 + 31 > tile_first_pos[r]) {
+        if (masked && key0 + 31 > tile_first_pos[r]) {
 #pragma unroll
             for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -730,10 +733,10 @@ __global__ __launch_bounds__(NW * 64) void attention_prefill_mfma_kernel(
         // this chunk sees none of its keys: nothing changes for it
         // the reference follows the maximum only past a move of more than 8 (see attention_mfma_kernel)
         const float m_top = fmaxf(m[r], mx * scale_log2e);
-        const bool moved = __builtin_amdgcn_ballot_w64(m_top > m[r] + 8.0f) != 0;
+        moved = __builtin_amdgcn_ballot_w64(m_top > m[r] + 8.0f) != 0;
         const float m_new = moved ? m_top : m[r];
         const float m_use = m_new == -INFINITY ? 0.f : m_new;
-        const float corr = fast_exp2(m[r] - m_use);
+        corr = fast_exp2(m[r] - m_use);
         float rs = 0.f;
         abf16x8_t pb;
 #pragma unroll
@@ -744,13 +747,20 @@ __global__ __launch_bounds__(NW * 64) void attention_prefill_mfma_kernel(
         }
         rs = rows_sum(rs);
         l[r] = l[r] * corr + rs;
-        if (moved) {
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[r][dt][i] *= corr;
-        }
         m[r] = m_new;
+        return pb;
+    };
+    auto rescale = [&](int r, float corr) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[r][dt][i] *= corr;
+    };
+    auto weights = [&](int r, int key0, const afloatx4_t (&st)[2]) {
+        bool moved;
+        float corr;
+        const abf16x8_t pb = weights_of(r, key0, st, true, moved, corr);
+        if (moved) rescale(r, corr);
         return pb;
     };
     auto values = [&](int r, abf16x8_t pb) {
@@ -758,25 +768,93 @@ __global__ __launch_bounds__(NW * 64) void attention_prefill_mfma_kernel(
         for (int dt = 0; dt < DT; ++dt)
             acc[r][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pb, acc[r][dt], 0, 0, 0);
     };
-    for (int c = wave; c < total_chunks; c += NW) {
-        const int key0 = c * 32;
-        const bool more = c + NW < total_chunks;
-        int pchunkn = 0;
-        if (more) pchunkn = next_pchunk();
-        if constexpr (R == 2) {
-            // The matrix instructions of one tile are issued before the vector work of the other, so that each
-            // runs in the other's shadow (a wavefront issues in order, and a matrix instruction holds only its
-            // own pipe).  A tile that does not see this chunk (the first tile at the last chunk of the second, an
-            // unused tile) is computed all the same: the mask leaves it weights of 0.
+    if constexpr (R == 2) {
+        // The scores of a chunk are issued one chunk ahead of their use: while the vector unit turns the
+        // current chunk's scores into weights, the matrix cores already multiply the next chunk's keys, and the
+        // values' products of one tile run under the other tile's vector work (a wavefront issues in order, and
+        // a matrix instruction holds only its own pipe).  A tile that does not see a chunk (the first tile at
+        // the last chunk of the second, an unused tile) is computed all the same: the mask leaves it weights of 0.
+        if (wave < total_chunks) {
             afloatx4_t s0[2], s1[2];
             scores(0, s0);
             scores(1, s1);
-            if (more) load_k(pchunkn, kf);
-            const abf16x8_t p0 = weights(0, key0, s0);
-            values(0, p0);
-            const abf16x8_t p1 = weights(1, key0, s1);
-            values(1, p1);
-        } else {
+            int pchunk_v = 0;                                  // the chunk whose keys kf holds or awaits
+            if (wave + NW < total_chunks) {
+                pchunk_v = next_pchunk();
+                load_k(pchunk_v, kf);
+            }
+            int c = wave;
+            // The chunks that lie before both tiles' rows and have two more behind them: no mask, no test
+            // for the end, so that the matrix instructions and the vector work stand in one stretch of code
+            // and are issued in turn (the order is said below: a wavefront issues in order, and a matrix
+            // instruction that waits for its pipe holds up the vector instructions behind it).
+            const int steady_end = min(total_chunks - 2 * NW, (pos0 + 1) / 32);
+            for (; c < steady_end; c += NW) {
+                afloatx4_t n0[2], n1[2];
+                const int pchunk_next = pchunk_v;
+                scores(0, n0);
+                scores(1, n1);
+                pchunk_v = next_pchunk();
+                load_k(pchunk_v, kf);
+                bool moved0, moved1;
+                float corr0, corr1;
+                const abf16x8_t p0 = weights_of(0, c * 32, s0, false, moved0, corr0);
+                // 16 matrix instructions among the vector work of one tile's weights
+#pragma unroll
+                for (int k = 0; k < 16; ++k) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+                }
+                if (moved0) rescale(0, corr0);
+                values(0, p0);
+                const abf16x8_t p1 = weights_of(1, c * 32, s1, false, moved1, corr1);
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+                }
+                if (moved1) rescale(1, corr1);
+                values(1, p1);
+                load_v(pchunk_next, vf);
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    s0[u] = n0[u];
+                    s1[u] = n1[u];
+                }
+            }
+            for (; c < total_chunks; c += NW) {
+                const int key0 = c * 32;
+                const bool more = c + NW < total_chunks;
+                afloatx4_t n0[2], n1[2];
+                const int pchunk_next = pchunk_v;
+                if (more) {
+                    scores(0, n0);
+                    scores(1, n1);
+                    if (c + 2 * NW < total_chunks) {
+                        pchunk_v = next_pchunk();
+                        load_k(pchunk_v, kf);
+                    }
+                }
+                const abf16x8_t p0 = weights(0, key0, s0);
+                values(0, p0);
+                const abf16x8_t p1 = weights(1, key0, s1);
+                values(1, p1);
+                if (more) {
+                    load_v(pchunk_next, vf);
+#pragma unroll
+                    for (int u = 0; u < 2; ++u) {
+                        s0[u] = n0[u];
+                        s1[u] = n1[u];
+                    }
+                }
+            }
+        }
+    } else {
+        for (int c = wave; c < total_chunks; c += NW) {
+            const int key0 = c * 32;
+            const bool more = c + NW < total_chunks;
+            int pchunkn = 0;
+            if (more) pchunkn = next_pchunk();
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 const bool active = r < n_tiles_used && key0 <= tile_last_pos[r];
@@ -785,8 +863,8 @@ __global__ __launch_bounds__(NW * 64) void attention_prefill_mfma_kernel(
                 if (r == R - 1 && more) load_k(pchunkn, kf);      // the last tile's scores are issued: keys are free
                 if (active) values(r, weights(r, key0, st));
             }
+            if (more) load_v(pchunkn, vf);
         }
-        if (more) load_v(pchunkn, vf);
     }
     if (NW > 1) {
         // wavefronts 1.. hand their running results to wavefront 0, one after the other through one buffer
