@@ -351,14 +351,19 @@ def attention_splits(n_tokens: int, nkv: int, group: int, max_keys: int) -> int:
       8 sequences at 4,096 keys 22/17/13/11/12/18, at 16,384 keys 72/42/30/26/28/32, at 32,768 149/84/55/48/48/53;
       16 sequences at 4,096 keys 25/18/17/17/20/27; 32 sequences 28/25/26/28/31/37; 64 sequences 47/46/48/50/52/68;
       one sequence at 16,384 keys 71/39/25/16/14/16, at 65,536 keys 296/154/83/46/31/26.
-    So: about 128 workgroups in all but at least 2 shares, a share of at least 512 keys, and at most 16 shares
+    So: about 128 workgroups in all (one share, and no merge kernel, once the step's sequences and kv heads give
+    that many by themselves: 64 sequences of the 0.5B shape save the merge's 4.7 us a layer), a share of at
+    least 512 keys, and at most 16 shares
     (32 from 16k keys on: the merge reads every share, but a workgroup's CU streams 37 GB/s at most, and one or
     two sequences give few workgroups.  In the whole step, one sequence at 32,000 keys: 3.82 against 3.90 ms
     with 32 instead of 16 shares, at 20,000 keys 3.68 against 3.71; two sequences 3.92 against 4.00)."""
     if n_tokens > 256:
         return 1
     groups = n_tokens * nkv * -(-group // 16)
-    return max(1, min(max(128 // max(groups, 1), 2), max_keys // 512, 16 if max_keys < 16384 else 32))
+    want = -(-128 // max(groups, 1))
+    if want == 1 and max_keys >= 4096:
+        want = 2            # long sequences: two shares even out the workgroups' ends (64 x 4,096 keys: 46 against 47 us)
+    return max(1, min(want, max_keys // 512, 16 if max_keys < 16384 else 32))
 
 
 def compress_keys(kpool: torch.Tensor, ckpool: torch.Tensor, nkv: int, page_table: torch.Tensor, page_size: int,
