@@ -108,7 +108,9 @@ struct SelectParams {
     int score_spilled, work_spilled;
 };
 
-template <typename T>
+// SPILL: the arrays lie in global scratch rows (a template switch, so that without it the compiler knows them
+// to be LDS and reads them with LDS instructions instead of generic ones)
+template <typename T, bool SPILL>
 __global__ __launch_bounds__(256) void sparse_select_kernel(const T* __restrict__ q, const T* __restrict__ ckpool,
                                                            PagedView pv, const int* __restrict__ positions,
                                                            const int* __restrict__ tok_slot, SelectParams sp,
@@ -119,11 +121,13 @@ __global__ __launch_bounds__(256) void sparse_select_kernel(const T* __restrict_
     const int p = positions[t];
     const long out_idx = (long)t * sp.nkv + g;
     // tmp[max_ck] score[max_ck] pool[max_blocks] flag[max_blocks] in LDS, or in this row of the global scratch
-    float* tmp = sp.score_spilled ? sp.spill + out_idx * sp.spill_stride : lds;
+    float* tmp = lds;
+    if constexpr (SPILL) tmp = sp.spill + out_idx * sp.spill_stride;
     float* score = tmp + sp.max_ck;
     float* pool = score + sp.max_ck;
     int* flag = (int*)(pool + sp.max_blocks);
-    float* qs = sp.score_spilled ? lds : (float*)(flag + sp.max_blocks);
+    float* qs = (float*)(flag + sp.max_blocks);
+    if constexpr (SPILL) qs = lds;
     if (p + 1 <= sp.dense_len) {
         if (tid == 0) sel_count[out_idx] = -1;
         return;
@@ -297,9 +301,10 @@ __global__ void select_scores_kernel(const bf16_t* __restrict__ q, const bf16_t*
                                      SelectParams sp, SelectScratch sc);
 __global__ void select_normalise_kernel(const int* __restrict__ positions, SelectParams sp, SelectScratch sc,
                                         int stats_in_lds);
+template <int SPILL>
 __global__ void select_blocks_kernel(const int* __restrict__ positions, SelectParams sp, SelectScratch sc,
                                      int* __restrict__ sel_blocks, int* __restrict__ sel_count, int stats_off);
-template <int HD, int NW>
+template <int HD, int NW, int SPILL>
 __global__ void sparse_select_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ ckpool, PagedView pv,
                                           const int* __restrict__ positions, const int* __restrict__ tok_slot,
                                           SelectParams sp, int* __restrict__ sel_blocks, int* __restrict__ sel_count);
@@ -412,12 +417,15 @@ extern "C" const char* cpmcu_sparse_select(const void* q, const void* ckpool, in
     PagedView pv{page_table, table_width, page_size};
     if (!pl.mfma) {
         sp.spill = pl.score_spilled ? scratch : nullptr;
-        if (dtype == CPMCU_F32)
-            sparse_select_kernel<float><<<grid, 256, pl.lds_main, stream>>>((const float*)q, (const float*)ckpool, pv,
-                                                                            positions, tok_slot, sp, sel_blocks, sel_count);
-        else
-            sparse_select_kernel<bf16_t><<<grid, 256, pl.lds_main, stream>>>((const bf16_t*)q, (const bf16_t*)ckpool, pv,
-                                                                             positions, tok_slot, sp, sel_blocks, sel_count);
+#define PLAIN(T, SP)                                                                                               \
+        sparse_select_kernel<T, SP><<<grid, 256, pl.lds_main, stream>>>((const T*)q, (const T*)ckpool, pv, positions, \
+                                                                        tok_slot, sp, sel_blocks, sel_count)
+        if (dtype == CPMCU_F32) {
+            if (pl.score_spilled) PLAIN(float, true); else PLAIN(float, false);
+        } else {
+            if (pl.score_spilled) PLAIN(bf16_t, true); else PLAIN(bf16_t, false);
+        }
+#undef PLAIN
         CPMCU_LAUNCH_CHECK("sparse_select");
         return nullptr;
     }
@@ -455,28 +463,34 @@ extern "C" const char* cpmcu_sparse_select(const void* q, const void* ckpool, in
             // the last kernel normalises the scores itself (the same sums in the same order): one kernel
             // of the chain less
             const size_t main8 = (pl.lds_main + 7) / 8 * 8;
-            select_blocks_kernel<<<grid, 1024, main8 + pl.lds_stats, stream>>>(positions, sp, sc, sel_blocks, sel_count,
-                                                                              (int)(main8 / sizeof(float)));
+            select_blocks_kernel<0><<<grid, 1024, main8 + pl.lds_stats, stream>>>(positions, sp, sc, sel_blocks, sel_count,
+                                                                                 (int)(main8 / sizeof(float)));
             CPMCU_LAUNCH_CHECK("select_blocks");
             return nullptr;
         }
         select_normalise_kernel<<<dim3(n, nkv, (sp.max_ck + 255) / 256), 256, pl.lds_stats, stream>>>(
             positions, sp, sc, pl.stats_in_lds ? 1 : 0);
         CPMCU_LAUNCH_CHECK("select_normalise");
-        select_blocks_kernel<<<grid, 1024, pl.lds_main, stream>>>(positions, sp, sc, sel_blocks, sel_count, 0);
+        const int spill = pl.work_spilled ? 2 : (pl.score_spilled ? 1 : 0);
+        if (spill == 2) select_blocks_kernel<2><<<grid, 1024, pl.lds_main, stream>>>(positions, sp, sc, sel_blocks, sel_count, 0);
+        else if (spill == 1) select_blocks_kernel<1><<<grid, 1024, pl.lds_main, stream>>>(positions, sp, sc, sel_blocks, sel_count, 0);
+        else select_blocks_kernel<0><<<grid, 1024, pl.lds_main, stream>>>(positions, sp, sc, sel_blocks, sel_count, 0);
         CPMCU_LAUNCH_CHECK("select_blocks");
         return nullptr;
     }
     sp.spill = pl.score_spilled ? scratch : nullptr;
     // few tokens (decode steps): 16 wavefronts share a (token, kv head)'s compressed keys; many: 4
+    const int spill = pl.work_spilled ? 2 : (pl.score_spilled ? 1 : 0);
+#define LAUNCH_S(HDv, NWv, SPv)                                                                              \
+    sparse_select_mfma_kernel<HDv, NWv, SPv><<<grid, NWv * 64, pl.lds_main, stream>>>(                       \
+        (const bf16_t*)q, (const bf16_t*)ckpool, pv, positions, tok_slot, sp, sel_blocks, sel_count)
 #define LAUNCH(HDv)                                                                                          \
     do {                                                                                                     \
-        if (n * nkv <= 256)                                                                                  \
-            sparse_select_mfma_kernel<HDv, 16><<<grid, 1024, pl.lds_main, stream>>>(                         \
-                (const bf16_t*)q, (const bf16_t*)ckpool, pv, positions, tok_slot, sp, sel_blocks, sel_count); \
-        else                                                                                                 \
-            sparse_select_mfma_kernel<HDv, 4><<<grid, 256, pl.lds_main, stream>>>(                           \
-                (const bf16_t*)q, (const bf16_t*)ckpool, pv, positions, tok_slot, sp, sel_blocks, sel_count); \
+        if (n * nkv <= 256) {                                                                                \
+            if (spill == 2) LAUNCH_S(HDv, 16, 2); else if (spill == 1) LAUNCH_S(HDv, 16, 1); else LAUNCH_S(HDv, 16, 0); \
+        } else {                                                                                             \
+            if (spill == 2) LAUNCH_S(HDv, 4, 2); else if (spill == 1) LAUNCH_S(HDv, 4, 1); else LAUNCH_S(HDv, 4, 0);    \
+        }                                                                                                    \
     } while (0)
     switch (hd) {
         case 16: LAUNCH(16); break;
@@ -489,6 +503,7 @@ extern "C" const char* cpmcu_sparse_select(const void* q, const void* ckpool, in
         default: LAUNCH(128); break;
     }
 #undef LAUNCH
+#undef LAUNCH_S
     CPMCU_LAUNCH_CHECK("sparse_select_mfma");
     return nullptr;
 }
@@ -509,7 +524,9 @@ extern "C" const char* cpmcu_sparse_select(const void* q, const void* ckpool, in
 typedef __bf16 sbf16x8_t __attribute__((ext_vector_type(8)));
 typedef float sfloatx4_t __attribute__((ext_vector_type(4)));
 
-template <int HD, int NW>
+// SPILL: 0 = scores and ranking arrays in LDS, 1 = scores in a scratch row, 2 = both (template switches, so that
+// the compiler knows which accesses are LDS)
+template <int HD, int NW, int SPILL>
 __global__ __launch_bounds__(NW * 64) void sparse_select_mfma_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ ckpool, PagedView pv,
     const int* __restrict__ positions, const int* __restrict__ tok_slot, SelectParams sp,
@@ -524,9 +541,13 @@ __global__ __launch_bounds__(NW * 64) void sparse_select_mfma_kernel(
     const int p = positions[t];
     const long out_idx = (long)t * sp.nkv + kvh;
     const int max_ck4 = (sp.max_ck + 3) / 4 * 4;
-    float* row_spill = sp.spill + out_idx * sp.spill_stride;
-    float* score = sp.score_spilled ? row_spill : lds;
-    float* work = sp.work_spilled ? row_spill + max_ck4 : (sp.score_spilled ? lds : lds + max_ck4);
+    float* score = lds;
+    float* work = lds + max_ck4;
+    if constexpr (SPILL >= 1) {
+        score = sp.spill + out_idx * sp.spill_stride;
+        work = lds;
+    }
+    if constexpr (SPILL == 2) work = sp.spill + out_idx * sp.spill_stride + max_ck4;
     if (p + 1 <= sp.dense_len) {
         if (tid == 0) sel_count[out_idx] = -1;
         return;
@@ -794,6 +815,7 @@ __global__ __launch_bounds__(256) void select_normalise_kernel(const int* __rest
 // stats_off (in floats, or 0): where in LDS the groups' (max, sum) pairs go when this kernel does the work of
 // select_normalise_kernel itself; 0: the scores come ready in sc.score (and are read from there, not copied
 // into LDS, when sp.score_spilled says that LDS cannot hold them)
+template <int SPILL>
 __global__ __launch_bounds__(1024) void select_blocks_kernel(const int* __restrict__ positions, SelectParams sp,
                                                              SelectScratch sc, int* __restrict__ sel_blocks,
                                                              int* __restrict__ sel_count, int stats_off) {
@@ -803,9 +825,13 @@ __global__ __launch_bounds__(1024) void select_blocks_kernel(const int* __restri
     const int t = blockIdx.x, kvh = blockIdx.y, tid = threadIdx.x;
     const int p = positions[t];
     const long out_idx = (long)t * sp.nkv + kvh;
-    float* score = sp.score_spilled ? sc.score + out_idx * sp.max_ck : lds;
-    float* work = sp.work_spilled ? sp.spill + out_idx * sp.spill_stride
-                                  : (sp.score_spilled ? lds : lds + (sp.max_ck + 3) / 4 * 4);
+    float* score = lds;
+    float* work = lds + (sp.max_ck + 3) / 4 * 4;
+    if constexpr (SPILL >= 1) {
+        score = sc.score + out_idx * sp.max_ck;
+        work = lds;
+    }
+    if constexpr (SPILL == 2) work = sp.spill + out_idx * sp.spill_stride;
     if (p + 1 <= sp.dense_len) {
         if (tid == 0) sel_count[out_idx] = -1;
         return;
@@ -841,7 +867,7 @@ __global__ __launch_bounds__(1024) void select_blocks_kernel(const int* __restri
             for (int h = 0; h < G; ++h) a += exp2f(s[(long)h * sp.max_ck] - ms[h]) * inv[h];
             score[j] = a;
         }
-    } else if (!sp.score_spilled) {
+    } else if constexpr (SPILL == 0) {
         for (int j = tid; j < n_vis; j += NW * 64) score[j] = sc.score[out_idx * sp.max_ck + j];
     }
     __syncthreads();
