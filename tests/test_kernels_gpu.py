@@ -73,14 +73,28 @@ def test_skinny_product_all_modes(M, N, K):
         assert float((act.double() - want).abs().max()) <= 2 ** -8 * float(want.abs().max()) + tol
 
 
-def test_skinny_split_heuristic_matches_what_the_kernel_accepts():
+def test_skinny_split_heuristic_gives_slices_that_sum_to_the_product():
+    """Whatever number of slices the heuristic chooses for a shape, the kernel takes it and the slices' partial
+    sums add up to the product (one-hot rows of x pick out columns of w, so the expected value is exact)."""
     from cpmcu_amd import ops
     for M in (1, 8, 64):
         for N, K in [(4608, 4096), (4096, 4096), (4096, 16384), (73448, 4096), (64, 64), (96, 160), (1000, 96)]:
             S = ops.skinny_split(M, N, K)
-            x, w = torch.zeros(M, K, dtype=torch.bfloat16, device=DEV), torch.zeros(N, K, dtype=torch.bfloat16, device=DEV)
+            assert 1 <= S <= 16 and (S == 1 or K // S >= 128)
+            x = torch.zeros(M, K, dtype=torch.bfloat16, device=DEV)
+            cols = [(7 * m + 3) * K // (7 * M + 4) for m in range(M)]            # spread over all slices
+            for m, c in enumerate(cols):
+                x[m, c] = 1.0
+            w = rnd(N, K, seed=N % 97, dtype=torch.bfloat16)
+            want = w[:, cols].T.float()
             if S > 1:
-                ops.gemm_skinny(x, w, torch.empty(S, M, N, dtype=torch.float32, device=DEV), mode="partial")
+                part = torch.full((S, M, N), float("nan"), dtype=torch.float32, device=DEV)
+                ops.gemm_skinny(x, w, part, mode="partial")
+                got = part.sum(0)
+            else:
+                got = torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)
+                ops.gemm_skinny(x, w, got)
+            assert torch.equal(got, want), (M, N, K, S)
 
 
 def test_products_refuse_what_they_do_not_take():
