@@ -181,21 +181,33 @@ class SequenceCache:
             freed += 1
         return need, freed
 
-    def room_for(self, extensions: Sequence[Tuple[int, int]]) -> Optional[str]:
-        """None if every group can take ``n_new`` more tokens for each (slot, n_new) at once, else the reason.
-        Each group is asked for what it really needs: a group that keeps a window counts the pages it gives
-        back.  A step that is cut into several passes never needs more than this."""
+    def room_for(self, passes: Sequence[Sequence[Tuple[int, int]]]) -> Optional[str]:
+        """None if the groups can take the tokens of a step that runs as these forward passes, each a list of
+        (slot, n_new) extended one after the other, else the reason.  Nothing is changed: the passes are played
+        through on counts alone.  Each group is asked for what it really needs: one that keeps a window gives
+        pages back from pass to pass, so a long prompt may bring more tokens than its pool holds."""
         for gi, g in enumerate(self.groups):
-            need = freed = 0
-            for slot, n_new in extensions:
-                old = self.length(slot)
-                a, b = self._group_need(g, slot, old, old + n_new)
-                need += a
-                freed += b
-            if need > len(g.free_pages) + freed:
-                return (f"the cache is full: this step needs {need} more pages of {self.page_size} tokens"
-                        f"{'' if len(self.groups) == 1 else f' in cache group {gi}'}, "
-                        f"{len(g.free_pages) + freed} are free of {g.n_pages}")
+            free = len(g.free_pages)
+            state: Dict[int, Tuple[int, int, int]] = {}        # slot -> (tokens, first held page number, page numbers)
+            for one in passes:
+                for slot, n_new in one:
+                    if slot not in state:
+                        pages = g.pages[slot]
+                        lo = next((pn for pn, p in enumerate(pages) if p >= 0), len(pages))
+                        state[slot] = (self.length(slot), lo, len(pages))
+                    old, lo, hi = state[slot]
+                    new = old + n_new
+                    first_kept = self._first_kept(g, old)
+                    lo2 = max(lo, first_kept)
+                    free += max(min(lo2, hi) - lo, 0)                  # given back before anything is taken
+                    hi2 = -(-new // self.page_size)
+                    need = max(hi2 - max(hi, first_kept), 0)
+                    if need > free:
+                        return (f"the cache is full: this step needs {need} more pages of {self.page_size} tokens"
+                                f"{'' if len(self.groups) == 1 else f' in cache group {gi}'} for slot {slot}, "
+                                f"{free} are free of {g.n_pages}")
+                    free -= need
+                    state[slot] = (new, lo2, max(hi, hi2))
         return None
 
     def pages_to_hold(self, length: int, step: int) -> List[int]:

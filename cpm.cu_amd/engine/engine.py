@@ -157,7 +157,7 @@ class Engine:
             for w in e.want:
                 if not 0 <= int(w) < n:
                     raise StepError(f"slot {e.slot}: wanted place {w} is outside the {n} tokens of this step")
-        full = self.cache.room_for([(e.slot, len(e.tokens)) for e in entries])
+        full = self.cache.room_for([[(entries[i].slot, b - a) for i, a, b in chunk] for chunk in self._chunks(entries)])
         if full is not None:
             raise StepError(f"{full} (max_tokens={self.options.max_tokens})")
 
@@ -244,7 +244,7 @@ class Engine:
             pages += have % cache.page_size == 0
         if pages:
             # a token that opens a page: ask the groups (one that keeps a window gives a page back for it)
-            full = cache.room_for([(s, 1) for s in slots])
+            full = cache.room_for([[(s, 1) for s in slots]])
             if full is not None:
                 raise StepError(f"{full} (max_tokens={self.options.max_tokens})")
         before = [live[s] for s in slots]

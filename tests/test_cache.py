@@ -119,7 +119,7 @@ def test_a_windowed_sequence_may_outgrow_the_pool():
     assert g.table.shape[1] == 25                                               # ceil(400 / 16)
     c.extend(s, 30)
     for _ in range(370):
-        assert c.room_for([(s, 1)]) is None
+        assert c.room_for([[(s, 1)]]) is None
         c.extend(s, 1)
         assert g.held(s) <= 3
         c.check()
@@ -134,17 +134,39 @@ def test_room_is_asked_of_every_group_and_counts_what_a_window_gives_back():
     c = make([FULL, WIN], max_tokens=64, max_slots=2, max_seq_len=400, page=16)
     a, b = c.acquire(), c.acquire()
     c.extend(a, 40)                                   # 3 of 4 pages in both groups
-    assert c.room_for([(b, 16)]) is None
-    msg = c.room_for([(b, 17)])                       # 2 pages: neither group has them
+    assert c.room_for([[(b, 16)]]) is None
+    msg = c.room_for([[(b, 17)]])                     # 2 pages: neither group has them
     assert msg is not None and "cache is full" in msg
-    assert c.room_for([(a, 24)]) is None              # a's 4th page
-    msg = c.room_for([(a, 25)])                       # a 5th page: the full-history group cannot, the window could
+    assert c.room_for([[(a, 24)]]) is None            # a's 4th page
+    msg = c.room_for([[(a, 25)]])                     # a 5th page: the full-history group cannot, the window could
     assert msg is not None and "group 0" in msg
+    assert c.room_for([[(a, 8), (b, 16)]]) is None and c.room_for([[(a, 8)], [(b, 17)]]) is not None
     assert c.pages_to_hold(400, 1) == [25, 3] and c.pages_to_hold(400, 64) == [25, 7]
     assert c.pages_to_hold(20, 64) == [2, 2] and c.capacity() == [4, 4]
     with pytest.raises(CacheError):
         c.extend(a, 25)
     assert c.length(a) == 40
+    c.check()
+
+
+def test_a_long_prompt_in_passes_fits_a_windowed_pool():
+    """What room_for plays through is what extend then does: a windowed group takes 300 tokens in passes of 32
+    (2 new pages beside the 2 a window of 20 still touches) through a pool of 4 pages, but not in one pass."""
+    c = make([WIN], max_tokens=64, max_slots=2, max_seq_len=400, page=16)
+    s = c.acquire()
+    passes = [[(s, 32)] for _ in range(9)] + [[(s, 12)]]
+    assert c.room_for(passes) is None
+    assert c.room_for([[(s, 64)], [(s, 64)]]) is not None          # the second pass would need 6 pages
+    assert c.room_for([[(s, 300)]]) is not None
+    for (slot, n), in passes:
+        c.extend(slot, n)
+        c.check()
+    assert c.length(s) == 300 and c.groups[0].held(s) <= 4
+    # a second sequence beside it: one page is left for it, not two
+    t = c.acquire()
+    assert c.room_for([[(t, 16)]]) is None or c.groups[0].held(s) == 4
+    c.release(s)
+    c.release(t)
     c.check()
 
 

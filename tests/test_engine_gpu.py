@@ -323,3 +323,47 @@ def test_built_in_yarn_factors_through_the_entry_point(tmp_path):
         check({"x": got}, {"x": ref}, dtype, f"yarn factors, {dtype}")
     with pytest.raises(ValueError, match="head_dim 128"):
         LLM(tiny.write_model(tiny.tiny_a(), str(tmp_path / "a"), seed=1), minicpm4_yarn=True)
+
+
+def test_a_forward_pass_that_fails_is_rolled_out_of_the_cache(model_dirs, references):
+    """A kernel that refuses in the middle of a step (forced here from the host) must not leave a sequence one
+    pass ahead of its cache rows: lengths and pages are as before the failing pass, and the same tokens then
+    give the right logits."""
+    from cpmcu_amd import StepEntry
+    cfg, w, reqs, refs = references["A"]
+    eng = engine_for(model_dirs, "A", "float32", max_step_tokens=16)
+    toks = reqs["d"]
+    s, t = eng.acquire(), eng.acquire()
+    eng.step([StepEntry(s, toks[:20], [])])
+    free = [len(g.free_pages) for g in eng.cache.groups]
+    real = eng.model.forward
+    calls = {"n": 0}
+
+    def failing(ctx):
+        calls["n"] += 1
+        if calls["n"] == 3:
+            raise RuntimeError("kernel refused")
+        return real(ctx)
+
+    eng.model.forward = failing
+    try:
+        with pytest.raises(RuntimeError, match="kernel refused"):
+            eng.step([StepEntry(s, toks[20:90], []), StepEntry(t, toks[:5], [])])       # 75 tokens: 5 passes of 16
+    finally:
+        eng.model.forward = real
+    assert eng.length(s) == 20 + 32 and eng.length(t) == 0          # two passes completed, the third was rolled back
+    eng.cache.check()
+    # single-token steps: the failing step leaves no trace
+    eng.model.forward = lambda ctx: (_ for _ in ()).throw(RuntimeError("kernel refused"))
+    try:
+        with pytest.raises(RuntimeError):
+            eng.step([StepEntry(s, [toks[52]], [0])])
+    finally:
+        eng.model.forward = real
+    assert eng.length(s) == 52
+    got = eng.step([StepEntry(s, toks[52:], list(range(len(toks) - 52)))]).cpu()
+    check({"d": got}, {"d": refs["d"][52:]}, "float32", "after a rolled-back pass")
+    eng.release(s)
+    eng.release(t)
+    eng.cache.check()
+    assert [len(g.free_pages) for g in eng.cache.groups] == [g.n_pages for g in eng.cache.groups] and free

@@ -83,9 +83,9 @@ def _define():
 
     MIXERS.register("toy_window_attention", WindowAttention)
 
-    def build(cfg: ToyConfig):
+    def build(cfg: ToyConfig, all_windowed: bool = False):
         layers = []
-        for i, kind in enumerate(("gqa_attention", "toy_window_attention")):
+        for i, kind in enumerate(("toy_window_attention" if all_windowed else "gqa_attention", "toy_window_attention")):
             p = f"layers.{i}."
             position = POSITION_ENCODINGS.build("rope", head_dim=cfg.head_dim, theta=cfg.rope_theta)
             extra = {"window": cfg.window} if kind == "toy_window_attention" else {}
@@ -104,13 +104,15 @@ def _define():
         norm = NORMS.build("rms_norm", name="norm.weight", hidden_size=cfg.hidden_size, eps=cfg.rms_norm_eps)
         return DecoderModel(cfg, emb, layers, norm, head)
 
-    register_architecture(Architecture("ToyWindowForCausalLM", ToyConfig, build), replace=True)
+    # an option of this architecture's own, declared to the registry (EngineOptions.model_options hands it over)
+    register_architecture(Architecture("ToyWindowForCausalLM", ToyConfig, build, options={"all_windowed": False}),
+                          replace=True)
     return ToyConfig
 
 
-def plain_toy(raw, w, toks):
-    """The same model, whole sequence, in float64 on the CPU: layer 0 sees every key before it, layer 1 the keys
-    from the block of position p - window + 1 on."""
+def plain_toy(raw, w, toks, all_windowed=False):
+    """The same model, whole sequence, in float64 on the CPU: layer 0 sees every key before it (unless
+    all_windowed), layer 1 the keys from the block of position p - window + 1 on."""
     import torch.nn.functional as F
     W = {k: v.double() for k, v in w.items()}
     n = len(toks)
@@ -136,7 +138,7 @@ def plain_toy(raw, w, toks):
         s = torch.einsum("qhd,khd->hqk", q, k) * hd ** -0.5
         qi, ki = torch.arange(n)[:, None], torch.arange(n)[None, :]
         seen = ki <= qi
-        if i == 1:
+        if i == 1 or all_windowed:
             seen = seen & (ki >= ((qi - win + 1).clamp(min=0) // BS) * BS)
         s = s.masked_fill(~seen[None], float("-inf"))
         o = torch.einsum("hqk,khd->qhd", torch.softmax(s, dim=-1), v).reshape(n, nh * hd)
@@ -189,6 +191,56 @@ def test_a_windowed_layer_beside_a_full_one(tmp_path, dtype):
             assert float((lg[1] - ref[i - 150]).abs().max()) < tol, i
             assert win.held(s) <= 3 and full.held(s) == i // 64 + 1
         assert float((torch.cat(outs) - ref).abs().max()) < tol
+        eng.release(s)
+        eng.release(other)
+        cache.check()
+    finally:
+        unregister_architecture("ToyWindowForCausalLM")
+        MIXERS.unregister("toy_window_attention")
+
+
+def test_a_model_of_windowed_layers_only_outgrows_the_cache_pool(tmp_path):
+    """With the architecture's own option `all_windowed` both layers keep a window: the one cache group then holds
+    a few pages a sequence however long it grows, so a sequence of 700 tokens runs in a cache of 256 (the prompt
+    in passes of 64 tokens, then token by token), and the planner's question of how many pages a sequence needs
+    is answered by the group."""
+    from safetensors.torch import load_file
+    from cpmcu_amd import Engine, EngineOptions, StepEntry, StepError
+    from cpmcu_amd.parts import MIXERS
+    from cpmcu_amd.registry import unregister_architecture
+    from cpmcu_amd.weights import write_model_dir
+    ToyConfig = _define()
+    try:
+        raw = {"architectures": ["ToyWindowForCausalLM"], "vocab_size": 120, "hidden_size": 64, "num_attention_heads": 4,
+               "num_key_value_heads": 2, "head_dim": 16, "intermediate_size": 96, "window": 64, "rope_theta": 10000.0,
+               "rms_norm_eps": 1e-5, "max_position_embeddings": 1024}
+        write_model_dir(ToyConfig.from_dict(raw), str(tmp_path), seed=8, std=0.1, norm_std=0.1)
+        w = load_file(str(tmp_path / "model.safetensors"))
+        with pytest.raises(ValueError, match="no option 'windowed'"):
+            Engine.from_dir(str(tmp_path), EngineOptions(dtype="float32", max_tokens=256, model_options={"windowed": True}))
+        eng = Engine.from_dir(str(tmp_path), EngineOptions(dtype="float32", max_tokens=256, max_slots=2, max_step_tokens=64,
+                                                           model_options={"all_windowed": True}))
+        cache = eng.cache
+        assert len(cache.groups) == 1 and cache.groups[0].needs.window == 64 and cache.capacity() == [4]
+        assert cache.pages_to_hold(700, 64) == [3] and cache.groups[0].table.shape[1] == 16
+        n = 700
+        toks = [int(t) for t in torch.randint(0, 120, (n,), generator=torch.Generator().manual_seed(3))]
+        ref = plain_toy(raw, w, toks, all_windowed=True).float()
+        s = eng.acquire()
+        outs = [eng.step([StepEntry(s, toks[:300], list(range(300)))]).cpu()]        # more tokens than the pool holds
+        for i in range(300, n):
+            outs.append(eng.step([StepEntry(s, [toks[i]], [0])]).cpu())
+            assert cache.groups[0].held(s) <= 3
+        assert eng.length(s) == n
+        got = torch.cat(outs)
+        err = (got - ref).abs().amax(1)
+        assert float(err.max()) < 1e-4, f"first wrong position {int((err >= 1e-4).nonzero()[0])}"
+        # a step that brings more tokens at once than the pool has room for is still refused, and changes nothing
+        other = eng.acquire()
+        eng.max_step_tokens = 512
+        with pytest.raises(StepError, match="cache is full"):
+            eng.step([StepEntry(other, toks[:200], [])])
+        assert eng.length(other) == 0
         eng.release(s)
         eng.release(other)
         cache.check()
