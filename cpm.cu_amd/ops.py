@@ -114,15 +114,15 @@ NORM_SLICE = 64        # columns a slice of add_norm_columns (common.h)
 
 # The kernels of decode steps that own a strip of output columns over all of K (qkv_rope, proj_add_norm) and
 # the norm cut by columns (add_norm_columns) save kernels of the chain, but every workgroup reads all of x.
-# Up to 16 rows they win at every width measured (MI355X, 4,096 columns: norm 4.7 against 6.6 us at 8 rows,
-# q/k/v + rotary 12.3 against 16.8 us at 8 rows and 15.1 against 18.0 at 16).  With more rows qkv_rope loses
-# (4,096 columns: 24.4 against 21.3 us at 32 rows; 1,024 columns: 16.8 + 4.7 against 8.9 + 5.1 + 4.2 us at 64),
-# and proj_add_norm wins only while a workgroup's copy of x stays small (1,024 columns, 64 rows: 8.6 against
-# 8.9 + 4.2 us).
+# Up to 16 rows they win at every width measured (MI355X, 4,096 columns: norm 4.7 against 6.6 us at 8 rows).
+# qkv_rope (workgroups spread evenly over the CUs) wins up to 32 rows (4,096 columns, q/k/v + rotary: 11.7
+# against 18.2 us at 16 rows, 15.6 against 19.7 at 24, 16.5 against 21.3 at 32; it loses beyond: 24.6 against
+# 21.3 at 48, 27.2 against 23.2 at 64), and proj_add_norm wins beyond 16 rows only while a workgroup's copy of
+# x stays small (1,024 columns, 64 rows: 8.6 against 8.9 + 4.2 us).
 STRIP_ROWS = 16
 STRIP_MAX_ROWS = 64
 STRIP_X_BYTES = 160 * 1024
-QKV_ROPE_MAX_ROWS = STRIP_ROWS
+QKV_ROPE_MAX_ROWS = 32
 
 
 def strip_kernels_ok(n: int, K: int) -> bool:

@@ -23,6 +23,7 @@ class Sampler:
         self.temperature = float(temperature)
         # no seed given: draws differ from run to run, as an unseeded generator's would
         self.seed = int(seed) if seed is not None else int.from_bytes(os.urandom(8), "little")
+        self._meta: Optional[torch.Tensor] = None
 
     @property
     def greedy(self) -> bool:
@@ -35,6 +36,31 @@ class Sampler:
         if self.greedy:
             ops.argmax(logits, out)
         else:
-            meta = torch.tensor([list(request_ids), list(steps)], dtype=torch.int32).to(logits.device)
-            ops.sample(logits, self.temperature, self.seed, meta[0].contiguous(), meta[1].contiguous(), out)
+            meta = self._upload(logits.device, request_ids, steps)
+            ops.sample(logits, self.temperature, self.seed, meta[0, :rows], meta[1, :rows], out)
         return out
+
+    def _upload(self, device, request_ids: Sequence[int], steps: Sequence[int]) -> torch.Tensor:
+        """Request ids and step numbers on the device, int32 [2, rows]: through a pinned buffer and into a device
+        buffer that both live as long as the sampler, so that a decode loop allocates nothing for them."""
+        rows = len(request_ids)
+        if self._meta is None or self._meta.shape[1] < rows or self._meta.device != device:
+            cap = max(rows, 64)
+            self._meta = torch.empty((2, cap), dtype=torch.int32, device=device)
+            self._stage = [torch.empty((2, cap), dtype=torch.int32).pin_memory() if device.type == "cuda"
+                           else torch.empty((2, cap), dtype=torch.int32) for _ in range(2)]
+            self._events = [None, None]
+            self._turn = 0
+        i = self._turn
+        self._turn ^= 1
+        if self._events[i] is not None:
+            self._events[i].synchronize()            # the copy that last used this staging buffer has finished
+        st = self._stage[i]
+        st[0, :rows] = torch.as_tensor(list(request_ids), dtype=torch.int32)
+        st[1, :rows] = torch.as_tensor(list(steps), dtype=torch.int32)
+        self._meta[:, :rows].copy_(st[:, :rows], non_blocking=True)
+        if device.type == "cuda":
+            ev = torch.cuda.Event()
+            ev.record()
+            self._events[i] = ev
+        return self._meta
