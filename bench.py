@@ -326,6 +326,15 @@ def other_scenarios(args, dev):
                       "layers_full_model": 32, "kernel_size": 32, "kernel_stride": 16, "block_size": 64, "topk": 64,
                       "window_size": 2048, "dense_len": 8192, "prompt_tokens": n_prompt, "new_tokens": new,
                       "parallelism": "1gpu", "hip_graph": bool(args.hip_graph)}, "points": {}}
+    # warm-up: one whole prompt and a few decode steps (kernel libraries loaded, the weights' decode layouts made,
+    # scratch grown to this context's sizes; none of that belongs to a step)
+    s = eng.acquire()
+    warm = [int(t) for t in torch.randint(0, cfg.vocab_size, (n_prompt + 4,), generator=g)]
+    for a in range(0, n_prompt, 2048):
+        eng.step([StepEntry(s, warm[a:min(a + 2048, n_prompt)], [])])
+    for i in range(4):
+        eng.step([StepEntry(s, [warm[n_prompt + i]], [0])])
+    eng.release(s)
     for batch in (1, 4):
         slots = [eng.acquire() for _ in range(batch)]
         ids = [[int(t) for t in torch.randint(0, cfg.vocab_size, (n_prompt + new,), generator=g)] for _ in slots]
