@@ -403,47 +403,44 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_mfma_kernel(
 }
 
 // out[token][head][:] = sum_s 2^(m_s - m) o_s / sum_s 2^(m_s - m) l_s   (splits without keys have l = 0)
+// Up to 64 shares: lane s of every wavefront holds share s's (max, sum), so that all of them come back in one
+// trip to memory and the common maximum and the denominator are wave reductions; a share's weight is then read
+// from its lane (the launcher takes no more than 64 shares).
+__device__ inline float share_weight(float w, int s) {       // lane s's w, for a uniform s
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w), s));
+}
+// HELD > 0: up to HELD shares and one feature a thread: the shares' outputs are asked for before anything
+// waits for the (max, sum) pairs, so that both come back in one trip to memory instead of two.
+template <int HELD>
 __global__ void attention_combine_kernel(const float* __restrict__ part_o, const float2* __restrict__ part_ml,
                                          bf16_t* __restrict__ out, int hd, int n_splits) {
-    __shared__ float wgt[64];
     const long row = blockIdx.x;             // token * nh + head
     const float2* ml = part_ml + row * n_splits;
     const float* po = part_o + row * n_splits * hd;
-    // Up to 16 shares and one feature a thread: the shares' outputs are asked for before anything waits for
-    // the (max, sum) pairs, so that both come back in one trip to memory instead of two.
-    const bool held = n_splits <= 16 && hd <= (int)blockDim.x;
-    float held_o[16];
-    if (held) {
+    const int lane = threadIdx.x & 63;
+    float held_o[HELD > 0 ? HELD : 1];
+    if (HELD > 0) {
         const int d = min((int)threadIdx.x, hd - 1);
 #pragma unroll
-        for (int s = 0; s < 16; ++s) held_o[s] = po[(long)min(s, n_splits - 1) * hd + d];
+        for (int s = 0; s < HELD; ++s) held_o[s] = po[(long)min(s, n_splits - 1) * hd + d];
     }
-    float m = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) {
-        const float2 v = ml[s];
-        if (v.y > 0.f) m = fmaxf(m, v.x);
-    }
-    float denom = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-        const float2 v = ml[s];
-        const float wv = v.y > 0.f ? exp2f(v.x - m) : 0.f;
-        denom += wv * v.y;
-        if (threadIdx.x == 0) wgt[s] = wv;
-    }
-    __syncthreads();
-    const float inv = 1.0f / denom;
-    if (held) {
+    float2 v = make_float2(-INFINITY, 0.f);
+    if (lane < n_splits) v = ml[lane];
+    const bool live = v.y > 0.f;
+    const float m = wave_max(live ? v.x : -INFINITY);
+    const float wv = live ? exp2f(v.x - m) : 0.f;
+    const float inv = 1.0f / wave_sum(wv * v.y);
+    if (HELD > 0) {
         float a = 0.f;
 #pragma unroll
-        for (int s = 0; s < 16; ++s)
-            if (s < n_splits) a += wgt[s] * held_o[s];
+        for (int s = 0; s < HELD; ++s) a += share_weight(wv, s) * held_o[s];   // lanes >= n_splits hold 0
         if ((int)threadIdx.x < hd) out[row * hd + threadIdx.x] = f32_to_bf16(a * inv);
         return;
     }
     for (int d = threadIdx.x; d < hd; d += blockDim.x) {
         float a = 0.f;
 #pragma unroll 8
-        for (int s = 0; s < n_splits; ++s) a += wgt[s] * po[(long)s * hd + d];
+        for (int s = 0; s < n_splits; ++s) a += share_weight(wv, s) * po[(long)s * hd + d];
         out[row * hd + d] = f32_to_bf16(a * inv);
     }
 }
@@ -455,8 +452,7 @@ static const char* attention_mfma_launch(const void* q, void* out, float* part_o
                                          const int* page_table, int table_width, int page_size,
                                          const int* positions, const int* tok_slot, const int* sel_blocks,
                                          const int* sel_count, int max_sel, int block_size, int n_splits,
-                                         int waves_per_group, int last_blocks_first, int merge,
-                                         hipStream_t stream) {
+                                         int waves_per_group, int last_blocks_first, hipStream_t stream) {
     CPMCU_REQUIRE(n > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_mfma: bad shape n=%d heads=%d kv_heads=%d", n, nh, nkv);
     CPMCU_REQUIRE(hd >= 16 && hd <= 128 && hd % 16 == 0,
                   "attention_mfma: head_dim %d has no matrix-core kernel (16, 32, ... 128 have; the plain kernel takes the rest)", hd);
@@ -501,11 +497,15 @@ static const char* attention_mfma_launch(const void* q, void* out, float* part_o
 #undef BY_NW
 #undef LAUNCH
     CPMCU_LAUNCH_CHECK("attention_mfma");
-    // merge == 0 leaves the shares (part_o, part_ml) for a consumer that merges them itself
-    // (gemm.hip: cpmcu_gemm_skinny_shares); `out` is then not written
-    if (n_splits > 1 && merge) {
-        attention_combine_kernel<<<(unsigned)((long)n * nh), hd > 64 ? 128 : 64, 0, stream>>>(
-            part_o, (const float2*)part_ml, (bf16_t*)out, hd, n_splits);
+    if (n_splits > 1) {
+        const unsigned rows = (unsigned)((long)n * nh), threads = hd > 64 ? 128 : 64;     // threads >= hd
+#define COMBINE(HELDv) attention_combine_kernel<HELDv><<<rows, threads, 0, stream>>>( \
+            part_o, (const float2*)part_ml, (bf16_t*)out, hd, n_splits)
+        if (n_splits <= 8) COMBINE(8);
+        else if (n_splits <= 16) COMBINE(16);
+        else if (n_splits <= 32) COMBINE(32);
+        else COMBINE(0);
+#undef COMBINE
         CPMCU_LAUNCH_CHECK("attention_combine");
     }
     return nullptr;
@@ -516,11 +516,10 @@ extern "C" const char* cpmcu_attention_mfma(const void* q, void* out, float* par
                                             const int* page_table, int table_width, int page_size,
                                             const int* positions, const int* tok_slot, const int* sel_blocks,
                                             const int* sel_count, int max_sel, int block_size, int n_splits,
-                                            int waves_per_group, int last_blocks_first, int merge,
-                                            hipStream_t stream) {
+                                            int waves_per_group, int last_blocks_first, hipStream_t stream) {
     return attention_mfma_launch(q, out, part_o, part_ml, n, nh, nkv, hd, scale, kpool, vtpool, page_table,
                                  table_width, page_size, positions, tok_slot, sel_blocks, sel_count, max_sel,
-                                 block_size, n_splits, waves_per_group, last_blocks_first, merge, stream);
+                                 block_size, n_splits, waves_per_group, last_blocks_first, stream);
 }
 
 // ---------------------------------------------------------------------------
@@ -586,7 +585,7 @@ extern "C" const char* cpmcu_attention_mfma_static(const void* q, void* out, int
     }
     return attention_mfma_launch(q, out, part_o, part_ml, n, nh, nkv, hd, scale, kpool, vtpool, page_table,
                                  table_width, page_size, positions, tok_slot, sel_blocks, sel_count, max_sel,
-                                 block_size, n_splits, waves_per_group, last_blocks_first, 1, stream);
+                                 block_size, n_splits, waves_per_group, last_blocks_first, stream);
 }
 
 // ===========================================================================

@@ -102,31 +102,20 @@ typedef float floatx4_t __attribute__((ext_vector_type(4)));
 #define SK_XC 512            // K columns of X staged at a time
 #define SK_XS (SK_XC + 8)    // LDS row stride in elements (16 bytes of padding)
 
-// X given as the shares of a split-KV attention (attention.hip: part_o [row][head][share][hd] float, part_ml
-// [row][head][share] (max, sum)) instead of a matrix: x[row][head*hd + d] = sum_s 2^(m_s - m) o_s[d] /
-// sum_s 2^(m_s - m) l_s, rounded to bf16, formed while X is staged.  The sums run in the order of
-// attention_combine_kernel, whose kernel and trip to memory this saves for steps of one or two tokens (with more
-// rows the shares, n_splits times the size of x and read by every workgroup, cost more than that kernel).
-struct XShares {
-    const float* part_o;
-    const float2* part_ml;
-    int n_splits, nh, hd;
-};
-
 // KW (1 or 2): groups of NW wavefronts a workgroup.  With 2, both groups own the same strips and share the
 // staged X; of every chunk of 4 K-blocks the first group multiplies blocks 0, 1 and the second blocks 2, 3, and
 // the second hands its sums to the first through LDS at the end.  With 48 and more rows a wavefront is busy
 // issuing (4 tiles of rows an operand load) rather than waiting, and one wavefront a SIMD cannot hide that:
 // twice the wavefronts on the same X traffic.
-template <int MT, int MODE, typename OT, int SPW, int NW, bool TILED, bool SHARES = false, int KW = 1>
+template <int MT, int MODE, typename OT, int SPW, int NW, bool TILED, int KW = 1>
 __global__ __launch_bounds__(NW * KW * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ X, long ldx,
                                                              const bf16_t* __restrict__ W, long ldw,
                                                              OT* __restrict__ Y, long ldy, int M, int N, int K, int KS,
                                                              float alpha, int I, long part_stride,
                                                              const float* __restrict__ row_ss, int ss_slices,
-                                                             float eps, XShares xsh) {
+                                                             float eps) {
     static_assert(MODE != 2 || SPW == 2, "gated output pairs a gate strip with an up strip");
-    static_assert(KW == 1 || (KW == 2 && !SHARES), "one or two groups of wavefronts");
+    static_assert(KW == 1 || KW == 2, "one or two groups of wavefronts");
     constexpr int NT = NW * KW * 64;
     constexpr int XV = MT * 16 * 64 / NT;     // 16-byte vectors of X a thread stages per chunk
     constexpr int BPW = 4 / KW;               // K-blocks of a chunk a wavefront multiplies
@@ -192,42 +181,7 @@ if (TILED) {
             const int idx = tid + v * NT;
             const int xrow = idx >> 6, vec = idx & 63;
             bf16x8_t val = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (SHARES) {
-                if (xrow < M && k0 + vec * 8 < k_end) {
-                    const int kcol = k0 + vec * 8, head = kcol / xsh.hd, d = kcol - head * xsh.hd;
-                    const long rh = (long)xrow * xsh.nh + head;
-                    const float2* ml = xsh.part_ml + rh * xsh.n_splits;
-                    const float* po = xsh.part_o + rh * xsh.n_splits * xsh.hd + d;
-                    // at most 8 shares: everything is asked for before anything is waited for (one trip to
-                    // memory; a share beyond the last repeats it and gets no weight)
-                    float2 t[8];
-                    float4 p0[8], p1[8];
-#pragma unroll
-                    for (int s = 0; s < 8; ++s) {
-                        const int sc = min(s, xsh.n_splits - 1);
-                        t[s] = ml[sc];
-                        p0[s] = *(const float4*)(po + (long)sc * xsh.hd);
-                        p1[s] = *(const float4*)(po + (long)sc * xsh.hd + 4);
-                    }
-                    float mx = -INFINITY;
-#pragma unroll
-                    for (int s = 0; s < 8; ++s)
-                        if (s < xsh.n_splits && t[s].y > 0.f) mx = fmaxf(mx, t[s].x);
-                    float denom = 0.f, a[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int s = 0; s < 8; ++s) {
-                        const float wv = (s < xsh.n_splits && t[s].y > 0.f) ? exp2f(t[s].x - mx) : 0.f;
-                        denom += wv * t[s].y;
-                        a[0] += wv * p0[s].x; a[1] += wv * p0[s].y; a[2] += wv * p0[s].z; a[3] += wv * p0[s].w;
-                        a[4] += wv * p1[s].x; a[5] += wv * p1[s].y; a[6] += wv * p1[s].z; a[7] += wv * p1[s].w;
-                    }
-                    const float inv = 1.0f / denom;
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) val[e] = (__bf16)(a[e] * inv);
-                }
-            } else if (xrow < M && k0 + vec * 8 < k_end) {
-                val = *(const bf16x8_t*)(X + (long)xrow * ldx + k0 + vec * 8);
-            }
+            if (xrow < M && k0 + vec * 8 < k_end) val = *(const bf16x8_t*)(X + (long)xrow * ldx + k0 + vec * 8);
             xr[v] = val;
         }
     };
@@ -366,13 +320,13 @@ extern "C" const char* cpmcu_gemm_skinny_v(const void* X, long ldx, const void* 
         const int rows_wg = (MODEv == 2) ? NW * 16 : NW * SPW * 16;                                               \
         dim3 grid(((MODEv == 2 ? I : N) + rows_wg - 1) / rows_wg, ksplit);                                        \
         if (tiled)                                                                                                \
-            gemm_skinny_kernel<MTv, MODEv, OT, SPW, NW, true, false, KWv><<<grid, NW * KWv * 64, 0, stream>>>(    \
+            gemm_skinny_kernel<MTv, MODEv, OT, SPW, NW, true, KWv><<<grid, NW * KWv * 64, 0, stream>>>(    \
                 (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (OT*)Y, ldy, M, N, K, KS, alpha, I, part_stride,    \
-                row_ss, ss_slices, eps, XShares{});                                                               \
+                row_ss, ss_slices, eps);                                                                          \
         else                                                                                                      \
-            gemm_skinny_kernel<MTv, MODEv, OT, SPW, NW, false, false, KWv><<<grid, NW * KWv * 64, 0, stream>>>(   \
+            gemm_skinny_kernel<MTv, MODEv, OT, SPW, NW, false, KWv><<<grid, NW * KWv * 64, 0, stream>>>(   \
                 (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (OT*)Y, ldy, M, N, K, KS, alpha, I, part_stride,    \
-                row_ss, ss_slices, eps, XShares{});                                                               \
+                row_ss, ss_slices, eps);                                                                          \
     } while (0)
 // shapes that measured best: one strip a wave in workgroups of 4 waves; gated output in workgroups of
 // 2 waves up to 16 rows of X (variant 1), of 4 waves above (variant 0)
@@ -413,32 +367,4 @@ extern "C" const char* cpmcu_gemm_skinny(const void* X, long ldx, const void* W,
     const int variant = out_mode == 2 ? (M <= 16 ? 1 : (M > 32 ? 4 : 0)) : 2;
     return cpmcu_gemm_skinny_v(X, ldx, W, ldw, Y, ldy, out_dtype, out_mode, M, N, K, ksplit, alpha, variant, tiled,
                                row_ss, ss_slices, eps, stream);
-}
-
-// The same product with X given as attention shares (see XShares): rows = tokens (at most 16), K = nh * hd,
-// tiled W, float output: out_mode 0 = Y[m,N], 1 = partial sums Y[ksplit][m][N].
-extern "C" const char* cpmcu_gemm_skinny_shares(const float* part_o, const float* part_ml, int n_splits, int nh, int hd,
-                                                const void* W, void* Y, long ldy, int out_mode, int M, int N,
-                                                int ksplit, float alpha, hipStream_t stream) {
-    const int K = nh * hd;
-    CPMCU_REQUIRE(M > 0 && M <= 16, "gemm_skinny_shares: %d rows (1..16 are taken)", M);
-    CPMCU_REQUIRE(part_o && part_ml && n_splits >= 1 && n_splits <= 8 && nh > 0 && hd > 0 && hd % 8 == 0,
-                  "gemm_skinny_shares: bad shares (%d shares: 1..8 are taken; heads %d, head_dim %d)", n_splits, nh, hd);
-    CPMCU_REQUIRE(N > 0 && W && Y && ((uintptr_t)W % 16 == 0) && ((uintptr_t)part_o % 16 == 0),
-                  "gemm_skinny_shares: null or misaligned operand");
-    CPMCU_REQUIRE(out_mode == 0 || out_mode == 1, "gemm_skinny_shares: output mode %d (0 or 1)", out_mode);
-    CPMCU_REQUIRE(ksplit >= 1 && (out_mode == 1 || ksplit == 1), "gemm_skinny_shares: a K-split (%d) needs partial-sum output", ksplit);
-    int KS = (K + ksplit - 1) / ksplit;
-    KS = (KS + 127) / 128 * 128;
-    CPMCU_REQUIRE((K + KS - 1) / KS == ksplit, "gemm_skinny_shares: K=%d cannot be cut into %d slices of whole 128-blocks", K, ksplit);
-    XShares xsh{part_o, (const float2*)part_ml, n_splits, nh, hd};
-    dim3 grid((N + 63) / 64, ksplit);
-    if (out_mode == 0)
-        gemm_skinny_kernel<1, 0, float, 1, 4, true, true><<<grid, 256, 0, stream>>>(
-            nullptr, K, (const bf16_t*)W, K, (float*)Y, ldy, M, N, K, KS, alpha, N / 2, (long)M * ldy, nullptr, 0, 0.f, xsh);
-    else
-        gemm_skinny_kernel<1, 1, float, 1, 4, true, true><<<grid, 256, 0, stream>>>(
-            nullptr, K, (const bf16_t*)W, K, (float*)Y, ldy, M, N, K, KS, alpha, N / 2, (long)M * ldy, nullptr, 0, 0.f, xsh);
-    CPMCU_LAUNCH_CHECK("gemm_skinny_shares");
-    return nullptr;
 }

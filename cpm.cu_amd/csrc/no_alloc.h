@@ -7,7 +7,7 @@
 // attention.hip; every GPU the library runs on holds its CPMCU_STATIC_SCRATCH_FLOATS * 4 bytes until the
 // process ends).
 //
-//   cpmcu_attention_mfma_static(...)  =  cpmcu_attention_mfma(..., merge = 1) without part_o / part_ml
+//   cpmcu_attention_mfma_static(...)  =  cpmcu_attention_mfma(...) without part_o / part_ml
 //
 // * Inputs and outputs are the caller's, as before: q, out [n, heads * head_dim] bf16, the paged key and
 //   value pools, page table, positions, token slots, optional block lists.

@@ -15,37 +15,20 @@
 // from global memory into the B operand, asked for together with the weight's block), add their results
 // through LDS, and the first wavefront finishes.
 //
-// For steps of one or two tokens a may also be given as the shares of a split-KV attention (attention.hip:
-// part_o [row][head][share][hd] float, part_ml [row][head][share] (max, sum)):
-//     a[row][head * hd + d] = sum_s 2^(m_s - m) o_s[d] / sum_s 2^(m_s - m) l_s, rounded to bf16.
-// Every workgroup then merges the rows into LDS at its start (the sums in the order of
-// attention_combine_kernel), while its first blocks of the weight are on their way, and takes the B operand
-// from there: the merge kernel and its trip to memory are saved too.
 // (reference: the output projections src/model/minicpm4/minicpm4_attn.cuh:205, 319 and src/model/ffn.cuh:77-84
-// followed by add + norm src/model/norm.cuh:53-99; the merge of the shares
-// src/flash_attn/src/flash_fwd_kernel.h:2393-2425)
+// followed by add + norm src/model/norm.cuh:53-99)
 #include "common.h"
-
-struct AShares {
-    const float* part_o;
-    const float2* part_ml;
-    int n_splits, nh, hd;
-};
-#define PN_SHARE_ROWS 2          // tokens a step may have when a comes as shares
-#define PN_SHARE_K 8192          // widest a (heads * head_dim) held in LDS
 
 typedef __bf16 pbf16x8_t __attribute__((ext_vector_type(8)));
 typedef float pfloatx4_t __attribute__((ext_vector_type(4)));
 
 // PF: 128-column blocks of the weight a wavefront keeps in flight; NW: wavefronts a workgroup; MT: tiles of 16 tokens
-template <int PF, int NW, int MT, bool SHARES = false>
+template <int PF, int NW, int MT>
 __global__ __launch_bounds__(NW * 64) void proj_add_norm_kernel(
     const bf16_t* __restrict__ A, long lda, const bf16_t* __restrict__ W, int M, int N, int K, float alpha,
     float* __restrict__ x, const float* __restrict__ w_norm, bf16_t* __restrict__ out, float* __restrict__ row_ss,
-    int n_strips, AShares ash) {
-    static_assert(!SHARES || MT == 1, "shares come for one or two tokens");
+    int n_strips) {
     __shared__ float red[NW - 1][MT][4][64];
-    __shared__ __attribute__((aligned(16))) bf16_t as[SHARES ? PN_SHARE_ROWS * PN_SHARE_K : 8];
     const int strip = blockIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
@@ -61,17 +44,15 @@ __global__ __launch_bounds__(NW * 64) void proj_add_norm_kernel(
     // ahead.  No load stands in a branch that depends on data: addresses are clamped instead (a block beyond
     // the wavefront's last repeats the matrix's last and is not multiplied; columns beyond K repeat the row's
     // last 8 and meet the weight's zero padding), so the waits count exactly.
-    pbf16x8_t wv[PF][4], av[PF][SHARES ? 1 : MT][SHARES ? 1 : 4];
-    auto load_block = [&](int kb, pbf16x8_t (&wd)[4], pbf16x8_t (&ad)[SHARES ? 1 : MT][SHARES ? 1 : 4]) {
+    pbf16x8_t wv[PF][4], av[PF][MT][4];
+    auto load_block = [&](int kb, pbf16x8_t (&wd)[4], pbf16x8_t (&ad)[MT][4]) {
         const int kbc = min(kb, nkb - 1);
 #pragma unroll
         for (int i = 0; i < 4; ++i) wd[i] = __builtin_nontemporal_load((const pbf16x8_t*)(wp + ((long)kbc * 4 + i) * 512));
-        if (!SHARES) {
 #pragma unroll
-            for (int t = 0; t < MT; ++t)
+        for (int t = 0; t < MT; ++t)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) ad[t][i] = *(const pbf16x8_t*)(ap[t] + min(kbc * 128 + i * 32 + g * 8, K - 8));
-        }
+            for (int i = 0; i < 4; ++i) ad[t][i] = *(const pbf16x8_t*)(ap[t] + min(kbc * 128 + i * 32 + g * 8, K - 8));
     };
     pfloatx4_t acc[MT];
 #pragma unroll
@@ -84,74 +65,27 @@ __global__ __launch_bounds__(NW * 64) void proj_add_norm_kernel(
     float4 xin[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) xin[t] = *(const float4*)(x + (long)min(t * 16 + r, M - 1) * N + min(col, N - 4));
-    const bf16_t* as_row = as + min(r, M - 1) * K + g * 8;        // SHARES: this lane's row of a in LDS
-    auto multiply = [&](int kb, pbf16x8_t (&wd)[4], pbf16x8_t (&ad)[SHARES ? 1 : MT][SHARES ? 1 : 4]) {
+    auto multiply = [&](pbf16x8_t (&wd)[4], pbf16x8_t (&ad)[MT][4]) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            if (SHARES) {
-                const pbf16x8_t b = *(const pbf16x8_t*)(as_row + min(kb * 128 + i * 32, K - 8 - g * 8));
-                acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wd[i], b, acc[0], 0, 0, 0);
-            } else {
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
-                for (int t = 0; t < MT; ++t)
-                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wd[i], ad[t][i], acc[t], 0, 0, 0);
-            }
-        }
+            for (int t = 0; t < MT; ++t)
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wd[i], ad[t][i], acc[t], 0, 0, 0);
     };
 #pragma unroll
     for (int j = 0; j < PF; ++j) load_block(kb0 + j, wv[j], av[j]);
-    if (SHARES) {
-        // the rows of a, merged from the shares: a thread a run of 8 features of one head; at most 8 shares,
-        // everything asked for before anything is waited for (a share beyond the last repeats it and gets
-        // no weight)
-        const int vecs = K / 8;
-        for (int v = threadIdx.x; v < M * vecs; v += NW * 64) {
-            const int row = v / vecs, kcol = (v - row * vecs) * 8;
-            const int head = kcol / ash.hd, d = kcol - head * ash.hd;
-            const long rh = (long)row * ash.nh + head;
-            const float2* ml = ash.part_ml + rh * ash.n_splits;
-            const float* po = ash.part_o + rh * ash.n_splits * ash.hd + d;
-            float2 tm[8];
-            float4 p0[8], p1[8];
-#pragma unroll
-            for (int s = 0; s < 8; ++s) {
-                const int sc = min(s, ash.n_splits - 1);
-                tm[s] = ml[sc];
-                p0[s] = *(const float4*)(po + (long)sc * ash.hd);
-                p1[s] = *(const float4*)(po + (long)sc * ash.hd + 4);
-            }
-            float mx = -INFINITY;
-#pragma unroll
-            for (int s = 0; s < 8; ++s)
-                if (s < ash.n_splits && tm[s].y > 0.f) mx = fmaxf(mx, tm[s].x);
-            float denom = 0.f, e[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int s = 0; s < 8; ++s) {
-                const float wt = (s < ash.n_splits && tm[s].y > 0.f) ? exp2f(tm[s].x - mx) : 0.f;
-                denom += wt * tm[s].y;
-                e[0] += wt * p0[s].x; e[1] += wt * p0[s].y; e[2] += wt * p0[s].z; e[3] += wt * p0[s].w;
-                e[4] += wt * p1[s].x; e[5] += wt * p1[s].y; e[6] += wt * p1[s].z; e[7] += wt * p1[s].w;
-            }
-            const float inv = 1.0f / denom;
-            pbf16x8_t val;
-#pragma unroll
-            for (int q = 0; q < 8; ++q) val[q] = (__bf16)(e[q] * inv);
-            *(pbf16x8_t*)(as + row * K + kcol) = val;
-        }
-        __syncthreads();
-    }
     int kb = kb0;
     for (; kb + 2 * PF <= kb1; kb += PF) {           // every block and every block asked for exists
 #pragma unroll
         for (int j = 0; j < PF; ++j) {
-            multiply(kb + j, wv[j], av[j]);
+            multiply(wv[j], av[j]);
             load_block(kb + j + PF, wv[j], av[j]);
         }
     }
     for (; kb < kb1; kb += PF) {                      // the last blocks: nothing more, or only what exists, is asked for
 #pragma unroll
         for (int j = 0; j < PF; ++j) {
-            if (kb + j < kb1) multiply(kb + j, wv[j], av[j]);
+            if (kb + j < kb1) multiply(wv[j], av[j]);
             if (kb + j + PF < kb1) load_block(kb + j + PF, wv[j], av[j]);
         }
     }
@@ -202,8 +136,7 @@ extern "C" const char* cpmcu_proj_add_norm(const void* A, long lda, const void* 
     const int strips = (N + 15) / 16;
 #define LAUNCH(PFv, NWv, MTv)                                                                                   \
     proj_add_norm_kernel<PFv, NWv, MTv><<<strips, NWv * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, M, N, \
-                                                                        K, alpha, x, w_norm, (bf16_t*)out, row_ss, strips, \
-                                                                        AShares{})
+                                                                        K, alpha, x, w_norm, (bf16_t*)out, row_ss, strips)
     // 4 blocks in flight in each of 4 wavefronts measured best (8 wavefronts: the same; 8 blocks: slower)
     // (more tokens hold more of a in registers for every block in flight: fewer blocks then)
     if (M <= 16) LAUNCH(4, 4, 1);
@@ -211,28 +144,6 @@ extern "C" const char* cpmcu_proj_add_norm(const void* A, long lda, const void* 
     else LAUNCH(2, 4, 4);
 #undef LAUNCH
     CPMCU_LAUNCH_CHECK("proj_add_norm");
-    return nullptr;
-}
-
-// The same with a given as attention shares (see AShares): one or two tokens, at most 8 shares, K = nh * hd
-// at most 8,192.
-extern "C" const char* cpmcu_proj_add_norm_shares(const float* part_o, const float* part_ml, int n_splits, int nh, int hd,
-                                                  const void* W, int M, int N, float alpha, float* x,
-                                                  const float* w_norm, void* out, float* row_ss, hipStream_t stream) {
-    const long K = (long)nh * hd;
-    CPMCU_REQUIRE(M > 0 && M <= PN_SHARE_ROWS, "proj_add_norm_shares: %d tokens (1..%d are taken)", M, PN_SHARE_ROWS);
-    CPMCU_REQUIRE(part_o && part_ml && n_splits >= 1 && n_splits <= 8 && nh > 0 && hd > 0 && hd % 8 == 0 && K <= PN_SHARE_K,
-                  "proj_add_norm_shares: bad shares (%d shares: 1..8 are taken; heads %d, head_dim %d, at most %d columns)",
-                  n_splits, nh, hd, PN_SHARE_K);
-    CPMCU_REQUIRE(N > 0 && N % 4 == 0, "proj_add_norm_shares: N=%d must be a multiple of 4", N);
-    CPMCU_REQUIRE(W && x && w_norm && out && row_ss, "proj_add_norm_shares: null pointer");
-    CPMCU_REQUIRE(((uintptr_t)part_o % 16 == 0) && ((uintptr_t)W % 16 == 0) && ((uintptr_t)x % 16 == 0) &&
-                  ((uintptr_t)w_norm % 16 == 0) && ((uintptr_t)out % 8 == 0), "proj_add_norm_shares: operands must be 16-byte aligned");
-    const int strips = (N + 15) / 16;
-    proj_add_norm_kernel<4, 4, 1, true><<<strips, 256, 0, stream>>>(nullptr, K, (const bf16_t*)W, M, N, (int)K, alpha, x, w_norm,
-                                                                  (bf16_t*)out, row_ss, strips,
-                                                                  AShares{part_o, (const float2*)part_ml, n_splits, nh, hd});
-    CPMCU_LAUNCH_CHECK("proj_add_norm_shares");
     return nullptr;
 }
 

@@ -264,7 +264,7 @@ def attention_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hd: in
                    positions: torch.Tensor, tok_slot: torch.Tensor, n_splits: int = 1,
                    part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None,
                    sel_blocks: Optional[torch.Tensor] = None, sel_count: Optional[torch.Tensor] = None,
-                   block_size: int = 0, waves_per_group: int = 0, last_blocks_first: int = 0, merge: bool = True):
+                   block_size: int = 0, waves_per_group: int = 0, last_blocks_first: int = 0):
     """bf16 attention on the matrix cores (head_dim 16, 32, ... 128; pages and key blocks multiples of 32).
     With n_splits > 1 every token's keys are shared among n_splits wavefronts and merged afterwards;
     part_o float32 [n, nh, n_splits, hd] and part_ml float32 [n, nh, n_splits, 2] are its scratch.
@@ -290,7 +290,7 @@ def attention_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hd: in
         _p(q), _p(out), _p(part_o), _p(part_ml), c_int(n), c_int(nh), c_int(nkv), c_int(hd), c_float(scale),
         _p(kpool), _p(vpool), _p(page_table), c_int(page_table.shape[1]), c_int(page_size), _p(positions),
         _p(tok_slot), _p(sel_blocks), _p(sel_count), c_int(max_sel), c_int(block_size), c_int(n_splits),
-        c_int(waves_per_group), c_int(last_blocks_first), c_int(1 if merge else 0), _stream()))
+        c_int(waves_per_group), c_int(last_blocks_first), _stream()))
 
 
 def attention_prefill_tokens_per_wave(nh: int, nkv: int, tiles_per_wave: int = 4) -> int:
@@ -347,23 +347,26 @@ def prefill_tiles(q_lens: Sequence[int], tokens_per_wave: int, device) -> torch.
 
 def attention_splits(n_tokens: int, nkv: int, group: int, max_keys: int) -> int:
     """Shares of a token's keys for steps of few tokens.  Measured on the MI355X (head size 128, 2 kv heads,
-    workgroups of 4 wavefronts, graph replay, attention + merge, in us for 1/2/4/8/16/32 shares):
-      8 sequences at 4,096 keys 22/17/13/11/12/18, at 16,384 keys 72/42/30/26/28/32, at 32,768 149/84/55/48/48/53;
-      16 sequences at 4,096 keys 25/18/17/17/20/27; 32 sequences 28/25/26/28/31/37; 64 sequences 47/46/48/50/52/68;
-      one sequence at 16,384 keys 71/39/25/16/14/16, at 65,536 keys 296/154/83/46/31/26.
-    So: about 128 workgroups in all (one share, and no merge kernel, once the step's sequences and kv heads give
-    that many by themselves: 64 sequences of the 0.5B shape save the merge's 4.7 us a layer), a share of at
-    least 512 keys, and at most 16 shares
-    (32 from 16k keys on: the merge reads every share, but a workgroup's CU streams 37 GB/s at most, and one or
-    two sequences give few workgroups.  In the whole step, one sequence at 32,000 keys: 3.82 against 3.90 ms
-    with 32 instead of 16 shares, at 20,000 keys 3.68 against 3.71; two sequences 3.92 against 4.00)."""
+    workgroups of 4 wavefronts, graph replay over keys that come from memory, attention + merge, in us for
+    1/2/4/8/16/32 shares):
+      8 sequences at 4,096 keys 38/24/17/13/12.5/14, at 16,384 keys 146/80/47/32/30/30, at 32,768 279/150/87/59/53/55;
+      16 sequences at 4,096 keys 43/30/21/18/20/23; 24 sequences 44/34/24/27/27/31; 32 sequences 48/32/30/32/34/39;
+      64 sequences 55/52/53/57/59/71;
+      one sequence at 4,096 keys 22/15/11/8.8/7.9/7.6, at 16,384 keys 140/74/41/25/17/12.5, at 65,536 531/275/140/76/46/28;
+      4 sequences at 32,768 keys 278/148/80/49/32/30.
+    So: as many shares as give about 256 workgroups in all, one for every CU (a CU takes in ~30 GB/s however
+    much it has in flight; the merge kernel costs ~3 us whatever the number of shares up to 32), a share of at
+    least 128 keys, at most 32 shares (beyond 32 the merge kernel no longer holds every share's output in
+    registers: one sequence at 32,000 keys, whole step, 3.89 ms with 64 shares against 3.60 with 32).  A step
+    that has 128 workgroups or more by itself takes two shares from 4,096 keys on (they even out the
+    workgroups' ends) and one below (no merge kernel: 64 sequences of the 0.5B shape)."""
     if n_tokens > 256:
         return 1
     groups = n_tokens * nkv * -(-group // 16)
-    want = -(-128 // max(groups, 1))
-    if want == 1 and max_keys >= 4096:
-        want = 2            # long sequences: two shares even out the workgroups' ends (64 x 4,096 keys: 46 against 47 us)
-    return max(1, min(want, max_keys // 512, 16 if max_keys < 16384 else 32))
+    want = max(1, 256 // max(groups, 1))
+    if groups >= 128:
+        want = 2 if max_keys >= 4096 else 1
+    return max(1, min(want, max_keys // 128, 32))
 
 
 def compress_keys(kpool: torch.Tensor, ckpool: torch.Tensor, nkv: int, page_table: torch.Tensor, page_size: int,
@@ -597,31 +600,6 @@ def gated_strip(x: torch.Tensor, w: "TiledWeight", out: torch.Tensor, row_scale:
                                            c_float(row_scale.eps if row_scale is not None else 0.0), _stream()))
 
 
-PROJ_NORM_SHARE_ROWS = 2        # tokens, shares and columns proj_add_norm_shares takes
-PROJ_NORM_SHARE_SPLITS = 8
-PROJ_NORM_SHARE_K = 8192
-
-
-def proj_add_norm_shares(part_o: torch.Tensor, part_ml: torch.Tensor, w: "TiledWeight", alpha: float,
-                         x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, sums: torch.Tensor):
-    """proj_add_norm whose a is the merged output of a split-KV attention, given as its shares (part_o float32
-    [m, heads, shares, hd], part_ml float32 [m, heads, shares, 2]; see gemm_skinny_shares): one or two tokens,
-    at most 8 shares, heads * hd at most 8,192."""
-    _need(part_o, "attention shares", torch.float32, (None, None, None, None))
-    n, nh, S, hd = part_o.shape
-    _need(part_ml, "attention share stats", torch.float32, (n, nh, S, 2))
-    if not isinstance(w, TiledWeight) or w.K != nh * hd:
-        raise KernelError(f"proj_add_norm_shares: the weight must be tiled for K = {nh * hd}")
-    N = w.N
-    _need(x, "proj residual", torch.float32, (n, N))
-    _need(weight, "proj norm weight", torch.float32, (N,))
-    _need(out, "proj out", torch.bfloat16, (n, N))
-    _need(sums, "proj row sums", torch.float32, (n, -(-N // 16)))
-    _check(_fn("qkv", "cpmcu_proj_add_norm_shares")(_p(part_o), _p(part_ml), c_int(S), c_int(nh), c_int(hd), _p(w.data),
-                                                    c_int(n), c_int(N), c_float(alpha), _p(x), _p(weight), _p(out),
-                                                    _p(sums), _stream()))
-
-
 def gemm_skinny(x: torch.Tensor, w, out: torch.Tensor, alpha: float = 1.0, mode: str = "plain",
                 row_scale: Optional[RowScale] = None):
     """bf16 product for at most 64 rows of x on the matrix cores, streaming w once; w is [N, K] as in the
@@ -660,31 +638,6 @@ def gemm_skinny(x: torch.Tensor, w, out: torch.Tensor, alpha: float = 1.0, mode:
                                             _p(row_scale.sums if row_scale is not None else None),
                                             c_int(row_scale.sums.shape[1] if row_scale is not None else 0),
                                             c_float(row_scale.eps if row_scale is not None else 0.0), _stream()))
-
-
-def gemm_skinny_shares(part_o: torch.Tensor, part_ml: torch.Tensor, w: "TiledWeight", out: torch.Tensor,
-                       alpha: float = 1.0, mode: str = "plain"):
-    """The skinny product whose x is the merged output of a split-KV attention, given as its shares: part_o
-    float32 [m, heads, shares, hd], part_ml float32 [m, heads, shares, 2] (attention_mfma with merge=False);
-    x[m, head*hd + d] = merged, rounded to bfloat16 as the merge kernel would.  w tiled [N, heads*hd]; out float32
-    [m, N] ('plain') or [S, m, N] ('partial')."""
-    _need(part_o, "attention shares", torch.float32, (None, None, None, None))
-    M, nh, S, hd = part_o.shape
-    _need(part_ml, "attention share stats", torch.float32, (M, nh, S, 2))
-    if not isinstance(w, TiledWeight) or w.K != nh * hd:
-        raise KernelError(f"gemm_skinny_shares: the weight must be tiled for K = {nh * hd}")
-    N = w.N
-    if mode == "plain":
-        _need(out, "gemm out", torch.float32, (M, N))
-        ksplit, omode = 1, 0
-    elif mode == "partial":
-        _need(out, "gemm partial sums", torch.float32, (None, M, N))
-        ksplit, omode = out.shape[0], 1
-    else:
-        raise KernelError(f"gemm_skinny_shares: unknown mode '{mode}'")
-    _check(_fn("gemm", "cpmcu_gemm_skinny_shares")(_p(part_o), _p(part_ml), c_int(S), c_int(nh), c_int(hd), _p(w.data),
-                                                   _p(out), c_long(N), c_int(omode), c_int(M), c_int(N),
-                                                   c_int(ksplit), c_float(alpha), _stream()))
 
 
 SKINNY_MAX_ROWS = 64
@@ -735,18 +688,9 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, alpha: float = 1
     gemm_nt_plain(x, w, out, alpha)
 
 
-# rows up to which the output projection merges the shares of a split-KV attention itself (the shares are
-# n_splits times the size of the merged rows and every workgroup of the product reads them: beyond two rows
-# that costs more than the merge kernel it saves; MI355X, 8B shape, one sequence at 4,096 keys: 3.47 against
-# 3.57 ms a step)
-ATTENTION_SHARES_MAX_ROWS = 2
-
-
 def attention(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, ctx,
-              sel_blocks=None, sel_count=None, block_size=0, window_blocks=0, leave_shares=False):
-    """Attention of the step's queries over the cache, with the kernel that suits the step.
-    With ``leave_shares`` a split-KV attention of few rows is not merged: (part_o, part_ml) are returned for
-    gemm_skinny_shares, and ``out`` is not written; otherwise, and always when None is returned, out is."""
+              sel_blocks=None, sel_count=None, block_size=0, window_blocks=0):
+    """Attention of the step's queries over the cache, with the kernel that suits the step; writes ``out``."""
     if sel_count is None and not ctx.single_token and attention_mfma_ok(q, hd, page_size):
         r, nw = attention_prefill_shape(q.shape[0], nh, nkv, hd)
         tpw = attention_prefill_tokens_per_wave(nh, nkv, r)
@@ -763,19 +707,12 @@ def attention(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, c
         if sel_count is not None:
             keys = min(keys, sel_blocks.shape[2] * block_size)
         splits = attention_splits(n, nkv, nh // nkv, keys)
-        # up to 8,192 keys 8 shares serve as well as 16; beyond, more shares and the merge kernel win
-        # (one sequence at 16,384 keys: 4.03 ms a step with 8 shares merged by the product, 3.91 with 16)
-        want_shares = leave_shares and n <= ATTENTION_SHARES_MAX_ROWS and hd % 8 == 0 and keys <= 8192
-        if want_shares:
-            splits = min(splits, 8)          # what the product that merges them takes
         part_o = part_ml = None
         if splits > 1:
             part_o = ctx.ws.get("attn.part_o", (n, nh, splits, hd), torch.float32)
             part_ml = ctx.ws.get("attn.part_ml", (n, nh, splits, 2), torch.float32)
-        leave = want_shares and splits > 1
         attention_mfma(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, ctx.positions, ctx.tok_slot,
-                       splits, part_o, part_ml, sel_blocks, sel_count, block_size, last_blocks_first=window_blocks,
-                       merge=not leave)
-        return (part_o, part_ml) if leave else None
+                       splits, part_o, part_ml, sel_blocks, sel_count, block_size, last_blocks_first=window_blocks)
+        return
     attention_plain(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, ctx.positions, ctx.tok_slot,
                     sel_blocks, sel_count, block_size)

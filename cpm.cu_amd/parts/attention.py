@@ -107,17 +107,11 @@ class GQAAttention(Mixer):
 
     def attend_and_project(self, q, ctx: StepContext, cache: CacheView, sel=None, defer_last: bool = False):
         """Attention of q over the cache (all keys up to each query, or the blocks listed in ``sel``), then the
-        output projection; for steps of one or two tokens the projection merges the shares of the split-KV
-        attention itself (one kernel of the chain less)."""
+        output projection."""
         sel_blocks, sel_count, bs, window_blocks = sel if sel is not None else (None, None, 0, 0)
         out = ctx.ws.get("attn.out", tuple(q.shape), q.dtype)
-        shares = ops.attention(q, out, self.nh, self.nkv, self.hd, self.scale, cache.streams["k"],
-                               cache.streams["v"], cache.page_table, cache.page_size, ctx, sel_blocks, sel_count, bs,
-                               window_blocks, leave_shares=self.o.takes_attention_shares())
-        if shares is not None:
-            if defer_last and self.o.defers_shares(shares[0]):
-                return DeferredBranch(self.o, None, ctx, "attn.o", shares=shares)
-            return self.o.forward_shares(shares[0], shares[1], ctx, "attn.o")
+        ops.attention(q, out, self.nh, self.nkv, self.hd, self.scale, cache.streams["k"], cache.streams["v"],
+                      cache.page_table, cache.page_size, ctx, sel_blocks, sel_count, bs, window_blocks)
         if defer_last and self.o.defers(out):
             return DeferredBranch(self.o, out, ctx, "attn.o")
         return self.o.forward(out, ctx, "attn.o", out_dtype=torch.float32, partials=True)

@@ -118,17 +118,13 @@ class DeferredBranch:
     runs that product together with the residual add takes it as it is (``Norm.takes_deferred_branch``), for
     everybody else ``evaluate()`` runs the product as the part would have and gives the tensor."""
 
-    def __init__(self, linear, a: Optional[torch.Tensor], ctx: "StepContext", tag: str, shares=None):
-        # ``shares``: the input given as the (outputs, statistics) of a split-KV attention instead of ``a``
-        self.linear, self.a, self.ctx, self.tag, self.shares = linear, a, ctx, tag, shares
+    def __init__(self, linear, a: torch.Tensor, ctx: "StepContext", tag: str):
+        self.linear, self.a, self.ctx, self.tag = linear, a, ctx, tag
         self._value: Optional[torch.Tensor] = None
 
     def evaluate(self) -> torch.Tensor:
         if self._value is None:
-            if self.shares is not None:
-                self._value = self.linear.forward_shares(self.shares[0], self.shares[1], self.ctx, self.tag)
-            else:
-                self._value = self.linear.forward(self.a, self.ctx, self.tag, out_dtype=torch.float32, partials=True)
+            self._value = self.linear.forward(self.a, self.ctx, self.tag, out_dtype=torch.float32, partials=True)
         return self._value
 
 

@@ -61,30 +61,6 @@ class Linear(Part):
         return (self.tiled is not None and x.dtype == torch.bfloat16 and ops.strip_kernels_ok(x.shape[0], self.in_features)
                 and self.in_features % 8 == 0 and self.out_features % 4 == 0)
 
-    def defers_shares(self, part_o: torch.Tensor) -> bool:
-        """The same for an input given as attention shares [n, heads, shares, hd] (ops.proj_add_norm_shares)."""
-        n, _, S, _ = part_o.shape
-        return (self.tiled is not None and n <= ops.PROJ_NORM_SHARE_ROWS and S <= ops.PROJ_NORM_SHARE_SPLITS
-                and self.in_features <= ops.PROJ_NORM_SHARE_K and self.out_features % 4 == 0)
-
-    def takes_attention_shares(self) -> bool:
-        """Whether forward_shares exists for this layer (bf16 engine with the decode product's weight layout)."""
-        return self.tiled is not None
-
-    def forward_shares(self, part_o: torch.Tensor, part_ml: torch.Tensor, ctx: StepContext, tag: str,
-                       alpha: float = 1.0) -> torch.Tensor:
-        """forward(x) for x = the merged output of a split-KV attention given as its shares (ops.attention with
-        leave_shares): the product merges them while it stages x.  Float32 [n, out] or partial sums [S, n, out]."""
-        n = part_o.shape[0]
-        S = ops.skinny_split(n, self.out_features, self.in_features)
-        if S > 1:
-            out = ctx.ws.get(tag, (S, n, self.out_features), torch.float32)
-            ops.gemm_skinny_shares(part_o, part_ml, self.tiled, out, alpha, mode="partial")
-        else:
-            out = ctx.ws.get(tag, (n, self.out_features), torch.float32)
-            ops.gemm_skinny_shares(part_o, part_ml, self.tiled, out, alpha)
-        return out
-
     def _gated_skinny(self, n: int, dtype) -> bool:
         return (dtype == torch.bfloat16 and n <= ops.SKINNY_MAX_ROWS and self.in_features % 8 == 0
                 and (self.tiled is None or (self.out_features // 2) % 16 == 0))

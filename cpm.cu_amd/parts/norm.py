@@ -49,13 +49,9 @@ class RMSNorm(Norm):
             # of that product owns 16 columns over all of K and finishes them itself
             lin = branch.linear
             fits = lin.out_features == self.hidden_size
-            if fits and (lin.defers_shares(branch.shares[0]) if branch.shares is not None else lin.defers(branch.a)):
+            if fits and lin.defers(branch.a):
                 sums = ctx.ws.get(tag + ".sums16", (n, -(-self.hidden_size // 16)), torch.float32)
-                if branch.shares is not None:
-                    ops.proj_add_norm_shares(branch.shares[0], branch.shares[1], lin.tiled, branch_scale, x,
-                                             self.weight, out, sums)
-                else:
-                    ops.proj_add_norm(branch.a, lin.tiled, branch_scale, x, self.weight, out, sums)
+                ops.proj_add_norm(branch.a, lin.tiled, branch_scale, x, self.weight, out, sums)
                 return out, ops.RowScale(sums, self.eps)
             branch = branch.evaluate()
         sums = ctx.ws.get(tag + ".sums", (n, ops.norm_slices(self.hidden_size)), torch.float32)

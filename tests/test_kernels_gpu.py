@@ -413,56 +413,6 @@ def test_attention_over_scrambled_pages(nh, nkv, hd, dtype):
         assert not ops.attention_mfma_ok(q.view(n, -1), hd, page)
 
 
-@pytest.mark.parametrize("nh,nkv,hd,n", [(8, 2, 64, 2), (32, 2, 128, 1), (6, 3, 48, 2), (4, 1, 16, 1)])
-def test_output_projection_merges_attention_shares(nh, nkv, hd, n):
-    """For steps of one or two tokens the product after the attention merges the split-KV shares itself: the
-    same numbers as the merge kernel followed by the product (same sums in the same order), plain and in
-    partial sums."""
-    from cpmcu_amd import ops
-    page, splits = 64, 5
-    lens = [700, 300][:n]
-    ks, vs, kpool, vpool, table = paged_setup(lens, nkv, hd, page, torch.bfloat16, seed=hd)
-    positions = [L - 1 for L in lens]
-    q = rnd(n, nh * hd, seed=3, dtype=torch.bfloat16)
-    pos_t = torch.tensor(positions, dtype=torch.int32, device=DEV)
-    slot_t = torch.arange(n, dtype=torch.int32, device=DEV)
-    merged = torch.empty(n, nh * hd, dtype=torch.bfloat16, device=DEV)
-    po = torch.full((n, nh, splits, hd), float("nan"), device=DEV)
-    pm = torch.full((n, nh, splits, 2), float("nan"), device=DEV)
-    ops.attention_mfma(q, merged, nh, nkv, hd, hd ** -0.5, kpool, vpool, table, page, pos_t, slot_t, splits, po, pm)
-    untouched = torch.full_like(merged, 7.0)
-    ops.attention_mfma(q, untouched, nh, nkv, hd, hd ** -0.5, kpool, vpool, table, page, pos_t, slot_t, splits, po, pm,
-                       merge=False)
-    assert bool((untouched == 7.0).all())
-    N, K = 200, nh * hd
-    w = ops.TiledWeight(rnd(N, K, seed=4, dtype=torch.bfloat16, scale=K ** -0.5))
-    want = torch.empty(n, N, device=DEV)
-    ops.gemm_skinny(merged, w, want, 0.5)
-    got = torch.full((n, N), float("nan"), device=DEV)
-    ops.gemm_skinny_shares(po, pm, w, got, 0.5)
-    assert torch.equal(got, want)
-    if K >= 256:
-        want_p = torch.empty(2, n, N, device=DEV)
-        ops.gemm_skinny(merged, w, want_p, 1.0, mode="partial")
-        got_p = torch.full((2, n, N), float("nan"), device=DEV)
-        ops.gemm_skinny_shares(po, pm, w, got_p, 1.0, mode="partial")
-        assert torch.equal(got_p, want_p)
-    # the product that also adds into the residual and does the norm's column work takes the shares too
-    xr, wn = rnd(n, N, seed=5), rnd(N, seed=6) + 1.0
-    outs = []
-    for shares in (False, True):
-        x = xr.clone()
-        xw = torch.full((n, N), float("nan"), dtype=torch.bfloat16, device=DEV)
-        sums = torch.full((n, -(-N // 16)), float("nan"), device=DEV)
-        if shares:
-            ops.proj_add_norm_shares(po, pm, w, 0.5, x, wn, xw, sums)
-        else:
-            ops.proj_add_norm(merged, w, 0.5, x, wn, xw, sums)
-        outs.append((x, xw, sums))
-    assert all(torch.equal(u, v) for u, v in zip(*outs))
-    assert float((outs[0][0] - (xr + want)).abs().max()) <= 1e-5 * float(want.abs().max() + 1)
-
-
 @pytest.mark.parametrize("nh,nkv,hd", [(16, 1, 64), (8, 1, 32), (4, 2, 128), (5, 5, 16), (40, 2, 32), (6, 2, 48), (2, 1, 96)])
 def test_prompt_attention_from_position_zero_and_continued(nh, nkv, hd):
     """Whole prompts from position 0 (where early tiles stop before late chunks) and a chunk that continues

@@ -51,7 +51,7 @@ def _call_pair(new, old, lens, n_tok, nh, nkv, hd, splits, seed):
     torch.cuda.synchronize()
     msg = new(_ptr(q), _ptr(out_new), *common, stream)
     assert msg is None, msg
-    msg = old(_ptr(q), _ptr(out_old), _ptr(po), _ptr(pm), *common, c_int(1), stream)
+    msg = old(_ptr(q), _ptr(out_old), _ptr(po), _ptr(pm), *common, stream)
     assert msg is None, msg
     torch.cuda.synchronize()
     return out_new, out_old
