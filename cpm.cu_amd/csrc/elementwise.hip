@@ -40,6 +40,26 @@ extern "C" const char* cpmcu_embed(const void* table, int dtype, const int* ids,
 // `branch` may be null (plain norm), and may come as `nparts` partial sums of
 // a split matrix product, `part_stride` elements apart.
 // ---------------------------------------------------------------------------
+// The sum of nparts partial results `stride` elements apart, added in the order of the parts, up to 4 (8)
+// loads asked for together (see add_parts4 below for why).
+template <int W, typename BT>
+__device__ inline float add_parts(float acc, const BT* p, int first, int nparts, long stride) {
+    float t[W];
+#pragma unroll
+    for (int j = 0; j < W; ++j) t[j] = to_f32(p[(long)min(first + j, nparts - 1) * stride]);
+#pragma unroll
+    for (int j = 0; j < W; ++j)
+        if (first + j < nparts) acc += t[j];
+    return acc;
+}
+template <typename BT>
+__device__ inline float sum_parts(const BT* p, int nparts, long stride) {
+    if (nparts <= 4) return add_parts<4>(0.f, p, 0, nparts, stride);
+    float b = 0.f;
+    for (int f = 0; f < nparts; f += 8) b = add_parts<8>(b, p, f, nparts, stride);
+    return b;
+}
+
 template <typename BT, typename OT>
 __global__ void add_rms_norm_kernel(float* __restrict__ x, const BT* __restrict__ branch, int nparts,
                                     long part_stride, float bscale, const float* __restrict__ w, float eps,
@@ -52,8 +72,7 @@ __global__ void add_rms_norm_kernel(float* __restrict__ x, const BT* __restrict_
     for (int c = threadIdx.x; c < H; c += blockDim.x) {
         float v = xr[c];
         if (branch) {
-            float b = 0.f;
-            for (int p = 0; p < nparts; ++p) b += to_f32(branch[p * part_stride + r * H + c]);
+            const float b = sum_parts(branch + r * H + c, nparts, part_stride);
             v += bscale * b;
             if (!rows) xr[c] = v;
         }
@@ -65,8 +84,7 @@ __global__ void add_rms_norm_kernel(float* __restrict__ x, const BT* __restrict_
     for (int c = threadIdx.x; c < H; c += blockDim.x) {
         float v = xr[c];
         if (branch && rows) {
-            float b = 0.f;
-            for (int p = 0; p < nparts; ++p) b += to_f32(branch[p * part_stride + r * H + c]);
+            const float b = sum_parts(branch + r * H + c, nparts, part_stride);
             v += bscale * b;
         }
         o[c] = from_f32<OT>(v * rs * w[c]);
@@ -86,6 +104,29 @@ __device__ inline float4 load4(const bf16_t* p) {
     r.w = __uint_as_float(u.y & 0xffff0000u);
     return r;
 }
+// acc + the partial results first .. first + W - 1 (of nparts, `stride` elements apart), added in the order of
+// the parts.  The W loads are asked for together: a loop of single loads whose trip count the compiler does not
+// know waits for each load before it asks for the next, a trip to memory a part.  A part beyond the last repeats
+// the last one and is not added.
+template <int W, typename BT>
+__device__ inline float4 add_parts4(float4 acc, const BT* p, int first, int nparts, long stride) {
+    float4 t[W];
+#pragma unroll
+    for (int j = 0; j < W; ++j) t[j] = load4(p + (long)min(first + j, nparts - 1) * stride);
+#pragma unroll
+    for (int j = 0; j < W; ++j)
+        if (first + j < nparts) {
+            acc.x += t[j].x; acc.y += t[j].y; acc.z += t[j].z; acc.w += t[j].w;
+        }
+    return acc;
+}
+template <typename BT>
+__device__ inline float4 sum_parts4(const BT* p, int nparts, long stride) {
+    float4 b = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (nparts <= 4) return add_parts4<4>(b, p, 0, nparts, stride);
+    for (int f = 0; f < nparts; f += 8) b = add_parts4<8>(b, p, f, nparts, stride);
+    return b;
+}
 
 template <typename BT, typename OT>
 __global__ __launch_bounds__(1024) void add_rms_norm_vec4_kernel(float* __restrict__ x, const BT* __restrict__ branch,
@@ -101,11 +142,7 @@ __global__ __launch_bounds__(1024) void add_rms_norm_vec4_kernel(float* __restri
     auto summed = [&](int c) {
         float4 v = *(const float4*)(xr + 4 * c);
         if (branch) {
-            float4 b = make_float4(0.f, 0.f, 0.f, 0.f);
-            for (int p = 0; p < nparts; ++p) {
-                const float4 t = load4(branch + p * part_stride + r * H + 4 * c);
-                b.x += t.x; b.y += t.y; b.z += t.z; b.w += t.w;
-            }
+            const float4 b = sum_parts4(branch + r * H + 4 * c, nparts, part_stride);
             v.x += bscale * b.x; v.y += bscale * b.y; v.z += bscale * b.z; v.w += bscale * b.w;
         }
         return v;
@@ -223,12 +260,7 @@ __global__ __launch_bounds__(256) void add_norm_columns_kernel(float* __restrict
     const long off = (long)min(row, n - 1) * H + min(c, H - 4);
     float4 v = *(const float4*)(x + off);
     if (branch) {
-        float4 b = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll 8
-        for (int p = 0; p < nparts; ++p) {
-            const float4 t = load4(branch + p * part_stride + off);
-            b.x += t.x; b.y += t.y; b.z += t.z; b.w += t.w;
-        }
+        const float4 b = sum_parts4(branch + off, nparts, part_stride);
         v.x += bscale * b.x; v.y += bscale * b.y; v.z += bscale * b.z; v.w += bscale * b.w;
     }
     float ss = 0.f;
@@ -368,9 +400,7 @@ __global__ void rope_store_kernel(const IT* __restrict__ qkv, long width, int np
     for (int head = group; head < heads; head += groups) {
         const IT* row = qkv + t * width + (long)head * hd;
         auto load = [&](int i) {
-            float s = 0.f;
-            for (int p = 0; p < nparts; ++p) s += to_f32(row[p * part_stride + i]);
-            return s;
+            return sum_parts(row + i, nparts, part_stride);
         };
         if (head < nh + nkv) {
             // queries go out as plain rows; keys into their page in the matrix cores' order (key_index)
