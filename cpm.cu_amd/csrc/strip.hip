@@ -137,9 +137,13 @@ extern "C" const char* cpmcu_proj_add_norm(const void* A, long lda, const void* 
 #define LAUNCH(PFv, NWv, MTv)                                                                                   \
     proj_add_norm_kernel<PFv, NWv, MTv><<<strips, NWv * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, M, N, \
                                                                         K, alpha, x, w_norm, (bf16_t*)out, row_ss, strips)
-    // 4 blocks in flight in each of 4 wavefronts measured best (8 wavefronts: the same; 8 blocks: slower)
+    // 4 blocks in flight in each of 4 wavefronts measured best at K = 4,096 (8 wavefronts: the same; 8 blocks:
+    // slower; 16 wavefronts of 4 blocks spill)
     // (more tokens hold more of a in registers for every block in flight: fewer blocks then)
-    if (M <= 16) LAUNCH(4, 4, 1);
+    // long rows (down: K = 16,384) in 8 wavefronts of 2 blocks in flight: 24.3 against 25.1 us at 8 tokens, 27.4
+    // against 29.6 at 16; at K = 4,096 the two are level
+    if (M <= 16 && K >= 8192) LAUNCH(2, 8, 1);
+    else if (M <= 16) LAUNCH(4, 4, 1);
     else if (M <= 32) LAUNCH(4, 4, 2);
     else LAUNCH(2, 4, 4);
 #undef LAUNCH
