@@ -156,23 +156,32 @@ __global__ __launch_bounds__(NW * KW * 64) void gemm_skinny_kernel(const bf16_t*
         }
     }
 
+    // In the main loop no load stands in a branch: the compiler waits for every load in flight where such a
+    // branch ends, and the weights asked for a chunk ahead would have to be there before the chunk's x is stored
+    // (that wait cost the 64-row products a trip to memory a chunk).  Only the slice's last chunks (`guard`) ask
+    // whether a block or a column exists.
     bf16x8_t a[KW][BPW][SPW][4];              // [chunk parity][block of the wavefront]
-    auto load_w = [&](int kb, bf16x8_t (&dst)[SPW][4]) {
+    auto load_w = [&](int kb, bf16x8_t (&dst)[SPW][4], const bool guard) {
+        if (guard && kb >= nkb) {             // uniform; the block is multiplied by zeros of x or not at all
+#pragma unroll
+            for (int s = 0; s < SPW; ++s)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) dst[s][i] = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+            return;
+        }
         const int k = k_begin + kb * 128 + g * 8;
 #pragma unroll
         for (int s = 0; s < SPW; ++s)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                bf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
-if (TILED) {
-                    // one 128-block of a strip is 2048 elements: [i][lane][8]
-                    if (kb < nkb) v = __builtin_nontemporal_load((const bf16x8_t*)(wp[s] + ((long)(k_begin / 128 + kb) * 4 + i) * 512));
-                } else if (kb < nkb && k + i * 32 < k_end) {
-                    v = __builtin_nontemporal_load((const bf16x8_t*)(wp[s] + k + i * 32));
-                }
-                dst[s][i] = v;
+                if (TILED)                    // one 128-block of a strip is 2048 elements: [i][lane][8]
+                    dst[s][i] = __builtin_nontemporal_load((const bf16x8_t*)(wp[s] + ((long)(k_begin / 128 + kb) * 4 + i) * 512));
+                else                          // columns beyond K repeat the row's last 8 and meet zeros of x
+                    dst[s][i] = __builtin_nontemporal_load((const bf16x8_t*)(wp[s] + min(k + i * 32, K - 8)));
             }
     };
+    // rows beyond the step repeat its last row (their results are not written); columns beyond the slice are
+    // read from the row's end and replaced by zeros when the chunk is stored
     bf16x8_t xr[XV];
     auto load_x = [&](int chunk) {
         const int k0 = k_begin + chunk * SK_XC;
@@ -180,17 +189,17 @@ if (TILED) {
         for (int v = 0; v < XV; ++v) {
             const int idx = tid + v * NT;
             const int xrow = idx >> 6, vec = idx & 63;
-            bf16x8_t val = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (xrow < M && k0 + vec * 8 < k_end) val = *(const bf16x8_t*)(X + (long)xrow * ldx + k0 + vec * 8);
-            xr[v] = val;
+            xr[v] = *(const bf16x8_t*)(X + (long)min(xrow, M - 1) * ldx + min(k0 + vec * 8, K - 8));
         }
     };
-    auto store_x = [&]() {
+    auto store_x = [&](int chunk, const bool guard) {
+        const int k0 = k_begin + chunk * SK_XC;
 #pragma unroll
         for (int v = 0; v < XV; ++v) {
             const int idx = tid + v * NT;
             const int xrow = idx >> 6, vec = idx & 63;
-            *(bf16x8_t*)(xs + xrow * SK_XS + vec * 8) = xr[v];
+            const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+            *(bf16x8_t*)(xs + xrow * SK_XS + vec * 8) = (!guard || k0 + vec * 8 < k_end) ? xr[v] : zero;
         }
     };
 
@@ -200,44 +209,52 @@ if (TILED) {
 #pragma unroll
         for (int t = 0; t < MT; ++t) acc[s][t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
+    // x first: loads return in the order of their issue, and the loop's first store of x must not wait for more
+    // weights than its later ones do (the compiler takes the stricter of the two for all)
+    load_x(0);
 #pragma unroll
     for (int p = 0; p < KW; ++p)
 #pragma unroll
-        for (int jj = 0; jj < BPW; ++jj) load_w(p * 4 + kw * BPW + jj, a[p][jj]);
-    load_x(0);
+        for (int jj = 0; jj < BPW; ++jj)          // a block beyond a short slice repeats its last one
+            load_w(min(p * 4 + kw * BPW + jj, nkb - 1), a[p][jj], false);
     // X may be x * w of a norm whose row factor is still to come (common.h: row_scales); the loop's first
     // barrier makes rs_s visible
     __shared__ float rs_s[MT * 16];
     if (row_ss) row_scales<NT, MT * 16>(row_ss, ss_slices, M, 1.0f / (float)K, eps, rs_s);
-    const int nchunk = (nkb + 3) / 4;
+    const int nchunk = (nkb + 3) / 4, nfull = nkb / 4;       // chunks in all, chunks of 4 whole blocks
     // a wavefront's weight blocks are asked for KW chunks (4 blocks of its own) ahead; the chunk's parity picks
-    // the registers, so the loop advances KW chunks a turn
-    for (int c0 = 0; c0 < nchunk; c0 += KW) {
+    // the registers, so the loops advance KW chunks a turn
+    auto one_chunk = [&](int c, bf16x8_t (&ap)[BPW][SPW][4], const bool guard) {
+        __syncthreads();
+        store_x(c, guard);
+        __syncthreads();
+        if (!guard || c + 1 < nchunk) load_x(c + 1);
 #pragma unroll
-        for (int p = 0; p < KW; ++p) {
-            const int c = c0 + p;
-            if (c >= nchunk) break;
-            __syncthreads();
-            store_x();
-            __syncthreads();
-            if (c + 1 < nchunk) load_x(c + 1);
+        for (int jj = 0; jj < BPW; ++jj) {
+            const int j = kw * BPW + jj;
+            // consecutive matrix instructions go to different accumulators (tiles of rows, then strips)
 #pragma unroll
-            for (int jj = 0; jj < BPW; ++jj) {
-                const int j = kw * BPW + jj;
-                // consecutive matrix instructions go to different accumulators (tiles of rows, then strips)
+            for (int i = 0; i < 4; ++i) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
+                for (int t = 0; t < MT; ++t) {
+                    const bf16x8_t b = *(const bf16x8_t*)(xs + (t * 16 + r) * SK_XS + j * 128 + g * 8 + i * 32);
 #pragma unroll
-                    for (int t = 0; t < MT; ++t) {
-                        const bf16x8_t b = *(const bf16x8_t*)(xs + (t * 16 + r) * SK_XS + j * 128 + g * 8 + i * 32);
-#pragma unroll
-                        for (int s = 0; s < SPW; ++s)
-                            acc[s][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[p][jj][s][i], b, acc[s][t], 0, 0, 0);
-                    }
+                    for (int s = 0; s < SPW; ++s)
+                        acc[s][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ap[jj][s][i], b, acc[s][t], 0, 0, 0);
                 }
-                load_w((c + KW) * 4 + j, a[p][jj]);
             }
+            load_w((c + KW) * 4 + j, ap[jj], guard);
         }
+    };
+    int c0 = 0;
+    for (; c0 + 2 * KW <= nfull; c0 += KW) {          // these chunks, the next x and the blocks asked for are whole
+#pragma unroll
+        for (int p = 0; p < KW; ++p) one_chunk(c0 + p, a[p], false);
+    }
+    for (; c0 < nchunk; c0 += KW) {                   // the slice's end
+#pragma unroll
+        for (int p = 0; p < KW; ++p)
+            if (c0 + p < nchunk) one_chunk(c0 + p, a[p], true);
     }
     if (KW > 1) {
         // the second group's sums go to the first through LDS (the staged X is no longer needed)
