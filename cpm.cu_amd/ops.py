@@ -649,12 +649,17 @@ def skinny_ok(x: torch.Tensor, w=None) -> bool:
 
 def skinny_split(M: int, N: int, K: int) -> int:
     """Slices of K for a skinny product whose consumer sums partial results.  A workgroup streams 64 rows
-    of the weight; about 1024 workgroups balance well over the 256 CUs, every slice should still stream 512
-    columns, and more rows make the partial sums themselves cost traffic (measured on the MI355X)."""
+    of the weight.  Up to 16 rows of x about 1024 small workgroups balance well over the 256 CUs; with more rows
+    a workgroup holds 33 or 67 KB of LDS and a CU two or four of them, and a CU with one workgroup more than
+    its neighbours ends late: at most one workgroup a CU then (MI355X, 64 rows, us for 2/4/8 slices: q/k/v
+    4,608 x 4,096 16.6/19.1/17.7, o 15.7/11.4/13.8, down 51.0/30.5/31.3; 32 rows: 12.5/13.6/13.2, 11.9/9.5/10.6,
+    37.8/24.6/25.7).  Every slice should still stream 512 columns, and more rows make the partial sums themselves
+    cost traffic."""
     wgs = -(-N // 64)
     cap = 16 if M <= 16 else (8 if M <= 32 else 4)
+    most = 1280 if M <= 16 else 256
     want = 1
-    while want * 2 <= cap and wgs * want * 2 <= 1280 and K // (want * 2) >= 512:
+    while want * 2 <= cap and wgs * want * 2 <= most and K // (want * 2) >= 512:
         want *= 2
     if want <= 1:
         return 1
