@@ -116,6 +116,10 @@ __global__ __launch_bounds__(NW * KW * 64) void gemm_skinny_kernel(const bf16_t*
                                                              float eps) {
     static_assert(MODE != 2 || SPW == 2, "gated output pairs a gate strip with an up strip");
     static_assert(KW == 1 || KW == 2, "one or two groups of wavefronts");
+    // whether the x operands are read from LDS a step ahead (below): it pays for 4 tiles of rows in the split and
+    // plain products (64 rows, us without/with: q/k/v 17.0/14.3, down 31.0/28.9, head 134/130, o 11.7/12.0), not
+    // for the gated product (53.8/55.3) and not for 2 tiles (q/k/v 12.5/11.4 but down 24.4/25.8)
+    constexpr bool AHEAD = MT >= 4 && MODE != 2;
     constexpr int NT = NW * KW * 64;
     constexpr int XV = MT * 16 * 64 / NT;     // 16-byte vectors of X a thread stages per chunk
     constexpr int BPW = 4 / KW;               // K-blocks of a chunk a wavefront multiplies
@@ -229,7 +233,7 @@ __global__ __launch_bounds__(NW * KW * 64) void gemm_skinny_kernel(const bf16_t*
         store_x(c, guard);
         __syncthreads();
         if (!guard || c + 1 < nchunk) load_x(c + 1);
-        if (MT < 4) {
+        if (!AHEAD) {
 #pragma unroll
             for (int jj = 0; jj < BPW; ++jj) {
                 const int j = kw * BPW + jj;
@@ -248,9 +252,8 @@ __global__ __launch_bounds__(NW * KW * 64) void gemm_skinny_kernel(const bf16_t*
             }
             return;
         }
-        // 4 tiles of rows: the x operands of a step (32 columns) are read from LDS a step ahead of the matrix
-        // instructions that use them; with one or two wavefronts a SIMD nothing else hides that latency
-        // (batch 64: 5.82 -> 5.76 ms a step; with 2 tiles the same lost 2%)
+        // the x operands of a step (32 columns) are read from LDS a step ahead of the matrix instructions that use
+        // them; with one or two wavefronts a SIMD nothing else hides that latency
         auto read_b = [&](int jj, int i, bf16x8_t (&b)[MT]) {
             const int j = kw * BPW + jj;
 #pragma unroll
