@@ -102,32 +102,24 @@ typedef float floatx4_t __attribute__((ext_vector_type(4)));
 #define SK_XC 512            // K columns of X staged at a time
 #define SK_XS (SK_XC + 8)    // LDS row stride in elements (16 bytes of padding)
 
-// KW (1 or 2): groups of NW wavefronts a workgroup.  With 2, both groups own the same strips and share the
-// staged X; of every chunk of 4 K-blocks the first group multiplies blocks 0, 1 and the second blocks 2, 3, and
-// the second hands its sums to the first through LDS at the end.  With 48 and more rows a wavefront is busy
-// issuing (4 tiles of rows an operand load) rather than waiting, and one wavefront a SIMD cannot hide that:
-// twice the wavefronts on the same X traffic.
-template <int MT, int MODE, typename OT, int SPW, int NW, bool TILED, int KW = 1>
-__global__ __launch_bounds__(NW * KW * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ X, long ldx,
+template <int MT, int MODE, typename OT, int SPW, int NW, bool TILED>
+__global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ X, long ldx,
                                                              const bf16_t* __restrict__ W, long ldw,
                                                              OT* __restrict__ Y, long ldy, int M, int N, int K, int KS,
                                                              float alpha, int I, long part_stride,
                                                              const float* __restrict__ row_ss, int ss_slices,
                                                              float eps) {
     static_assert(MODE != 2 || SPW == 2, "gated output pairs a gate strip with an up strip");
-    static_assert(KW == 1 || KW == 2, "one or two groups of wavefronts");
     // whether the x operands are read from LDS a step ahead (below): it pays for 4 tiles of rows in the split and
     // plain products (64 rows, us without/with: q/k/v 17.0/14.3, down 31.0/28.9, head 134/130, o 11.7/12.0), not
     // for the gated product (53.8/55.3) and not for 2 tiles (q/k/v 12.5/11.4 but down 24.4/25.8)
     constexpr bool AHEAD = MT >= 4 && MODE != 2;
-    constexpr int NT = NW * KW * 64;
+    constexpr int NT = NW * 64;
     constexpr int XV = MT * 16 * 64 / NT;     // 16-byte vectors of X a thread stages per chunk
-    constexpr int BPW = 4 / KW;               // K-blocks of a chunk a wavefront multiplies
+    constexpr int BPW = 4;                    // K-blocks of a chunk
     __shared__ __attribute__((aligned(16))) bf16_t xs[MT * 16 * SK_XS];
     const int tid = threadIdx.x, lane = tid & 63;
-    const int wave_wg = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int kw = KW > 1 ? wave_wg / NW : 0;              // which blocks of a chunk
-    const int wave = KW > 1 ? wave_wg - kw * NW : wave_wg; // which strips
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, g = lane >> 4;
     const int k_begin = blockIdx.y * KS;
     const int k_end = min(K, k_begin + KS);
@@ -164,7 +156,7 @@ __global__ __launch_bounds__(NW * KW * 64) void gemm_skinny_kernel(const bf16_t*
     // branch ends, and the weights asked for a chunk ahead would have to be there before the chunk's x is stored
     // (that wait cost the 64-row products a trip to memory a chunk).  Only the slice's last chunks (`guard`) ask
     // whether a block or a column exists.
-    bf16x8_t a[KW][BPW][SPW][4];              // [chunk parity][block of the wavefront]
+    bf16x8_t a[BPW][SPW][4];                  // a chunk's blocks of the wavefront's strips
     auto load_w = [&](int kb, bf16x8_t (&dst)[SPW][4], const bool guard) {
         if (guard && kb >= nkb) {             // uniform; the block is multiplied by zeros of x or not at all
 #pragma unroll
@@ -217,17 +209,13 @@ __global__ __launch_bounds__(NW * KW * 64) void gemm_skinny_kernel(const bf16_t*
     // weights than its later ones do (the compiler takes the stricter of the two for all)
     load_x(0);
 #pragma unroll
-    for (int p = 0; p < KW; ++p)
-#pragma unroll
-        for (int jj = 0; jj < BPW; ++jj)          // a block beyond a short slice repeats its last one
-            load_w(min(p * 4 + kw * BPW + jj, nkb - 1), a[p][jj], false);
+    for (int jj = 0; jj < BPW; ++jj) load_w(min(jj, nkb - 1), a[jj], false);   // beyond a short slice: its last block again
     // X may be x * w of a norm whose row factor is still to come (common.h: row_scales); the loop's first
     // barrier makes rs_s visible
     __shared__ float rs_s[MT * 16];
     if (row_ss) row_scales<NT, MT * 16>(row_ss, ss_slices, M, 1.0f / (float)K, eps, rs_s);
     const int nchunk = (nkb + 3) / 4, nfull = nkb / 4;       // chunks in all, chunks of 4 whole blocks
-    // a wavefront's weight blocks are asked for KW chunks (4 blocks of its own) ahead; the chunk's parity picks
-    // the registers, so the loops advance KW chunks a turn
+    // a block's weights are asked for again, a chunk ahead, as soon as the block is multiplied
     auto one_chunk = [&](int c, bf16x8_t (&ap)[BPW][SPW][4], const bool guard) {
         __syncthreads();
         store_x(c, guard);
@@ -236,7 +224,7 @@ __global__ __launch_bounds__(NW * KW * 64) void gemm_skinny_kernel(const bf16_t*
         if (!AHEAD) {
 #pragma unroll
             for (int jj = 0; jj < BPW; ++jj) {
-                const int j = kw * BPW + jj;
+                const int j = jj;
                 // consecutive matrix instructions go to different accumulators (tiles of rows, then strips)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
@@ -248,14 +236,14 @@ __global__ __launch_bounds__(NW * KW * 64) void gemm_skinny_kernel(const bf16_t*
                             acc[s][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ap[jj][s][i], b, acc[s][t], 0, 0, 0);
                     }
                 }
-                load_w((c + KW) * 4 + j, ap[jj], guard);
+                load_w((c + 1) * 4 + j, ap[jj], guard);
             }
             return;
         }
         // the x operands of a step (32 columns) are read from LDS a step ahead of the matrix instructions that use
         // them; with one or two wavefronts a SIMD nothing else hides that latency
         auto read_b = [&](int jj, int i, bf16x8_t (&b)[MT]) {
-            const int j = kw * BPW + jj;
+            const int j = jj;
 #pragma unroll
             for (int t = 0; t < MT; ++t) b[t] = *(const bf16x8_t*)(xs + (t * 16 + r) * SK_XS + j * 128 + g * 8 + i * 32);
         };
@@ -263,7 +251,7 @@ __global__ __launch_bounds__(NW * KW * 64) void gemm_skinny_kernel(const bf16_t*
         read_b(0, 0, bq[0]);
 #pragma unroll
         for (int jj = 0; jj < BPW; ++jj) {
-            const int j = kw * BPW + jj;
+            const int j = jj;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int step = jj * 4 + i;
@@ -274,7 +262,7 @@ __global__ __launch_bounds__(NW * KW * 64) void gemm_skinny_kernel(const bf16_t*
                     for (int s = 0; s < SPW; ++s)
                         acc[s][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ap[jj][s][i], bq[step & 1][t], acc[s][t], 0, 0, 0);
             }
-            load_w((c + KW) * 4 + j, ap[jj], guard);
+            load_w((c + 1) * 4 + j, ap[jj], guard);
         }
         if (!guard) {
             // the order the scheduler is to keep: x of the next chunk asked for, then step by step the next
@@ -292,38 +280,8 @@ __global__ __launch_bounds__(NW * KW * 64) void gemm_skinny_kernel(const bf16_t*
         }
     };
     int c0 = 0;
-    for (; c0 + 2 * KW <= nfull; c0 += KW) {          // these chunks, the next x and the blocks asked for are whole
-#pragma unroll
-        for (int p = 0; p < KW; ++p) one_chunk(c0 + p, a[p], false);
-    }
-    for (; c0 < nchunk; c0 += KW) {                   // the slice's end
-#pragma unroll
-        for (int p = 0; p < KW; ++p)
-            if (c0 + p < nchunk) one_chunk(c0 + p, a[p], true);
-    }
-    if (KW > 1) {
-        // the second group's sums go to the first through LDS (the staged X is no longer needed)
-        float* red = (float*)xs;
-        static_assert(KW == 1 || NW * SPW * MT * 4 * 64 * sizeof(float) <= sizeof(xs), "sums of a group fit into the X buffer");
-        __syncthreads();
-        if (kw == 1) {
-#pragma unroll
-            for (int s = 0; s < SPW; ++s)
-#pragma unroll
-                for (int t = 0; t < MT; ++t)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) red[(((wave * SPW + s) * MT + t) * 4 + i) * 64 + lane] = acc[s][t][i];
-        }
-        __syncthreads();
-        if (kw == 1) return;
-#pragma unroll
-        for (int s = 0; s < SPW; ++s)
-#pragma unroll
-            for (int t = 0; t < MT; ++t)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[s][t][i] += red[(((wave * SPW + s) * MT + t) * 4 + i) * 64 + lane];
-    }
-
+    for (; c0 + 2 <= nfull; ++c0) one_chunk(c0, a, false);   // this chunk, the next x and the blocks asked for are whole
+    for (; c0 < nchunk; ++c0) one_chunk(c0, a, true);        // the slice's end
     // lane (r, g) of tile t holds token t*16 + r, rows 4g .. 4g+3 of each strip
     OT* Yp = Y + (MODE == 1 ? (long)blockIdx.y * part_stride : 0);
 #pragma unroll
@@ -353,14 +311,16 @@ __global__ __launch_bounds__(NW * KW * 64) void gemm_skinny_kernel(const bf16_t*
 }
 
 // out_mode: 0 = Y[m,N] in out_dtype; 1 = float partial sums Y[ksplit][m][N]; 2 = gated (N = 2*I rows of W, Y[m,I] bf16)
-// variant: gated output 0 = 4 waves a workgroup, 1 = 2 waves; 4 = two groups of 4 waves (33..64 rows, any mode)
 // row_ss (or null): X is x * w of a norm cut by columns, whose sums of squares [M][ss_slices] these are (a
 // slice for every 64 columns after add_norm_columns, for every 16 after proj_add_norm); the output is multiplied
-// by rsqrt(sum of the row's slices / K + eps) row by row
-extern "C" const char* cpmcu_gemm_skinny_v(const void* X, long ldx, const void* W, long ldw, void* Y, long ldy,
-                                           int out_dtype, int out_mode, int M, int N, int K, int ksplit, float alpha,
-                                           int variant, int tiled, const float* row_ss, int ss_slices,
-                                           float eps, hipStream_t stream) {
+// by rsqrt(sum of the row's slices / K + eps) row by row.
+// Workgroups that measured best on the MI355X: 4 wavefronts of one strip each (more, smaller workgroups balance
+// better over 256 CUs); for the gated output 2 wavefronts of a gate and an up strip each at every number of rows
+// (32,768 x 4,096, us with 4 wavefronts / 2 / two groups of 4 that share the staged x: 17 rows 50.9/46.5/52.9,
+// 32 rows 49.5/46.1/52.2, 64 rows 51.9/49.5/52.8).
+extern "C" const char* cpmcu_gemm_skinny(const void* X, long ldx, const void* W, long ldw, void* Y, long ldy,
+                                         int out_dtype, int out_mode, int M, int N, int K, int ksplit, float alpha,
+                                         int tiled, const float* row_ss, int ss_slices, float eps, hipStream_t stream) {
     CPMCU_REQUIRE(M > 0 && M <= 64, "gemm_skinny: %d rows (1..64 are taken; more rows belong to the tiled product)", M);
     CPMCU_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "gemm_skinny: K=%d must be a positive multiple of 8 (N=%d)", K, N);
     CPMCU_REQUIRE(ldx % 8 == 0 && ldx >= K && (tiled || (ldw % 8 == 0 && ldw >= K)),
@@ -377,56 +337,32 @@ extern "C" const char* cpmcu_gemm_skinny_v(const void* X, long ldx, const void* 
     const int MT = (M + 15) / 16 == 3 ? 4 : (M + 15) / 16;
     const int I = N / 2;
     const long part_stride = (long)M * ldy;
-#define LAUNCH(MTv, MODEv, OT, SPW, NW, KWv)                                                                      \
+#define LAUNCH(MTv, MODEv, OT, SPW, NW)                                                                           \
     do {                                                                                                          \
         const int rows_wg = (MODEv == 2) ? NW * 16 : NW * SPW * 16;                                               \
         dim3 grid(((MODEv == 2 ? I : N) + rows_wg - 1) / rows_wg, ksplit);                                        \
         if (tiled)                                                                                                \
-            gemm_skinny_kernel<MTv, MODEv, OT, SPW, NW, true, KWv><<<grid, NW * KWv * 64, 0, stream>>>(    \
+            gemm_skinny_kernel<MTv, MODEv, OT, SPW, NW, true><<<grid, NW * 64, 0, stream>>>(                      \
                 (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (OT*)Y, ldy, M, N, K, KS, alpha, I, part_stride,    \
                 row_ss, ss_slices, eps);                                                                          \
         else                                                                                                      \
-            gemm_skinny_kernel<MTv, MODEv, OT, SPW, NW, false, KWv><<<grid, NW * KWv * 64, 0, stream>>>(   \
+            gemm_skinny_kernel<MTv, MODEv, OT, SPW, NW, false><<<grid, NW * 64, 0, stream>>>(                     \
                 (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (OT*)Y, ldy, M, N, K, KS, alpha, I, part_stride,    \
                 row_ss, ss_slices, eps);                                                                          \
     } while (0)
-// shapes that measured best: one strip a wave in workgroups of 4 waves; gated output in workgroups of
-// 2 waves up to 16 rows of X (variant 1), of 4 waves above (variant 0)
-#define BY_VAR(MTv, MODEv, OT)                                  \
-    do {                                                        \
-        if (MODEv == 2) {                                       \
-            if (variant == 1) LAUNCH(MTv, MODEv, OT, 2, 2, 1);  \
-            else if (variant == 4 && MTv == 4) LAUNCH(4, MODEv, OT, 2, 4, 2); \
-            else LAUNCH(MTv, MODEv, OT, 2, 4, 1);               \
-        } else if (variant == 4 && MTv == 4) LAUNCH(4, (MODEv == 2 ? 0 : MODEv), OT, 1, 4, 2); \
-        else LAUNCH(MTv, (MODEv == 2 ? 0 : MODEv), OT, 1, 4, 1); \
+#define BY_MT(MODEv, OT, SPW, NW)                     \
+    do {                                              \
+        if (MT == 1) LAUNCH(1, MODEv, OT, SPW, NW);   \
+        else if (MT == 2) LAUNCH(2, MODEv, OT, SPW, NW); \
+        else LAUNCH(4, MODEv, OT, SPW, NW);           \
     } while (0)
-#define BY_MT(MODEv, OT)                         \
-    do {                                         \
-        if (MT == 1) BY_VAR(1, MODEv, OT);       \
-        else if (MT == 2) BY_VAR(2, MODEv, OT);  \
-        else BY_VAR(4, MODEv, OT);               \
-    } while (0)
-    if (out_mode == 0 && out_dtype == CPMCU_F32) BY_MT(0, float);
-    else if (out_mode == 0 && out_dtype == CPMCU_BF16) BY_MT(0, bf16_t);
-    else if (out_mode == 1) BY_MT(1, float);
-    else if (out_mode == 2) BY_MT(2, bf16_t);
+    if (out_mode == 0 && out_dtype == CPMCU_F32) BY_MT(0, float, 1, 4);
+    else if (out_mode == 0 && out_dtype == CPMCU_BF16) BY_MT(0, bf16_t, 1, 4);
+    else if (out_mode == 1) BY_MT(1, float, 1, 4);
+    else if (out_mode == 2) BY_MT(2, bf16_t, 2, 2);
     else CPMCU_FAIL("gemm_skinny: unknown output mode %d / dtype %d", out_mode, out_dtype);
 #undef BY_MT
-#undef BY_VAR
 #undef LAUNCH
     CPMCU_LAUNCH_CHECK("gemm_skinny");
     return nullptr;
-}
-
-// The variant that measured best on the MI355X for each shape: one strip a wave (more, smaller
-// workgroups balance better over 256 CUs); gated output with 2 waves a workgroup up to 16 rows, and with two
-// groups of 4 waves that share the staged X from 33 rows on (64 rows, 32,768 x 4,096: 54.4 against 59.9 us; the
-// split products gain nothing from it: down 33.1 against 34.0 us, o 15.0 against 13.8).
-extern "C" const char* cpmcu_gemm_skinny(const void* X, long ldx, const void* W, long ldw, void* Y, long ldy,
-                                         int out_dtype, int out_mode, int M, int N, int K, int ksplit, float alpha,
-                                         int tiled, const float* row_ss, int ss_slices, float eps, hipStream_t stream) {
-    const int variant = out_mode == 2 ? (M <= 16 ? 1 : (M > 32 ? 4 : 0)) : 2;
-    return cpmcu_gemm_skinny_v(X, ldx, W, ldw, Y, ldy, out_dtype, out_mode, M, N, K, ksplit, alpha, variant, tiled,
-                               row_ss, ss_slices, eps, stream);
 }
