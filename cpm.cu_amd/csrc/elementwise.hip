@@ -94,6 +94,11 @@ __global__ void add_rms_norm_kernel(float* __restrict__ x, const BT* __restrict_
 // The same with 4 columns a thread and 16-byte accesses (H a multiple of 4, float branch or none):
 // the decode steps' norms have few rows and up to 16 partial sums to add, so the row's work
 // is spread over up to 1024 threads.
+__device__ inline void store4(float* p, float a, float b, float c, float d) { *(float4*)p = make_float4(a, b, c, d); }
+__device__ inline void store4(bf16_t* p, float a, float b, float c, float d) {
+    const bf16_t o0 = f32_to_bf16(a), o1 = f32_to_bf16(b), o2 = f32_to_bf16(c), o3 = f32_to_bf16(d);
+    *(uint2*)p = make_uint2((uint32_t)o0.v | ((uint32_t)o1.v << 16), (uint32_t)o2.v | ((uint32_t)o3.v << 16));
+}
 __device__ inline float4 load4(const float* p) { return *(const float4*)p; }
 __device__ inline float4 load4(const bf16_t* p) {
     const uint2 u = *(const uint2*)p;
@@ -149,10 +154,7 @@ __global__ __launch_bounds__(1024) void add_rms_norm_vec4_kernel(float* __restri
     };
     auto emit = [&](int c, float4 v, float rs) {
         const float4 wv = *(const float4*)(w + 4 * c);
-        o[4 * c + 0] = from_f32<OT>(v.x * rs * wv.x);
-        o[4 * c + 1] = from_f32<OT>(v.y * rs * wv.y);
-        o[4 * c + 2] = from_f32<OT>(v.z * rs * wv.z);
-        o[4 * c + 3] = from_f32<OT>(v.w * rs * wv.w);
+        store4(o + 4 * c, v.x * rs * wv.x, v.y * rs * wv.y, v.z * rs * wv.z, v.w * rs * wv.w);   // one store of 16 or 8 bytes
     };
     if (H4 <= (int)blockDim.x) {
         // the whole row fits the block: each thread keeps its 4 columns in registers between the two phases
@@ -209,7 +211,7 @@ extern "C" const char* cpmcu_add_rms_norm(float* x, const void* branch, int bran
     CPMCU_REQUIRE(n_out > 0 && H > 0, "add_rms_norm: empty shape rows=%d H=%d", n_out, H);
     CPMCU_REQUIRE(!branch || nparts >= 1, "add_rms_norm: nparts=%d", nparts);
     if (H % 4 == 0 && ((uintptr_t)x % 16 == 0) && (!branch || ((uintptr_t)branch % 16 == 0 && part_stride % 4 == 0)) &&
-        ((uintptr_t)w % 16 == 0) && (out_dtype == CPMCU_F32 || out_dtype == CPMCU_BF16) &&
+        ((uintptr_t)w % 16 == 0) && ((uintptr_t)out % 16 == 0) && (out_dtype == CPMCU_F32 || out_dtype == CPMCU_BF16) &&
         (branch_dtype == CPMCU_F32 || branch_dtype == CPMCU_BF16)) {
         const int h4 = H / 4;
         // many rows: smaller blocks keep more rows in flight on a CU; few rows: spread a row over many threads
