@@ -174,3 +174,25 @@ def test_minicpm4_yarn_installs_the_built_in_factors_for_head_size_128_only():
 def test_neutral_properties_of_a_configuration():
     cfg = MiniCPMConfig.from_dict(tiny.tiny_b())
     assert cfg.vocabulary_size == 1000 and cfg.longest_sequence == 512 and tuple(cfg.stop_token_ids) == (1, 7)
+
+
+def test_share_and_slice_heuristics_stay_within_what_the_kernels_take():
+    """The host-side choices of split-KV shares and K slices: at most 32 shares of at least 128 keys, about one
+    workgroup a CU; slices of whole 128-column blocks that cover K."""
+    from cpmcu_amd import ops
+    for n in (1, 2, 3, 8, 16, 24, 64, 200, 257):
+        for nkv, group in ((1, 4), (2, 16), (8, 5), (2, 40)):
+            for keys in (1, 100, 128, 700, 4096, 8192, 33000, 140000):
+                s = ops.attention_splits(n, nkv, group, keys)
+                assert 1 <= s <= 32
+                assert s == 1 or keys // s >= 128
+                groups = n * nkv * -(-group // 16)
+                assert s == 1 or s * groups <= 256 or (groups >= 128 and s == 2)
+    for M in (1, 16, 17, 32, 33, 64):
+        for N, K in ((4096, 4096), (4608, 4096), (4096, 16384), (100, 104), (73448, 4096), (1024, 896)):
+            S = ops.skinny_split(M, N, K)
+            assert S >= 1
+            if S > 1:
+                ks = -(-(-(-K // S)) // 128) * 128
+                assert -(-K // ks) == S and ks >= 512
+                assert M <= 16 or -(-N // 64) * S <= 256
