@@ -92,11 +92,11 @@ def edge_keys(L, splits, nw):
     (9000, 8, 2, 32, ((1, 1), (1, 4), (16, 4), (32, 4), (16, 1))),
     (20000, 4, 1, 32, ((1, 1), (1, 4), (16, 4), (32, 4), (32, 1))),
     (4100, 32, 2, 128, ((8, 4), (16, 4))),
-    (16400, 32, 2, 128, ((1, 4), (8, 4), (16, 4), (32, 4))),
-    (33000, 32, 2, 128, ((16, 4), (32, 4), (8, 1))),
+    (16400, 32, 2, 128, ((1, 4), (8, 4), (16, 4), (32, 4), (48, 4))),
+    (33000, 32, 2, 128, ((16, 4), (32, 4), (8, 1), (64, 4))),
 ])
 def test_decode_attention_over_long_contexts(L, nh, nkv, hd, shapes):
-    """One and two tokens over thousands of keys: 1 to 32 shares, 1 and 4 wavefronts a workgroup, wavefronts
+    """One and two tokens over thousands of keys: 1 to 64 shares (every form of the merge kernel), 1 and 4 wavefronts a workgroup, wavefronts
     with more than 64 and more than 128 chunks; random queries against the float64 reference, then one
     outstanding key at a time at the edges of the walk."""
     from cpmcu_amd import ops
