@@ -1,10 +1,16 @@
 """Command-line options, with the reference's names and meanings where it has them
 (cpmcu/common/args.py:22-131): every option has a --kebab and a --snake spelling and
 booleans accept true/false values.  Options of speculative decoding and servers are absent.
+
+The options that belong to an architecture (the reference's sparse-attention group, --minicpm4-yarn, the
+names --model-type accepts) are not spelled here: every registered architecture declares its own
+(registry.Flag), and the parser offers what is declared.
 """
 from __future__ import annotations
 
 import argparse
+
+from .registry import declared_flags, declared_model_types
 
 
 def str2bool(v):
@@ -25,12 +31,12 @@ def add_model_config_args(parser: argparse.ArgumentParser):
     g = parser.add_argument_group("Model Configuration")
     g.add_argument("--model-path", "--model_path", "--model", type=str, default=None,
                    help="Folder with config.json and safetensors weights (or, with --random-weights, where to write them)")
-    g.add_argument("--model-type", "--model_type", type=str, default="auto", choices=["auto", "minicpm", "minicpm4"],
-                   help="Model type (default: auto-detect); minicpm4 turns block-sparse attention on")
+    g.add_argument("--model-type", "--model_type", type=str, default="auto",
+                   choices=["auto"] + declared_model_types(),
+                   help="Model type (default: auto: config.json decides); a name sets the flags its architecture "
+                        "gives it")
     g.add_argument("--dtype", type=str, default="bfloat16", choices=["bfloat16", "float32"],
                    help="Model dtype (default: bfloat16; float32 runs everything in true 32-bit)")
-    _flag(g, "--minicpm4-yarn", "--minicpm4_yarn", default=False,
-          help="Replace the LongRoPE factors by the built-in long-context list (default: False)")
     g.add_argument("--random-weights", "--random_weights", action="store_true",
                    help="Write a model folder with random weights from --config and --seed, then run on it")
     g.add_argument("--config", type=str, default=None, help="config.json to draw random weights for")
@@ -50,17 +56,17 @@ def add_model_config_args(parser: argparse.ArgumentParser):
                    help="Longest sequence (default: the model's max_position_embeddings)")
     _flag(s, "--perf", default=False, help="Print the timer summary at the end (default: False)")
 
-    a = parser.add_argument_group("Sparse Attention")
-    a.add_argument("--sink-window-size", "--sink_window_size", type=int, default=None,
-                   help="Initial blocks always attended to (default: sparse_config.init_blocks)")
-    a.add_argument("--block-window-size", "--block_window_size", type=int, default=None,
-                   help="Trailing window in blocks (default: sparse_config.window_size / block_size)")
-    a.add_argument("--sparse-topk-k", "--sparse_topk_k", type=int, default=None,
-                   help="Blocks chosen by score (default: sparse_config.topk)")
-    a.add_argument("--sparse-switch", "--sparse_switch", type=int, default=None,
-                   help="Context up to which attention stays dense (default: sparse_config.dense_len)")
-    _flag(a, "--use-compress-lse", "--use_compress_lse", default=False,
-          help="Not supported (scores are normalised over the keys they come from); must stay False")
+    # what the registered architectures declare; not given = None = the architecture's own default
+    groups = {"Model Configuration": g, "System Configuration": s}
+    for f in declared_flags():
+        grp = groups.get(f.group)
+        if grp is None:
+            grp = groups[f.group] = parser.add_argument_group(f.group)
+        names = sorted({"--" + f.name.replace("_", "-"), "--" + f.name})
+        if f.kind is bool:
+            _flag(grp, *names, default=None, help=f.help)
+        else:
+            grp.add_argument(*names, dest=f.name, type=f.kind, default=None, help=f.help)
 
 
 def create_cli_parser() -> argparse.ArgumentParser:

@@ -108,6 +108,7 @@ def run_generation(args):
     from . import get_architecture
     from .config.base import architecture_name, read_config_json
     from .llm import LLM
+    from .registry import declared_flags
 
     model_path = args.model_path
     if args.random_weights:
@@ -125,17 +126,23 @@ def run_generation(args):
     if not os.path.isdir(model_path):
         raise FileNotFoundError(f"model folder not found: {model_path} (there is no download: give a local folder)")
 
-    # 'minicpm4' switches the block-sparse attention on, 'minicpm' (and 'llama') off (cpmcu/common/utils.py:123);
-    # 'auto' leaves it to the architecture, which turns it on iff its configuration describes it
-    apply_sparse = {"minicpm4": True, "auto": None}.get(args.model_type, False)
+    # the architecture that config.json names declares its flags and what a --model-type name sets
+    arch = get_architecture(architecture_name(read_config_json(model_path)))
+    flags = {f.name: getattr(args, f.name, None) for f in arch.flags}
+    if args.model_type != "auto":
+        if args.model_type not in arch.model_types:
+            raise ValueError(f"--model-type {args.model_type}: architecture '{arch.name}' knows "
+                             f"{sorted(arch.model_types) or 'no model types'} (and 'auto')")
+        for k, v in arch.model_types[args.model_type].items():
+            if flags.get(k) is None:
+                flags[k] = v
+    foreign = [f.name for f in declared_flags() if f.name not in flags and getattr(args, f.name, None) is not None]
+    if foreign:
+        raise ValueError(f"architecture '{arch.name}' has no flags {foreign}")
     tokenizer = load_tokenizer(model_path)
     llm = LLM(model_path, memory_limit=args.memory_limit, chunk_length=args.chunk_length, dtype=args.dtype,
-              cuda_graph=args.hip_graph, apply_sparse=apply_sparse,
-              sink_window_size=args.sink_window_size, block_window_size=args.block_window_size,
-              sparse_topk_k=args.sparse_topk_k, sparse_switch=args.sparse_switch,
-              use_compress_lse=args.use_compress_lse, temperature=args.temperature, random_seed=args.random_seed,
-              max_tokens=args.max_tokens, max_seq_len=args.max_seq_len, max_batch=args.batch,
-              minicpm4_yarn=args.minicpm4_yarn)
+              cuda_graph=args.hip_graph, temperature=args.temperature, random_seed=args.random_seed,
+              max_tokens=args.max_tokens, max_seq_len=args.max_seq_len, max_batch=args.batch, **flags)
     llm.tokenizer = tokenizer
     llm.perf.enabled = bool(args.perf)
     prompts = make_prompts(args, tokenizer, llm.config.vocabulary_size)

@@ -30,39 +30,33 @@ class LLM:
                  chunk_length: int = 1024,
                  dtype=None,
                  cuda_graph: bool = False,
-                 apply_sparse: Optional[bool] = False,
-                 sink_window_size: Optional[int] = None,
-                 block_window_size: Optional[int] = None,
-                 sparse_topk_k: Optional[int] = None,
-                 sparse_switch: Optional[int] = None,
-                 use_compress_lse: bool = False,
                  temperature: float = 0.0,
                  random_seed: Optional[int] = None,
                  max_tokens: Optional[int] = None,
                  max_seq_len: Optional[int] = None,
                  max_batch: Optional[int] = None,
                  device: str = "cuda:0",
-                 minicpm4_yarn: bool = False):
+                 **model_flags):
         self.path = path
         raw = read_config_json(path)
         self.arch = get_architecture(architecture_name(raw))
         self.config = self.arch.config_class.from_dict(raw)
         if dtype is None:
             dtype = raw.get("torch_dtype", "bfloat16")
+            if dtype == "float16":
+                dtype = "bfloat16"     # a float16 checkpoint is served in bfloat16 (the loader converts it)
         if dtype in (torch.float16, "float16"):
             raise ValueError("float16 is not built into this engine: use bfloat16 (serving) or float32 (exact)")
         if dtype not in _DTYPE_NAMES:
             raise ValueError(f"Unsupported dtype: {dtype}")
         self.dtype = _DTYPE_NAMES[dtype]
-        # The reference's model flags (cpmcu/common/args.py:38-40, 72-83) go to the architecture, which knows
-        # what they mean for its configuration and which options of its model they switch; an architecture that
-        # has no such flags refuses any that is set.
-        flags = {"apply_sparse": apply_sparse, "sink_window_size": sink_window_size,
-                 "block_window_size": block_window_size, "sparse_topk_k": sparse_topk_k,
-                 "sparse_switch": sparse_switch, "use_compress_lse": use_compress_lse or None,
-                 "minicpm4_yarn": minicpm4_yarn or None}
-        self.config, self.model_options = self.arch.with_flags(self.config, flags)
-        self.apply_sparse = apply_sparse
+        # The reference's model flags (apply_sparse, sink_window_size, block_window_size, sparse_topk_k,
+        # sparse_switch, use_compress_lse, minicpm4_yarn: cpmcu/llm.py:31-36, cpmcu/common/args.py:38-40, 72-83)
+        # are keywords that this class does not spell: they go to the architecture that config.json names, which
+        # declares the flags it knows, says what they mean for its configuration and which options of its model
+        # they switch, and refuses the others.  A flag that is None or not given leaves the architecture's default.
+        self.model_flags = dict(model_flags)
+        self.config, self.model_options = self.arch.with_flags(self.config, self.model_flags)
         self.memory_limit = memory_limit
         self.chunk_length = chunk_length
         self.cuda_graph = cuda_graph

@@ -16,7 +16,7 @@ import torch
 
 from ..config.minicpm import MiniCPMConfig
 from ..parts import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, LMHead, PartSpec, TokenEmbedding)
-from ..registry import Architecture, register_architecture
+from ..registry import Architecture, Flag, register_architecture
 from .decoder import DecoderModel
 
 ARCHITECTURE = "MiniCPMForCausalLM"
@@ -118,9 +118,15 @@ def apply_flags(cfg: MiniCPMConfig, flags: Dict[str, object]) -> Tuple[MiniCPMCo
     if "apply_sparse" in flags:
         options["sparse"] = bool(flags["apply_sparse"])
     sc = cfg.sparse_config
-    if flags.get("apply_sparse"):
-        if sc is None:
-            raise ValueError("apply_sparse: config.json has no sparse_config (kernel_size, kernel_stride, block_size ...)")
+    # absent (the command line's model type 'auto'): block-sparse attention is on iff config.json describes it
+    sparse_on = bool(flags["apply_sparse"]) if "apply_sparse" in flags else sc is not None
+    if flags.get("apply_sparse") and sc is None:
+        raise ValueError("apply_sparse: config.json has no sparse_config (kernel_size, kernel_stride, block_size ...)")
+    over_flags = [k for k in ("sink_window_size", "block_window_size", "sparse_topk_k", "sparse_switch") if k in flags]
+    if over_flags and not sparse_on:
+        raise ValueError(f"{over_flags} change the block-sparse attention, which is off: "
+                         + ("apply_sparse is false" if sc is not None else "config.json has no sparse_config"))
+    if over_flags:
         over = {}
         if "sink_window_size" in flags:
             over["init_blocks"] = flags["sink_window_size"]
@@ -130,8 +136,7 @@ def apply_flags(cfg: MiniCPMConfig, flags: Dict[str, object]) -> Tuple[MiniCPMCo
             over["topk"] = flags["sparse_topk_k"]
         if "sparse_switch" in flags:
             over["dense_len"] = flags["sparse_switch"]
-        if over:
-            cfg = dataclasses.replace(cfg, sparse_config=SparseConfig.from_dict({**sc.to_dict(), **over}))
+        cfg = dataclasses.replace(cfg, sparse_config=SparseConfig.from_dict({**sc.to_dict(), **over}))
     if flags.get("minicpm4_yarn"):
         from ..config.minicpm4_yarn import MINICPM4_YARN_FACTORS
         if cfg.head_dim != 2 * len(MINICPM4_YARN_FACTORS):
@@ -147,4 +152,19 @@ def apply_flags(cfg: MiniCPMConfig, flags: Dict[str, object]) -> Tuple[MiniCPMCo
 register_architecture(Architecture(
     name=ARCHITECTURE, config_class=MiniCPMConfig, build=build, options={"tied": None, "sparse": True},
     split_fused=split_fused, ignore_tensor=ignore_tensor, checkpoint_options=checkpoint_options,
-    apply_flags=apply_flags))
+    apply_flags=apply_flags,
+    flags=(
+        Flag("minicpm4_yarn", bool, "Replace the LongRoPE factors by the built-in long-context list (default: False)"),
+        Flag("apply_sparse", bool, "Block-sparse attention on or off (default: on iff config.json has sparse_config)",
+             "Sparse Attention"),
+        Flag("sink_window_size", int, "Initial blocks always attended to (default: sparse_config.init_blocks)",
+             "Sparse Attention"),
+        Flag("block_window_size", int, "Trailing window in blocks (default: sparse_config.window_size / block_size)",
+             "Sparse Attention"),
+        Flag("sparse_topk_k", int, "Blocks chosen by score (default: sparse_config.topk)", "Sparse Attention"),
+        Flag("sparse_switch", int, "Context up to which attention stays dense (default: sparse_config.dense_len)",
+             "Sparse Attention"),
+        Flag("use_compress_lse", bool, "Not supported (scores are normalised over the keys they come from); must "
+             "stay False", "Sparse Attention")),
+    # 'minicpm4' switches the block-sparse attention on, 'minicpm' off (cpmcu/common/utils.py:123)
+    model_types={"minicpm4": {"apply_sparse": True}, "minicpm": {"apply_sparse": False}}))

@@ -10,7 +10,18 @@ an architecture's own file names its options or its configuration's fields.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Callable, Dict, Iterable, List, Mapping, Optional
+from typing import Any, Callable, Dict, Iterable, List, Mapping, Optional, Sequence
+
+
+@dataclass(frozen=True)
+class Flag:
+    """A front-end flag that an architecture declares: ``name`` is the keyword of ``LLM(...)`` and, with dashes
+    or underscores, the command-line option; ``kind`` is int, float, str or bool (a boolean takes true/false
+    values on the command line)."""
+    name: str
+    kind: type = int
+    help: str = ""
+    group: str = "Model Configuration"
 
 
 @dataclass
@@ -27,6 +38,10 @@ class Architecture:
     # (config, flags) -> (config, options): the front end's flags (the reference's command-line and ``LLM``
     # argument names) as this architecture understands them; flags it does not know must be refused
     apply_flags: Optional[Callable] = None
+    # the flags ``apply_flags`` knows, as the front ends should offer them (command-line options, keywords of
+    # ``LLM``); and the command line's --model-type names with the flags each one sets
+    flags: Sequence[Flag] = ()
+    model_types: Mapping[str, Mapping[str, Any]] = field(default_factory=dict)
 
     def build_model(self, config, options: Optional[Mapping[str, Any]] = None,
                     checkpoint_names: Optional[Iterable[str]] = None):
@@ -74,3 +89,18 @@ def get_architecture(name: str) -> Architecture:
 
 def architectures() -> List[str]:
     return sorted(_ARCHITECTURES)
+
+
+def declared_flags() -> List[Flag]:
+    """Every flag that a registered architecture declares, once by name (the first declaration's help stands)."""
+    seen: Dict[str, Flag] = {}
+    for name in sorted(_ARCHITECTURES):
+        for f in _ARCHITECTURES[name].flags:
+            if f.name in seen and seen[f.name].kind is not f.kind:
+                raise ValueError(f"flag '{f.name}' is declared as {seen[f.name].kind.__name__} and as {f.kind.__name__}")
+            seen.setdefault(f.name, f)
+    return list(seen.values())
+
+
+def declared_model_types() -> List[str]:
+    return sorted({t for a in _ARCHITECTURES.values() for t in a.model_types})

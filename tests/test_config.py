@@ -133,12 +133,21 @@ def test_head_sizes_the_kernels_do_not_take_are_refused_when_the_model_is_built(
 def test_front_end_flags_go_through_the_architecture():
     arch = get_architecture("MiniCPMForCausalLM")
     cfg = MiniCPMConfig.from_dict(tiny.tiny_b())
-    same, opts = arch.with_flags(cfg, {"apply_sparse": False, "sparse_topk_k": 9})
+    same, opts = arch.with_flags(cfg, {"apply_sparse": False})
     assert same == cfg and opts == {"sparse": False}
+    with pytest.raises(ValueError, match="sparse_topk_k.*apply_sparse is false"):
+        arch.with_flags(cfg, {"apply_sparse": False, "sparse_topk_k": 9})
+    with pytest.raises(ValueError, match="sparse_switch.*no sparse_config"):
+        arch.with_flags(MiniCPMConfig.from_dict(tiny.tiny_a()), {"sparse_switch": 9})
     new, opts = arch.with_flags(cfg, {"apply_sparse": True, "sparse_topk_k": 9, "block_window_size": 3, "sink_window_size": 2,
                                       "sparse_switch": 100})
     sc = new.sparse_config
     assert opts == {"sparse": True} and (sc.topk, sc.window_size, sc.init_blocks, sc.dense_len) == (9, 48, 2, 100)
+    # the command line's model type 'auto' gives no apply_sparse at all: the configuration decides, and the
+    # overrides still arrive
+    new, opts = arch.with_flags(cfg, {"apply_sparse": None, "sparse_topk_k": 3, "sparse_switch": 5})
+    assert opts == {} and (new.sparse_config.topk, new.sparse_config.dense_len) == (3, 5)
+    assert new.sparse_config.window_size == cfg.sparse_config.window_size
     with pytest.raises(ValueError, match="use_compress_lse"):
         arch.with_flags(cfg, {"use_compress_lse": True})
     with pytest.raises(ValueError, match="no sparse_config"):
@@ -196,3 +205,78 @@ def test_share_and_slice_heuristics_stay_within_what_the_kernels_take():
                 ks = -(-(-(-K // S)) // 128) * 128
                 assert -(-K // ks) == S and ks >= 512
                 assert M <= 16 or -(-N // 64) * S <= 256
+
+
+def test_model_type_auto_keeps_the_sparse_overrides(model_dirs):
+    """The command line's default model type gives no apply_sparse; the sparse options it does give must still
+    reach the configuration of a model whose config.json describes the block-sparse attention."""
+    from cpmcu_amd.args import parse_cli_args
+    from cpmcu_amd.llm import LLM
+    args = parse_cli_args(["--model-path", model_dirs["B"], "--sparse-topk-k", "3", "--sparse_switch", "5"])
+    assert args.model_type == "auto" and args.apply_sparse is None and args.sparse_topk_k == 3
+    arch = get_architecture("MiniCPMForCausalLM")
+    flags = {f.name: getattr(args, f.name) for f in arch.flags}
+    llm = LLM(model_dirs["B"], **flags)
+    assert (llm.config.sparse_config.topk, llm.config.sparse_config.dense_len) == (3, 5)
+    assert llm.model_options == {}
+    assert type(arch.build_model(llm.config, llm.model_options).layers[0].mixer).__name__ == "InfLLMv2Attention"
+    # a model without sparse_config refuses them instead of dropping them
+    with pytest.raises(ValueError, match="no sparse_config"):
+        LLM(model_dirs["A"], sparse_topk_k=3)
+    # a float16 checkpoint is served in bfloat16 unless a dtype is asked for; float16 itself is refused
+    assert LLM(model_dirs["A"]).dtype == "bfloat16"
+    with pytest.raises(ValueError, match="float16"):
+        LLM(model_dirs["A"], dtype="float16")
+
+
+def test_an_architecture_brings_its_own_front_end_flags(tmp_path):
+    """Nothing in args.py, cli.py or llm.py spells a model flag: an architecture registered here declares one and
+    a model type, and the parser, the command line's flag hand-over and ``LLM`` know them."""
+    import json
+    from dataclasses import dataclass, replace
+
+    from cpmcu_amd.args import create_cli_parser
+    from cpmcu_amd.config.base import ModelConfig
+    from cpmcu_amd.llm import LLM
+    from cpmcu_amd.registry import Architecture, Flag, register_architecture, unregister_architecture
+
+    @dataclass(frozen=True)
+    class FlagToyConfig(ModelConfig):
+        depth: int = 1
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls("FlagToyForTests", depth=int(raw.get("depth", 1)))
+
+        def to_dict(self):
+            return {"architectures": [self.architecture], "depth": self.depth}
+
+        vocabulary_size = 10
+
+    def apply_flags(cfg, flags):
+        assert set(flags) <= {"toy_depth", "toy_fast"}
+        if "toy_depth" in flags:
+            cfg = replace(cfg, depth=flags["toy_depth"])
+        return cfg, ({"fast": flags["toy_fast"]} if "toy_fast" in flags else {})
+
+    arch = Architecture("FlagToyForTests", FlagToyConfig, build=lambda cfg, fast=False: None, options={"fast": False},
+                        apply_flags=apply_flags,
+                        flags=(Flag("toy_depth", int, "layers to run", "Toy"), Flag("toy_fast", bool, "fast path", "Toy")),
+                        model_types={"toyfast": {"toy_fast": True}})
+    register_architecture(arch)
+    try:
+        p = create_cli_parser()
+        a = p.parse_args(["--toy-depth", "3", "--model-type", "toyfast", "--toy_fast", "false"])
+        assert a.toy_depth == 3 and a.toy_fast is False and a.model_type == "toyfast"
+        assert a.sparse_topk_k is None                     # MiniCPM4's own are still there
+        d = tmp_path / "m"
+        d.mkdir()
+        (d / "config.json").write_text(json.dumps({"architectures": ["FlagToyForTests"], "depth": 2}))
+        llm = LLM(str(d), toy_depth=5, toy_fast=True)
+        assert llm.config.depth == 5 and llm.model_options == {"fast": True}
+        with pytest.raises(AssertionError):
+            LLM(str(d), sparse_topk_k=2)                   # not this architecture's flag
+    finally:
+        unregister_architecture("FlagToyForTests")
+    with pytest.raises(SystemExit):
+        create_cli_parser().parse_args(["--toy-depth", "3"])
