@@ -95,13 +95,78 @@ class _Group:
         return sum(1 for p in self.pages[slot] if p >= 0)
 
 
+def _element_size(dtype: torch.dtype) -> int:
+    return torch.empty((), dtype=dtype).element_size()
+
+
+def _window_pages(window: int, step: int, page_size: int) -> int:
+    """The most pages a sequence holds in a group that keeps a trailing window, when it grows by at most
+    ``step`` tokens at once: the step's first query still reads window - 1 tokens back."""
+    return (step + window - 2) // page_size + 2
+
+
+def _pool_pages(needs: CacheNeeds, n_pages: int, max_slots: int, max_seq_len: int, step: int, page_size: int) -> int:
+    """Pages of a group's pool: a group that keeps every token gets one for every page of tokens the cache
+    holds; a group that keeps a window never holds more than its window's pages for every slot."""
+    if needs.window is None:
+        return n_pages
+    per_slot = min(-(-max_seq_len // page_size), _window_pages(needs.window, step, page_size))
+    return min(n_pages, max_slots * per_slot)
+
+
 class SequenceCache:
     """Slots, pages and per-slot state for all cache entries of a model."""
 
+    @staticmethod
+    def plan_bytes(needs: Sequence[CacheNeeds], max_tokens: int, max_slots: int, max_seq_len: int,
+                   page_size: int, dtype: torch.dtype, max_step_tokens: Optional[int] = None) -> int:
+        """Device bytes of a cache built with these arguments (pools, per-slot state, page tables), without
+        building it: what an engine checks against its memory limit beforehand."""
+        n_pages = -(-max_tokens // page_size)
+        seq_pages = -(-max_seq_len // page_size)
+        step = max_step_tokens or max_seq_len
+        total = 0
+        seen = set()
+        for n in needs:
+            pool = _pool_pages(n, n_pages, max_slots, max_seq_len, step, page_size)
+            for _, st in n.streams:
+                total += pool * (page_size // st.every) * st.width * _element_size(st.dtype or dtype)
+            for _, st in n.state:
+                count = 1
+                for d in st.shape:
+                    count *= int(d)
+                total += max_slots * count * _element_size(st.dtype or dtype)
+            if n.group_key() not in seen:
+                seen.add(n.group_key())
+                total += max_slots * (seq_pages if n.window is not None else min(seq_pages, n_pages)) * 4
+        return total
+
+    @staticmethod
+    def tokens_for(needs: Sequence[CacheNeeds], budget_bytes: int, max_slots: int, max_seq_len: int,
+                   page_size: int, dtype: torch.dtype, max_step_tokens: Optional[int] = None) -> int:
+        """The most tokens (a whole number of pages, at most max_slots sequences of max_seq_len) whose cache fits
+        ``budget_bytes``; 0 if not even a page for every slot does."""
+        hi = max_slots * (-(-max_seq_len // page_size))
+
+        def fits(pages: int) -> bool:
+            return SequenceCache.plan_bytes(needs, pages * page_size, max_slots, max_seq_len, page_size, dtype,
+                                            max_step_tokens) <= budget_bytes
+        if not fits(max_slots):
+            return 0
+        lo = max_slots
+        while lo < hi:
+            mid = (lo + hi + 1) // 2
+            if fits(mid):
+                lo = mid
+            else:
+                hi = mid - 1
+        return lo * page_size
+
     def __init__(self, needs: List[CacheNeeds], max_tokens: int, max_slots: int, max_seq_len: int,
-                 page_size: int = 64, device="cpu", dtype=torch.float32):
+                 page_size: int = 64, device="cpu", dtype=torch.float32, max_step_tokens: Optional[int] = None):
         if page_size <= 0 or max_tokens <= 0 or max_slots <= 0 or max_seq_len <= 0:
             raise CacheError("cache sizes must be positive")
+        self.max_step_tokens = int(max_step_tokens or max_seq_len)
         self.page_size = page_size
         self.max_slots = max_slots
         self.max_seq_len = max_seq_len
@@ -120,11 +185,13 @@ class SequenceCache:
         self.entry_group = [0] * len(needs)
         for key, entries in by_key.items():
             width = seq_pages if needs[entries[0]].window is not None else self.table_width
-            g = _Group(needs[entries[0]], entries, self.n_pages, max_slots, width, page_size, self.device, dtype)
+            pool = _pool_pages(needs[entries[0]], self.n_pages, max_slots, max_seq_len, self.max_step_tokens, page_size)
+            g = _Group(needs[entries[0]], entries, pool, max_slots, width, page_size, self.device, dtype)
             for e in entries:
                 self.entry_group[e] = len(self.groups)
             self.groups.append(g)
         self._has_window = any(g.needs.window is not None for g in self.groups)
+        self.has_state = any(g.needs.state for g in self.groups)
         self.free_slots: List[int] = list(range(max_slots - 1, -1, -1))
         self.live: Dict[int, int] = {}        # slot -> tokens held
         self._views: Dict[int, CacheView] = {}
@@ -219,7 +286,7 @@ class SequenceCache:
             if g.needs.window is None:
                 out.append(full)
             else:
-                out.append(min(full, (step + g.needs.window - 2) // self.page_size + 2))
+                out.append(min(full, _window_pages(g.needs.window, step, self.page_size)))
         return out
 
     def capacity(self) -> List[int]:
@@ -270,12 +337,22 @@ class SequenceCache:
 
     def truncate(self, slot: int, length: int):
         """Forget the slot's tokens from ``length`` on (a step that failed after extend): their pages return
-        to the pools.  Pages that a windowed group gave back while the slot grew stay given back; no query at
-        or beyond ``length`` reads them."""
+        to the pools.  Pages that a windowed group gave back while the slot grew stay given back, so a group
+        that keeps a window can only go back to a length whose next query reads none of them (the start of the
+        slot's last extend always is one); a shorter length is refused and nothing changes."""
         have = self.length(slot)
         if not 0 <= length <= have:
             raise CacheError(f"slot {slot}: cannot truncate {have} tokens to {length}")
         n_pg = -(-length // self.page_size)
+        for gi, g in enumerate(self.groups):
+            if g.needs.window is None:
+                continue
+            pages = g.pages[slot]
+            gone = [pn for pn in range(self._first_kept(g, length), min(n_pg, len(pages))) if pages[pn] < 0]
+            if gone:
+                raise CacheError(f"slot {slot}: cannot truncate to {length} tokens: cache group {gi} keeps a window of "
+                                 f"{g.needs.window} tokens and has already given back page {gone[0]}, which the query "
+                                 f"at position {length} would read")
         for g in self.groups:
             pages = g.pages[slot]
             while len(pages) > n_pg:
@@ -283,6 +360,23 @@ class SequenceCache:
                 if p >= 0:
                     g.free_pages.append(p)
         self.live[slot] = length
+
+    # ---- fixed-size state ----
+    def snapshot_state(self, slots: Sequence[int]):
+        """Copies of the slots' fixed-size state (None when no entry has any): what restore_state puts back
+        after a forward pass that advanced the state and then failed."""
+        if not self.has_state:
+            return None
+        idx = torch.tensor(list(slots), dtype=torch.long).to(self.device)
+        return idx, [[(t, t.index_select(0, idx)) for t in g.state[e].values()] for g in self.groups for e in g.entries]
+
+    def restore_state(self, snapshot):
+        if snapshot is None:
+            return
+        idx, saved = snapshot
+        for entry in saved:
+            for t, rows in entry:
+                t.index_copy_(0, idx, rows)
 
     def extend_one(self, slot: int) -> int:
         """extend(slot, 1) for the decode loop: nothing but the length changes while the token fits the

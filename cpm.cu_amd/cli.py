@@ -153,13 +153,15 @@ def run_generation(args):
         if tokenizer is not None and tokenizer.eos_token_id is not None and tokenizer.eos_token_id not in terminators:
             terminators.append(tokenizer.eos_token_id)
 
-    log("Initializing model storage...")
+    log("Loading model weights and sizing the cache...")
     if args.max_tokens is None and args.batch is None:
         llm.max_batch = len(prompts)
     max_len = llm.init_storage()
-    log(f"Maximum context length under current memory limit: {max_len} tokens")
-    log("Loading model weights...")
     llm.load_from_hf()
+    mem = llm.engine.memory_report()
+    log(f"Maximum context length under current memory limit: {max_len} tokens "
+        f"(weights {mem['weight_bytes'] / 2**30:.2f} GiB, workspace {mem['workspace_bytes'] / 2**30:.2f} GiB, cache "
+        f"{mem['cache_bytes'] / 2**30:.2f} GiB for {mem['max_tokens']} tokens in {mem['slots']} slots)")
     log("Model loading completed!")
 
     if len(prompts) == 1 and args.use_stream:

@@ -26,14 +26,32 @@ from ..weights.loader import checkpoint_names, load_tensors
 _DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "fp32": torch.float32, "bf16": torch.bfloat16}
 
 
+def _bytes_on(tensors, device) -> int:
+    """Bytes of the distinct storages of those tensors that lie on ``device``."""
+    seen = {}
+    for t in tensors:
+        if t.device == device:
+            st = t.untyped_storage()
+            seen[st.data_ptr()] = st.nbytes()
+    return sum(seen.values())
+
+
 class StepError(ValueError):
     """A step was refused; nothing was run and the cache is unchanged."""
+
+
+class EngineMemoryError(ValueError):
+    """Weights, workspace and cache together exceed the engine's memory limit; said when the engine is built."""
 
 
 @dataclass
 class EngineOptions:
     dtype: str = "bfloat16"                 # 'bfloat16' (serving kernels) or 'float32' (everything in true 32-bit)
-    max_tokens: int = 8192                  # tokens all live sequences hold together (each rounded up to a page)
+    # tokens all live sequences hold together (each rounded up to a page); None: what memory_limit leaves
+    max_tokens: Optional[int] = 8192
+    # fraction of the device's memory that weights, workspace and cache may take together (the reference's
+    # memory_limit, src/model/memory.cuh:22-43); checked when the engine is built.  None: not checked
+    memory_limit: Optional[float] = None
     max_seq_len: Optional[int] = None       # longest sequence; default: what the configuration says the model is for
     max_slots: Optional[int] = None         # live sequences; default: one per page, at most 1024
     max_step_tokens: int = 2048             # tokens one forward pass carries (the reference's chunk_length)
@@ -44,6 +62,9 @@ class EngineOptions:
     # options of the architecture's own (those its registry entry declares, e.g. 'sparse' for MiniCPM4)
     model_options: Dict[str, Any] = field(default_factory=dict)
     max_graphs: int = 32                    # captured decode steps kept (one per batch size and position bound)
+    # run a prompt pass of max_step_tokens tokens and decode passes on a scratch cache while the engine is built,
+    # so that the workspace has its full size before the memory figure is made and no later step allocates
+    rehearse: bool = True
 
 
 @dataclass
@@ -54,7 +75,11 @@ class StepEntry:
 
 
 class Engine:
-    def __init__(self, config: ModelConfig, model, tensors: Dict[str, torch.Tensor], options: EngineOptions):
+    def __init__(self, config: ModelConfig, model, tensors: Dict[str, torch.Tensor], options: EngineOptions,
+                 allocated_before: Optional[int] = None):
+        """``tensors``: the checkpoint's tensors on the device; the dictionary is emptied once the parts have
+        taken what they keep.  ``allocated_before``: the device allocator's count before those tensors were
+        loaded (from_dir and from_tensors pass it), from which the weights' share of memory is measured."""
         if options.dtype not in _DTYPES:
             raise ValueError(f"dtype '{options.dtype}' is not supported (float32, bfloat16)")
         self.options = options
@@ -65,32 +90,128 @@ class Engine:
             raise RuntimeError("the engine runs on a GPU only (device 'cuda:N'); there is no CPU path")
         if not torch.cuda.is_available():
             raise RuntimeError("no GPU is visible: the engine's kernels cannot run")
+        if self.device.index is None:
+            self.device = torch.device("cuda", torch.cuda.current_device())
         self.dtype = _DTYPES[options.dtype]
-        if options.page_size <= 0 or options.page_size % 32:
-            raise ValueError(f"page_size {options.page_size}: the cache kernels lay a page out in chunks of 32 tokens; "
+        page = options.page_size
+        if page <= 0 or page % 32:
+            raise ValueError(f"page_size {page}: the cache kernels lay a page out in chunks of 32 tokens; "
                              f"give a positive multiple of 32")
+        if options.max_tokens is None and options.memory_limit is None:
+            raise ValueError("give max_tokens, or a memory_limit from which the cache is sized")
+        if options.memory_limit is not None and not 0 < options.memory_limit <= 1:
+            raise ValueError(f"memory_limit {options.memory_limit} must be a fraction of the device's memory in (0, 1]")
         max_seq_len = options.max_seq_len or config.longest_sequence or options.max_tokens
+        if not max_seq_len:
+            raise ValueError("max_seq_len is needed: the configuration names no longest sequence and max_tokens is open")
         self.max_seq_len = int(max_seq_len)
+        self.max_step_tokens = max(int(options.max_step_tokens), 1)
+        if options.max_tokens is not None:
+            max_slots = options.max_slots or min(-(-options.max_tokens // page), 1024)
+        else:
+            max_slots = options.max_slots or 1
+        if allocated_before is None:
+            allocated_before = torch.cuda.memory_allocated(self.device) - _bytes_on(tensors.values(), self.device)
         self.workspace = Workspace(self.device)
         # parts check here, at bind time, what their kernels take of these sizes: an engine that was built runs
-        self.runtime = Runtime(self.device, self.dtype, self.workspace, self.max_seq_len, options.tiled_weights,
-                               options.page_size)
+        self.runtime = Runtime(self.device, self.dtype, self.workspace, self.max_seq_len, options.tiled_weights, page)
         with torch.cuda.device(self.device):
             model.bind_all(tensors, self.runtime)
-        n_pages = -(-options.max_tokens // options.page_size)
-        max_slots = options.max_slots or min(n_pages, 1024)
-        self.cache = SequenceCache(model.cache_needs(), options.max_tokens, max_slots, self.max_seq_len,
-                                   options.page_size, self.device, self.dtype)
-        self.max_step_tokens = max(int(options.max_step_tokens), 1)
-        cap = 3 * self.max_step_tokens + 3 * max_slots + 1 + self.max_step_tokens
-        self._meta = torch.zeros(cap, dtype=torch.int32, device=self.device)
+            parts = model.all_parts()
+            for part in parts:
+                part.reserve_workspace(self.workspace, self.runtime, self.max_step_tokens, max_slots)
+        tensors.clear()
+        # a part that cannot be recorded and replayed keeps the whole model's steps eager
+        self.graph_capturable = all(part.graph_capturable for part in parts)
         self.vocab_size = model.vocab_size
         self.steps_run = 0
         self.perf = None                       # utils.perf.PerfTimers; while enabled, steps run eagerly (no graph)
         self._graphs: Dict[Tuple[int, int], tuple] = {}
+        cap = 3 * self.max_step_tokens + 3 * max_slots + 1 + self.max_step_tokens
+        self._meta = torch.zeros(cap, dtype=torch.int32, device=self.device)
         self._stage = [torch.empty(cap, dtype=torch.int32).pin_memory() for _ in range(4)]
         self._stage_ev: List[Optional[torch.cuda.Event]] = [None] * 4
         self._stage_i = 0
+        needs = model.cache_needs()
+        self._rehearsing = False
+        self.max_tokens = options.max_tokens or 0
+        if options.rehearse:
+            self._rehearse(needs, max_slots)
+        # the memory figure: everything this engine holds beside the cache is allocated by now
+        torch.cuda.synchronize(self.device)
+        held = torch.cuda.memory_allocated(self.device) - allocated_before
+        ws_bytes = self.workspace.bytes()
+        self.weight_bytes = max(held - ws_bytes, 0)        # every copy of the weights, and the product library's scratch
+        total = torch.cuda.get_device_properties(self.device).total_memory
+        limit = int(options.memory_limit * total) if options.memory_limit is not None else None
+        plan = lambda tokens: SequenceCache.plan_bytes(needs, tokens, max_slots, self.max_seq_len, page, self.dtype,
+                                                        self.max_step_tokens)
+        # what the device can still give: free memory, and what torch's allocator holds without using it
+        free_now = torch.cuda.mem_get_info(self.device)[0] + (torch.cuda.memory_reserved(self.device)
+                                                              - torch.cuda.memory_allocated(self.device))
+        if options.max_tokens is None:
+            tokens = SequenceCache.tokens_for(needs, min(limit - held, free_now - (256 << 20)), max_slots, self.max_seq_len, page, self.dtype,
+                                              self.max_step_tokens)
+            if tokens == 0:
+                raise EngineMemoryError(self._memory_message(limit, total, plan(max_slots * page), max_slots * page))
+            self.max_tokens = tokens
+        else:
+            self.max_tokens = int(options.max_tokens)
+            if limit is not None and held + plan(self.max_tokens) > limit:
+                raise EngineMemoryError(self._memory_message(limit, total, plan(self.max_tokens), self.max_tokens))
+        self.cache = SequenceCache(needs, self.max_tokens, max_slots, self.max_seq_len, page, self.device, self.dtype,
+                                   self.max_step_tokens)
+        self.workspace.sealed = True
+
+    def _memory_message(self, limit: int, total: int, cache_bytes: int, tokens: int) -> str:
+        gib = lambda b: f"{b / 2**30:.2f} GiB"
+        return (f"memory limit exceeded: weights {gib(self.weight_bytes)} + workspace {gib(self.workspace.bytes())} + "
+                f"cache {gib(cache_bytes)} (for {tokens} tokens) = "
+                f"{gib(self.weight_bytes + self.workspace.bytes() + cache_bytes)}, the limit is {gib(limit)} "
+                f"({self.options.memory_limit:.0%} of the device's {gib(total)})")
+
+    def _rehearse(self, needs, max_slots: int):
+        """One prompt pass of max_step_tokens tokens and decode passes of the largest and of small batches, on a
+        scratch cache that is freed afterwards: every part asks the workspace for what its largest steps need,
+        and the product library sets itself up, before the memory figure is made."""
+        page = self.options.page_size
+        n_prompt = min(self.max_step_tokens, self.max_seq_len)
+        B = max(min(max_slots, self.max_step_tokens), 1)
+        tokens = -(-n_prompt // page) * page + B * page
+        self.cache = SequenceCache(needs, tokens, B + 1, self.max_seq_len, page, self.device, self.dtype,
+                                   self.max_step_tokens)
+        self._rehearsing = True
+        try:
+            s = self.acquire()
+            self.step([StepEntry(s, [0] * n_prompt, [n_prompt - 1])])
+            self.release(s)
+            # kernels change with the number of rows at powers of two at most: those sizes and their successors
+            sizes = {1}
+            b = 2
+            while b < max(B, n_prompt):
+                sizes.update((b, b + 1))
+                b *= 2
+            for b in sorted(sizes | {B}, reverse=True):
+                if b <= B:
+                    slots = [self.acquire() for _ in range(b)]
+                    self.step([StepEntry(x, [0], [0]) for x in slots])         # a decode step of b sequences
+                    for x in slots:
+                        self.release(x)
+                if 2 <= b < n_prompt:
+                    s = self.acquire()
+                    self.step([StepEntry(s, [0] * b, [b - 1])])                  # a short prompt of b tokens
+                    self.release(s)
+        finally:
+            self._rehearsing = False
+            self.cache = None
+            self.steps_run = 0
+        torch.cuda.synchronize(self.device)
+        torch.cuda.empty_cache()
+
+    @property
+    def uses_graph(self) -> bool:
+        """Whether single-token steps replay a captured graph."""
+        return bool(self.options.hip_graph) and self.graph_capturable and not self._rehearsing
 
     # ------------------------------------------------------------------
     @classmethod
@@ -104,11 +225,13 @@ class Engine:
         if config is None:
             config = arch.config_class.from_dict(raw)
         model = arch.build_model(config, options.model_options, checkpoint_names(model_dir))
+        dev = torch.device(options.device)
+        before = torch.cuda.memory_allocated(dev) if dev.type == "cuda" and torch.cuda.is_available() else None
         tensors = load_tensors(
             model_dir, model.all_weight_specs(), device=options.device,
             split_fused=(lambda n, t: arch.split_fused(config, n, t)) if arch.split_fused else None,
             ignore=(lambda n: arch.ignore_tensor(config, n)) if arch.ignore_tensor else None)
-        return cls(config, model, tensors, options)
+        return cls(config, model, tensors, options, before)
 
     @classmethod
     def from_tensors(cls, config: ModelConfig, tensors: Dict[str, torch.Tensor],
@@ -119,7 +242,11 @@ class Engine:
         from ..weights.loader import _compare
         _compare(model.all_weight_specs(), {k: tuple(v.shape) for k, v in tensors.items()}, "the given tensors")
         dev = torch.device(options.device)
-        return cls(config, model, {k: v.to(dev) for k, v in tensors.items()}, options)
+        before = None
+        if dev.type == "cuda" and torch.cuda.is_available():
+            dev = torch.device("cuda", dev.index if dev.index is not None else torch.cuda.current_device())
+            before = torch.cuda.memory_allocated(dev) - _bytes_on(tensors.values(), dev)
+        return cls(config, model, {k: v.to(dev) for k, v in tensors.items()}, options, before)
 
     # ------------------------------------------------------------------
     def acquire(self) -> int:
@@ -159,7 +286,7 @@ class Engine:
                     raise StepError(f"slot {e.slot}: wanted place {w} is outside the {n} tokens of this step")
         full = self.cache.room_for([[(entries[i].slot, b - a) for i, a, b in chunk] for chunk in self._chunks(entries)])
         if full is not None:
-            raise StepError(f"{full} (max_tokens={self.options.max_tokens})")
+            raise StepError(f"{full} (max_tokens={self.max_tokens})")
 
     def _chunks(self, entries: Sequence[StepEntry]):
         """Cut a step into forward passes of at most max_step_tokens tokens.  Yields lists of
@@ -246,18 +373,19 @@ class Engine:
             # a token that opens a page: ask the groups (one that keeps a window gives a page back for it)
             full = cache.room_for([[(s, 1) for s in slots]])
             if full is not None:
-                raise StepError(f"{full} (max_tokens={self.options.max_tokens})")
+                raise StepError(f"{full} (max_tokens={self.max_tokens})")
         before = [live[s] for s in slots]
         pos = np.fromiter((cache.extend_one(s) for s in slots), dtype=np.int32, count=B)
         cache.sync()
         sl = np.asarray(slots, dtype=np.int32)
-        graph = bool(self.options.hip_graph)
+        graph = self.uses_graph
         rows = np.arange(B, dtype=np.int32) if graph else np.asarray(want_rows, dtype=np.int32)
         host = np.concatenate([tok.astype(np.int32), pos, sl, np.arange(B + 1, dtype=np.int32), sl, pos + 1, rows])
+        state = cache.snapshot_state(slots)
         try:
             logits = self._run(host, B, B, [1] * B, int(pos.max()), True, graph, int(rows.size), device_tokens)
         except BaseException:
-            self._roll_back(slots, before)
+            self._roll_back(slots, before, state)
             raise
         if not want_rows:
             return None
@@ -324,7 +452,7 @@ class Engine:
         q_lens = [b - a for _, a, b in chunk]
         n = sum(q_lens)
         single = n == B
-        graph = bool(self.options.hip_graph) and single
+        graph = self.uses_graph and single
         tok = np.empty(n, dtype=np.int32)
         pos = np.empty(n, dtype=np.int32)
         tslot = np.empty(n, dtype=np.int32)
@@ -335,6 +463,7 @@ class Engine:
         dest: List[int] = []
         o = 0
         before = [cache.length(entries[i].slot) for i, _, _ in chunk]
+        state = cache.snapshot_state([entries[i].slot for i, _, _ in chunk])
         for bi, (i, a, b) in enumerate(chunk):
             e = entries[i]
             first = cache.extend(e.slot, b - a)
@@ -358,7 +487,7 @@ class Engine:
         try:
             logits = self._run(host, n, B, q_lens, int(pos.max()), single, graph, int(want_rows.size))
         except BaseException:
-            self._roll_back([entries[i].slot for i, _, _ in chunk], before)
+            self._roll_back([entries[i].slot for i, _, _ in chunk], before, state)
             raise
         if rows:
             dest_t = torch.tensor([dest, rows], dtype=torch.long).to(self.device, non_blocking=True)
@@ -367,14 +496,16 @@ class Engine:
             else:
                 result.index_copy_(0, dest_t[0], logits)
 
-    def _roll_back(self, slots: Sequence[int], lengths: Sequence[int]):
+    def _roll_back(self, slots: Sequence[int], lengths: Sequence[int], state=None):
         """A forward pass failed after the cache had made room for its tokens (a kernel refused a size, the
         device ran out of memory): the slots forget that pass's tokens, so that lengths and cache rows agree
-        again.  Passes of the same step that had completed before stay (a step that validation refuses, by
-        contrast, changes nothing at all)."""
+        again, and fixed-size state that the pass may have advanced is put back as it was before the pass
+        (``state``: SequenceCache.snapshot_state, None for a model without such state).  Passes of the same
+        step that had completed before stay (a step that validation refuses, by contrast, changes nothing at all)."""
         for s, n in zip(slots, lengths):
             if s in self.cache.live and self.cache.length(s) > n:
                 self.cache.truncate(s, n)
+        self.cache.restore_state(state)
 
     def _upload(self, host: np.ndarray, dst: torch.Tensor):
         """Step metadata to the device through pinned memory, without waiting for the GPU."""
@@ -394,5 +525,8 @@ class Engine:
 
     # ------------------------------------------------------------------
     def memory_report(self) -> Dict[str, int]:
-        return {"cache_bytes": self.cache.bytes(), "workspace_bytes": self.workspace.bytes(),
-                "pages": self.cache.n_pages, "slots": self.cache.max_slots}
+        """Bytes the engine holds on the device: weights (every copy, with the product library's scratch), the
+        workspace, the cache; and what the cache holds in tokens."""
+        return {"weight_bytes": self.weight_bytes, "workspace_bytes": self.workspace.bytes(),
+                "cache_bytes": self.cache.bytes(), "pages": self.cache.n_pages, "slots": self.cache.max_slots,
+                "max_tokens": self.max_tokens}

@@ -143,7 +143,10 @@ def _run_batch_overlapped(engine, prompts, batch, max_new_tokens, stop, sampler,
     out: Dict[int, List[int]] = {i: [] for i in batch}
     n_gen: Dict[int, int] = {}
     finished = set()
-    staging = [torch.empty(len(batch), dtype=torch.int32).pin_memory() for _ in range(2)]
+    on_gpu = getattr(engine, "device", None) is not None and engine.device.type == "cuda"
+    staging = [torch.empty(len(batch), dtype=torch.int32) for _ in range(2)]
+    if on_gpu:
+        staging = [t.pin_memory() for t in staging]
     try:
         _sync(engine)
         t0 = time.time()
@@ -190,12 +193,15 @@ def _run_batch_overlapped(engine, prompts, batch, max_new_tokens, stop, sampler,
                 host = staging[turn][:len(active)]
                 turn ^= 1
                 host.copy_(sampled, non_blocking=True)
-                ev = torch.cuda.Event()
-                ev.record()
+                ev = None
+                if on_gpu:
+                    ev = torch.cuda.Event()
+                    ev.record()
                 launched = (list(active), sampled, host, ev)
             if inflight is not None:
                 ids, _, host, ev = inflight
-                ev.synchronize()
+                if ev is not None:
+                    ev.synchronize()
                 resolve(ids, host.tolist())
             inflight = launched
             active, feed_host, feed_dev = [], None, None

@@ -74,38 +74,30 @@ class LLM:
 
     # ------------------------------------------------------------------
     def init_storage(self) -> int:
-        """Decide how many tokens the cache holds (cpmcu/llm.py:115-116 returns the same number):
-        what ``memory_limit`` of the GPU's memory leaves after the weights, unless max_tokens was given."""
-        if self.max_tokens is None:
-            from .weights.loader import checkpoint_files
-            import os
-            total = torch.cuda.get_device_properties(torch.device(self.device)).total_memory
-            weight_bytes = sum(os.path.getsize(f) for f in checkpoint_files(self.path))
-            weight_bytes *= 2          # float32: upcast weights; bfloat16: the second copy in the decode layout
-            model = self.arch.build_model(self.config, self.model_options)
-            esize = 4 if self.dtype == "float32" else 2
-            per_token = sum(sum(s.width / s.every for _, s in n.streams) for n in model.cache_needs()) * esize
-            budget = total * self.memory_limit - weight_bytes - (2 << 30)
-            if budget <= per_token * 64:
-                raise MemoryError(f"memory limit exceeded: {self.memory_limit:.0%} of {total / 2**30:.1f} GiB leaves "
-                                  f"no room for a cache beside {weight_bytes / 2**30:.1f} GiB of weights")
-            limit = self.max_seq_len or self.config.longest_sequence
-            slots = self.max_batch or 1
-            fit = budget // per_token
-            self.max_tokens = int((min(fit, limit * slots) if limit else fit) // 64 * 64)
-        self.max_total_length = min(self.max_tokens, self.max_seq_len or self.config.longest_sequence or self.max_tokens)
+        """Build the engine and return the longest sequence it can hold (cpmcu/llm.py:115-116 returns the same
+        number).  The reference takes ``memory_limit`` of the device's memory in one allocation and gives the
+        cache what the weights leave (src/model/memory.cuh:22-43, src/model/kvcache.cuh:50); here the weights
+        are read and the workspace is sized first, since their measured bytes, not an estimate, decide what is
+        left: the cache gets ``max_tokens`` tokens if that was given, else all that fits under the limit for
+        ``max_batch`` sequences (default one) of at most ``max_seq_len`` tokens.  Weights, workspace and cache
+        beyond the limit are refused here, with the three numbers, before any step runs."""
+        if self.engine is None:
+            slots = self.max_batch if (self.max_batch or self.max_tokens is not None) else 1
+            opts = EngineOptions(dtype=self.dtype, max_tokens=self.max_tokens, memory_limit=self.memory_limit,
+                                 max_seq_len=self.max_seq_len, max_slots=slots, max_step_tokens=self.chunk_length,
+                                 device=self.device, hip_graph=self.cuda_graph, model_options=dict(self.model_options))
+            # the engine reads config.json itself; what the flags changed is handed over through the typed config
+            self.engine = Engine.from_dir(self.path, opts, config=self.config)
+            self.engine.perf = self.perf
+            self.max_tokens = self.engine.max_tokens
+        self.max_total_length = min(self.max_tokens, self.engine.max_seq_len)
         return self.max_total_length
 
     def load_from_hf(self):
-        """Build the engine and load the checkpoint (after init_storage, as in the reference: cpmcu/cli.py:257, 285)."""
-        if self.max_total_length is None:
+        """The reference's second call (cpmcu/cli.py:257, 285).  The weights were read when init_storage built
+        the engine, so nothing is left to do but to say so when the order is wrong."""
+        if self.engine is None:
             raise RuntimeError("call init_storage() before load_from_hf()")
-        opts = EngineOptions(dtype=self.dtype, max_tokens=self.max_tokens, max_seq_len=self.max_seq_len,
-                             max_slots=self.max_batch, max_step_tokens=self.chunk_length, device=self.device,
-                             hip_graph=self.cuda_graph, model_options=dict(self.model_options))
-        # the engine reads config.json itself; what the flags changed is handed over through the typed config
-        self.engine = Engine.from_dir(self.path, opts, config=self.config)
-        self.engine.perf = self.perf
         return self
 
     def _need_engine(self) -> Engine:

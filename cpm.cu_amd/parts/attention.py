@@ -55,6 +55,20 @@ class GQAAttention(Mixer):
         self.rt = rt
         self._qkv_fused = None               # the q/k/v weight re-laid for the fused decode kernel, made at first use
 
+    def reserve_workspace(self, ws, rt: Runtime, max_step_tokens: int, max_slots: int):
+        # the q/k/v weight in the fused decode kernel's order, if any step of this engine can run that kernel
+        plain_rotation = self.position is None or self.position.rotary_params() is not None
+        if (self._qkv_fused is None and plain_rotation and rt.dtype == torch.bfloat16 and self.qkv.tiled is not None
+                and self.hd % 16 == 0 and self.hidden_size % 8 == 0 and rt.page_size % 32 == 0):
+            self._qkv_fused = ops.qkv_rope_weight(self.qkv.weight, self.nh, self.nkv, self.hd)
+        # split-KV shares of steps of few tokens: their number grows with the context
+        if rt.dtype == torch.bfloat16:
+            most = max((n * ops.attention_splits(n, self.nkv, self.nh // self.nkv, rt.max_seq_len)
+                        for n in range(1, min(max_step_tokens, 256) + 1)), default=0)
+            if most > 1:
+                ws.get("attn.part_o", (most, self.nh, self.hd), torch.float32)
+                ws.get("attn.part_ml", (most, self.nh, 2), torch.float32)
+
     def cache_needs(self) -> CacheNeeds:
         w = self.nkv * self.hd
         return CacheNeeds(streams=(("k", StreamSpec(w)), ("v", StreamSpec(w))))
@@ -79,7 +93,7 @@ class GQAAttention(Mixer):
         nh, nkv, hd = self.nh, self.nkv, self.hd
         plain_rotation = self.position is None or self.position.rotary_params() is not None
         if self._fused_projection(n, h.dtype, cache, writes_cache):
-            if self._qkv_fused is None:
+            if self._qkv_fused is None:           # a part used outside an engine (reserve_workspace makes it)
                 self._qkv_fused = ops.qkv_rope_weight(self.qkv.weight, nh, nkv, hd)
             rot = self.position.rotary_params() if self.position is not None else None
             inv_freq, mag = (rot if rot is not None else (None, 1.0))
@@ -141,6 +155,17 @@ class InfLLMv2Attention(GQAAttention):
         if rt.page_size % self.st:
             raise ValueError(f"infllm_v2: kernel_stride {self.st} must divide the cache page of {rt.page_size} tokens "
                              f"(a compressed key's row lies in the page of its first key)")
+
+    def reserve_workspace(self, ws, rt: Runtime, max_step_tokens: int, max_slots: int):
+        super().reserve_workspace(ws, rt, max_step_tokens, max_slots)
+        # the selection's scores grow with the context: sized here for the longest sequence, for steps of few
+        # tokens (many small workgroups through scratch) and of many
+        few = max(256 // self.nkv, 1)
+        need = max(ops.sparse_select_scratch(rt.dtype, n, self.nh, self.nkv, self.hd, rt.max_seq_len - 1, self.ks,
+                                             self.st, self.bs)
+                   for n in {1, min(few, max_step_tokens), min(few + 1, max_step_tokens), max_step_tokens})
+        if need:
+            ws.get("attn.sel_scores", (need,), torch.float32)
 
     def cache_needs(self) -> CacheNeeds:
         w = self.nkv * self.hd

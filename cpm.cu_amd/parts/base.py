@@ -61,6 +61,8 @@ class Workspace:
         self.device = torch.device(device)
         self._buf: Dict[str, torch.Tensor] = {}
         self.generation = 0           # counts the times a buffer moved (captured graphs hold the old address)
+        self.sealed = False           # set by the engine once it is built: what is asked for later is noted
+        self.grown: List[str] = []    # names of buffers made or enlarged after that
 
     def get(self, name: str, shape: Sequence[int], dtype: torch.dtype) -> torch.Tensor:
         n = 1
@@ -73,6 +75,8 @@ class Workspace:
                 self.generation += 1
             buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=self.device)
             self._buf[name] = buf
+            if self.sealed:
+                self.grown.append(name)
         return buf[:nbytes].view(dtype).view(*shape)
 
     def bytes(self) -> int:
@@ -168,7 +172,25 @@ class Part:
     def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime):
         """Take the tensors named by weight_specs (already on the device) and prepare for forward."""
 
+    # False for a part whose forward reads device data on the host, allocates, or launches different work from
+    # step to step (a router that counts tokens per expert, a recurrence that loops in Python over lengths):
+    # such a forward cannot be recorded once and replayed.  An engine whose model holds one runs every step
+    # eagerly, whatever its hip_graph option says.
+    graph_capturable = True
+
+    def reserve_workspace(self, ws: "Workspace", rt: Runtime, max_step_tokens: int, max_slots: int):
+        """Called once when the engine is built, after bind: ask ``ws`` for the scratch whose size grows with the
+        context (``rt.max_seq_len``) rather than with the step, so that it is part of the engine's memory figure
+        and no later step has to grow it.  Scratch that depends on the step's tokens only is sized by the
+        engine's rehearsal passes and needs nothing here."""
+
     # helpers over the tree
+    def all_parts(self) -> List["Part"]:
+        out: List["Part"] = [self]
+        for p in self.parts():
+            out.extend(p.all_parts())
+        return out
+
     def all_weight_specs(self) -> List[WeightSpec]:
         out = list(self.weight_specs())
         for p in self.parts():

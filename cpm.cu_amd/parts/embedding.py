@@ -53,6 +53,11 @@ class LMHead(Part):
         self.rt = rt
         self.tiled = None
 
+    def reserve_workspace(self, ws, rt: Runtime, max_step_tokens: int, max_slots: int):
+        # the table in the decode product's layout (made here and not at bind: a tied table is bound by its owner)
+        if self.tiled is None and rt.dtype == torch.bfloat16 and rt.tiled_weights:
+            self.tiled = ops.TiledWeight(self.tied_to.table if self.tied_to is not None else self.weight)
+
     def forward(self, y: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         w = self.tied_to.table if self.tied_to is not None else self.weight
         if self.tiled is None and self.rt.dtype == torch.bfloat16 and self.rt.tiled_weights:

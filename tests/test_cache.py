@@ -185,3 +185,63 @@ def test_truncate_gives_the_tail_back():
     c.truncate(s, 0)
     assert all(len(g.free_pages) == g.n_pages for g in c.groups)
     c.check()
+
+
+def test_truncate_below_what_a_window_gave_back_is_refused():
+    """Going back is only safe to a length whose next query reads no page that the group already gave back
+    (the start of the last extend always is one)."""
+    c = make([FULL, WIN], max_tokens=256, max_slots=2, max_seq_len=128)
+    s = c.acquire()
+    c.extend(s, 40)
+    c.extend(s, 50)                      # the windowed group keeps from position 40 - 20 + 1 = 21 on: page 0 goes
+    win = c.groups[1]
+    assert win.pages[s][0] == -1 and win.pages[s][1] >= 0
+    free = [len(g.free_pages) for g in c.groups]
+    with pytest.raises(CacheError, match="has already given back page 0"):
+        c.truncate(s, 30)                # the query at 30 reads back to 11, which lay in page 0
+    assert c.length(s) == 90 and [len(g.free_pages) for g in c.groups] == free
+    c.truncate(s, 40)                    # the engine's roll-back: the start of the last extend
+    assert c.length(s) == 40
+    c.check()
+    c.extend(s, 50)
+    c.check()
+
+
+def test_planned_bytes_equal_built_bytes_and_window_pools_are_small():
+    needs = [FULL, FULL, CK, WIN, STATE]
+    for max_tokens, slots, seq, step in ((256, 4, 128, None), (1024, 3, 512, 32), (64, 2, 40, 7)):
+        c = SequenceCache(needs, max_tokens, slots, seq, 16, "cpu", torch.float32, step)
+        tables = sum(g.table.numel() * 4 for g in c.groups)
+        plan = SequenceCache.plan_bytes(needs, max_tokens, slots, seq, 16, torch.float32, step)
+        assert plan == c.bytes() + tables
+    # the windowed group's pool holds its window for every slot, not a page for every token of the cache
+    c = SequenceCache([FULL, WIN], 4096, 3, 2048, 16, "cpu", torch.float32, 32)
+    assert c.groups[0].n_pages == 256 and c.groups[1].n_pages == 3 * ((32 + 20 - 2) // 16 + 2)
+    assert c.pages_to_hold(2048, 32) == [128, (32 + 20 - 2) // 16 + 2]
+    # and a walk at that step never finds the small pool empty
+    slots = [c.acquire() for _ in range(3)]
+    for _ in range(40):
+        for s in slots:
+            c.extend(s, 32)
+    c.check()
+    # the most tokens for a budget: the plan of the answer fits, one page more does not
+    for budget in (10_000, 100_000, 1_000_000):
+        t = SequenceCache.tokens_for(needs, budget, 4, 512, 16, torch.float32, 32)
+        if t:
+            assert SequenceCache.plan_bytes(needs, t, 4, 512, 16, torch.float32, 32) <= budget
+            assert t == 4 * 512 or SequenceCache.plan_bytes(needs, t + 16, 4, 512, 16, torch.float32, 32) > budget
+    assert SequenceCache.tokens_for(needs, 100, 4, 512, 16, torch.float32, 32) == 0
+
+
+def test_state_snapshot_and_restore():
+    c = make([FULL, STATE])
+    assert c.has_state and not make([FULL]).has_state and make([FULL]).snapshot_state([0]) is None
+    a, b = c.acquire(), c.acquire()
+    h = c.view(1).state["h"]
+    h[a] = 1.5
+    h[b] = -2.0
+    snap = c.snapshot_state([b])
+    h[a] = 7.0
+    h[b] = 9.0
+    c.restore_state(snap)
+    assert float(h[b].min()) == float(h[b].max()) == -2.0 and float(h[a].min()) == 7.0

@@ -175,6 +175,7 @@ def test_greedy_generation_through_the_entry_point(model_dirs, references, name)
     llm16.engine.release(s)
     margin = lg.topk(2, dim=-1).values
     sure = (margin[:, 0] - margin[:, 1]) > 0.02
+    assert int(sure.sum()) * 2 >= len(toks16), f"only {int(sure.sum())} of {len(toks16)} choices are clear: nothing is compared"
     assert [t for t, ok in zip(lg.argmax(-1).tolist(), sure.tolist()) if ok] == [t for t, ok in zip(toks16, sure.tolist()) if ok]
 
 

@@ -1,4 +1,6 @@
-"""The generation loop's decisions, with a stand-in engine and sampler (CPU)."""
+"""The generation loop's decisions, with a stand-in engine and sampler (CPU).  Every scenario runs through both
+forms of the loop: the plain one, and the one that the GPU engine gets, in which the host is one step behind
+(a stand-in engine that takes ``device_tokens`` is given that one)."""
 import pytest
 import torch
 
@@ -22,7 +24,8 @@ class FakeCache:
 class FakeEngine:
     """Logits that make greedy emit (last token + 1) % vocab; records every step."""
 
-    def __init__(self, vocab=50, slots=4, max_tokens=4096, max_seq_len=512):
+    def __init__(self, vocab=50, slots=4, max_tokens=4096, max_seq_len=512, overlapped=False):
+        self.accepts_device_tokens = overlapped
         class O:
             pass
         self.options = O()
@@ -45,7 +48,11 @@ class FakeEngine:
         del self.held[s]
         self.free.append(s)
 
-    def step(self, entries):
+    def step(self, entries, device_tokens=None):
+        if device_tokens is not None:
+            assert self.accepts_device_tokens and all(len(e.tokens) == 1 for e in entries)
+            assert device_tokens.dtype == torch.int32 and tuple(device_tokens.shape) == (len(entries),)
+            entries = [type(e)(e.slot, [int(t)], e.want) for e, t in zip(entries, device_tokens)]
         self.log.append([(e.slot, list(e.tokens)) for e in entries])
         rows = []
         for e in entries:
@@ -64,8 +71,12 @@ class ArgmaxSampler:
         return logits.argmax(-1).to(torch.int32)
 
 
-def test_unequal_prompts_stop_tokens_and_early_leavers():
-    eng = FakeEngine()
+BOTH = pytest.mark.parametrize("overlapped", [False, True], ids=["plain loop", "host one step behind"])
+
+
+@BOTH
+def test_unequal_prompts_stop_tokens_and_early_leavers(overlapped):
+    eng = FakeEngine(overlapped=overlapped)
     prompts = [[1, 2, 3], [10], [20, 21, 22, 23, 24]]
     outs = generate(eng, prompts, max_new_tokens=6, stop_token_ids=[13, 27], sampler=ArgmaxSampler())
     assert outs[0].tokens == [4, 5, 6, 7, 8, 9] and outs[0].finish_reason == "length"
@@ -74,22 +85,27 @@ def test_unequal_prompts_stop_tokens_and_early_leavers():
     # step 0 carries the whole prompts; then one token each; finished sequences leave the batch
     assert [len(t) for _, t in eng.log[0]] == [3, 1, 5]
     assert all(len(t) == 1 for step in eng.log[1:] for _, t in step)
-    assert [len(step) for step in eng.log] == [3, 3, 3, 1, 1, 1]
+    # with the host one step behind, the two sequences that stop at their third token have been fed once more
+    # before the host saw the stop token; what that step chose for them is dropped
+    assert [len(step) for step in eng.log] == ([3, 3, 3, 3, 1, 1] if overlapped else [3, 3, 3, 1, 1, 1])
     assert not eng.held and sorted(eng.free) == [0, 1, 2, 3]
-    # the first sampled token counts toward the length: 6 tokens need 5 single-token steps
-    assert len(eng.log) == 6
+    # the first sampled token counts toward the length: 6 tokens need 5 single-token steps; a sequence that ends
+    # by length is never fed its last token, in either loop
+    assert len(eng.log) == 6 and eng.log[-1] == [(0, [8])]
 
 
-def test_first_token_can_already_stop():
-    eng = FakeEngine()
+@BOTH
+def test_first_token_can_already_stop(overlapped):
+    eng = FakeEngine(overlapped=overlapped)
     outs = generate(eng, [[4], [8]], max_new_tokens=5, stop_token_ids=[5], sampler=ArgmaxSampler())
     assert outs[0].tokens == [5] and outs[0].finish_reason == "stop"
     assert outs[1].tokens == [9, 10, 11, 12, 13]
     assert [len(s) for s in eng.log] == [2, 1, 1, 1, 1]
 
 
-def test_more_requests_than_slots_run_as_batches_one_after_another():
-    eng = FakeEngine(slots=2)
+@BOTH
+def test_more_requests_than_slots_run_as_batches_one_after_another(overlapped):
+    eng = FakeEngine(slots=2, overlapped=overlapped)
     prompts = [[i] for i in range(5)]
     s = ArgmaxSampler()
     outs = generate(eng, prompts, max_new_tokens=2, sampler=s)
@@ -130,12 +146,37 @@ def test_plan_batches_asks_every_cache_group():
     assert plan_batches([900], 10, 8, two_groups, [20, 2], 1000) == [[0]]
 
 
-def test_a_failing_step_gives_the_slots_back():
-    eng = FakeEngine()
+@BOTH
+@pytest.mark.parametrize("fail_at", [0, 1, 2])
+def test_a_failing_step_gives_the_slots_back(overlapped, fail_at):
+    eng = FakeEngine(overlapped=overlapped)
+    real = eng.step
 
-    def boom(entries):
-        raise RuntimeError("kernel refused")
+    def boom(entries, device_tokens=None):
+        if len(eng.log) == fail_at:
+            raise RuntimeError("kernel refused")
+        return real(entries, device_tokens) if overlapped else real(entries)
     eng.step = boom
     with pytest.raises(RuntimeError):
-        generate(eng, [[1], [2]], 3, sampler=ArgmaxSampler())
-    assert not eng.held
+        generate(eng, [[1], [2]], 4, sampler=ArgmaxSampler())
+    assert not eng.held and sorted(eng.free) == [0, 1, 2, 3]
+
+
+@BOTH
+def test_the_sampler_sees_request_and_step_of_every_row(overlapped):
+    """Request index and the count of tokens already generated key the random numbers: they must be the same in
+    both loops, also for the sequences that are still running after others have left."""
+    calls = []
+
+    class Recording(ArgmaxSampler):
+        def sample(self, logits, request_ids, steps):
+            calls.append((list(request_ids), list(steps)))
+            return super().sample(logits, request_ids, steps)
+    eng = FakeEngine(overlapped=overlapped)
+    outs = generate(eng, [[1, 2], [10], [30]], max_new_tokens=4, stop_token_ids=[12], sampler=Recording())
+    assert [o.tokens for o in outs] == [[3, 4, 5, 6], [11, 12], [31, 32, 33, 34]]
+    used = {(r, st) for ids, steps in calls for r, st in zip(ids, steps)}
+    assert {(0, k) for k in range(4)} | {(1, 0), (1, 1)} | {(2, k) for k in range(4)} <= used
+    # nothing is drawn for a sequence beyond the step after its stop token (overlapped) or its stop token (plain)
+    assert used - {(1, 2)} == {(0, k) for k in range(4)} | {(1, 0), (1, 1)} | {(2, k) for k in range(4)}
+    assert ((1, 2) in used) == overlapped

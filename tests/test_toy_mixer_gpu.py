@@ -33,6 +33,8 @@ def _define():
         def cache_needs(self):
             return CacheNeeds(state=(("h", StateSpec((self.hidden_size,), torch.float32)),))
 
+        graph_capturable = False        # the scan below reads the batch on the host and loops in Python
+
         def forward(self, h, ctx, cache, writes_cache=True):
             state = cache.state["h"]
             out = torch.empty_like(h)
@@ -136,7 +138,10 @@ def test_toy_mixer_registers_builds_and_steps(tmp_path, dtype):
                "intermediate_size": 56, "decay": 0.6, "rms_norm_eps": 1e-5, "max_position_embeddings": 64}
         write_model_dir(ToyConfig.from_dict(raw), str(tmp_path), seed=4, std=0.1, norm_std=0.1)
         w = load_file(str(tmp_path / "model.safetensors"))
-        eng = Engine.from_dir(str(tmp_path), EngineOptions(dtype=dtype, max_tokens=256, max_slots=2))
+        # hip_graph is asked for (the command line's default); the mixer says that it cannot be captured, and
+        # the engine then runs every step eagerly
+        eng = Engine.from_dir(str(tmp_path), EngineOptions(dtype=dtype, max_tokens=256, max_slots=2, hip_graph=True))
+        assert not eng.graph_capturable and not eng.uses_graph
         assert len(eng.cache.groups) == 1 and eng.model.n_cache_entries == 3
         assert eng.cache.view(1).state["h"].shape == (2, 40) and not eng.cache.view(1).streams
         toks = [int(t) for t in torch.randint(0, 90, (23,), generator=torch.Generator().manual_seed(0))]
@@ -156,9 +161,26 @@ def test_toy_mixer_registers_builds_and_steps(tmp_path, dtype):
             outs.append(lg[:1])
             assert float((lg[1] - ref[i - 5]).abs().max()) < tol
         assert float((torch.cat(outs) - ref).abs().max()) < tol
+        assert not eng._graphs
         eng.release(s2)
         eng.release(other)
         eng.cache.check()
+        # a forward pass that fails after the mixer advanced its state: the state is put back, and the same
+        # tokens then give the logits of a first try
+        s3 = eng.acquire()
+        eng.step([StepEntry(s3, toks[:9], [])])
+        real = eng.model.final_norm.forward
+        for bring in (toks[9:15], toks[9:10]):                  # a pass of several tokens, a single-token step
+            eng.model.final_norm.forward = lambda *a, **k: (_ for _ in ()).throw(RuntimeError("kernel refused"))
+            try:
+                with pytest.raises(RuntimeError, match="kernel refused"):
+                    eng.step([StepEntry(s3, bring, [0])])
+            finally:
+                eng.model.final_norm.forward = real
+            assert eng.length(s3) == 9
+        got = eng.step([StepEntry(s3, toks[9:], list(range(14)))]).cpu()
+        assert float((got - ref[9:]).abs().max()) < tol
+        eng.release(s3)
     finally:
         unregister_architecture("ToyDecayForCausalLM")
         MIXERS.unregister("toy_decay")
