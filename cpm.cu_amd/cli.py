@@ -22,6 +22,17 @@ def log(msg: str):
     print(f"[cpmcu_amd] {msg}", file=sys.stderr, flush=True)
 
 
+# what the configuration summary shows (cpmcu/common/display.py:62-90 groups the same facts)
+SUMMARY_SECTIONS = (
+    ("Model", (("model_path", "Model Path"), ("model_type", "Model Type"), ("dtype", "Data Type"),
+               ("minicpm4_yarn", "MiniCPM4 YARN"))),
+    ("Generation", (("num_generate", "Num Generate"), ("temperature", "Temperature"), ("random_seed", "Random Seed"),
+                    ("use_stream", "Use Stream"), ("ignore_eos", "Ignore EOS"), ("use_chat_template", "Chat Template"))),
+    ("System", (("hip_graph", "HIP Graph"), ("memory_limit", "Memory Limit"), ("chunk_length", "Chunk Length"),
+                ("max_tokens", "Max Tokens"), ("max_seq_len", "Max Seq Len"), ("batch", "Batch"))),
+)
+
+
 class TextTokenizer:
     """tokenizer.json (and the chat template of tokenizer_config.json) if the model folder has them."""
 
@@ -109,6 +120,9 @@ def run_generation(args):
     from .config.base import architecture_name, read_config_json
     from .llm import LLM
     from .registry import declared_flags
+    from .utils.display import Display
+
+    display = Display(plain=args.plain_output)
 
     model_path = args.model_path
     if args.random_weights:
@@ -139,6 +153,10 @@ def run_generation(args):
     foreign = [f.name for f in declared_flags() if f.name not in flags and getattr(args, f.name, None) is not None]
     if foreign:
         raise ValueError(f"architecture '{arch.name}' has no flags {foreign}")
+    sections = list(SUMMARY_SECTIONS)
+    if arch.flags:
+        sections.append((arch.name, tuple((f.name, f.name.replace("_", " ").title()) for f in arch.flags)))
+    display.configuration(args, sections)
     tokenizer = load_tokenizer(model_path)
     llm = LLM(model_path, memory_limit=args.memory_limit, chunk_length=args.chunk_length, dtype=args.dtype,
               cuda_graph=args.hip_graph, temperature=args.temperature, random_seed=args.random_seed,
@@ -167,7 +185,8 @@ def run_generation(args):
     if len(prompts) == 1 and args.use_stream:
         tokens = []
         prefill_time = decode_time = 0.0
-        for ev in llm.generate(prompts[0], args.num_generate, terminators, use_stream=True):
+        for ev in llm.generate(prompts[0], args.num_generate, terminators, use_stream=True,
+                               progress_callback=display.progress_callback()):
             tokens.append(ev["token"])
             prefill_time = max(prefill_time, ev["prefill_time"])
             decode_time = max(decode_time, ev["decode_time"])
@@ -176,7 +195,7 @@ def run_generation(args):
         sys.stdout.write("\n")
         stats = [(len(prompts[0]), prefill_time, len(tokens), decode_time)]
     else:
-        outs = llm.generate(prompts, args.num_generate, terminators)
+        outs = llm.generate(prompts, args.num_generate, terminators, progress_callback=display.progress_callback())
         stats = []
         for i, c in enumerate(outs):
             text = tokenizer.decode(c.tokens) if tokenizer is not None else " ".join(str(t) for t in c.tokens)
@@ -187,8 +206,7 @@ def run_generation(args):
     t_prefill = max(s[1] for s in stats)
     n_dec = sum(max(s[2] - 1, 0) for s in stats)
     t_dec = max(s[3] for s in stats)
-    log(f"Prefill length: {n_prompt}  time: {t_prefill:.2f} s  speed: {n_prompt / max(t_prefill, 1e-9):.2f} tok/s")
-    log(f"Decode length: {n_dec}  time: {t_dec:.2f} s  speed: {n_dec / max(t_dec, 1e-9):.2f} tok/s")
+    display.performance(n_prompt, t_prefill, n_dec, t_dec)
     if args.perf:
         llm.print_perf_summary()
 

@@ -126,6 +126,7 @@ class Engine:
         self.vocab_size = model.vocab_size
         self.steps_run = 0
         self.perf = None                       # utils.perf.PerfTimers; while enabled, steps run eagerly (no graph)
+        self.on_pass = None                    # called (tokens done, tokens of the step) after every forward pass
         self._graphs: Dict[Tuple[int, int], tuple] = {}
         cap = 3 * self.max_step_tokens + 3 * max_slots + 1 + self.max_step_tokens
         self._meta = torch.zeros(cap, dtype=torch.int32, device=self.device)
@@ -332,9 +333,13 @@ class Engine:
                 row_of.setdefault((i, int(w)), []).append(n_rows)
                 n_rows += 1
         result = torch.empty((n_rows, self.vocab_size), dtype=torch.float32, device=self.device) if n_rows else None
+        done, total = 0, sum(len(e.tokens) for e in entries)
         with torch.cuda.device(self.device):
             for chunk in self._chunks(entries):
                 self._forward(entries, chunk, row_of, result)
+                done += sum(b - a for _, a, b in chunk)
+                if self.on_pass is not None:
+                    self.on_pass(done, total)
         self.steps_run += 1
         return result
 

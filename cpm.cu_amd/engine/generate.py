@@ -93,6 +93,20 @@ def _sync(engine):
         torch.cuda.synchronize(engine.device)
 
 
+def _prompt_step(engine, prompts, batch, slots, on_prefill):
+    """The batch's prompts in one step; an engine that cuts a step into forward passes reports each of them
+    ('advance': tokens done so far)."""
+    entries = [StepEntry(slots[i], list(prompts[i]), [len(prompts[i]) - 1]) for i in batch]
+    if on_prefill is None or not hasattr(engine, "on_pass"):
+        return engine.step(entries)
+    before = engine.on_pass
+    engine.on_pass = lambda done, total: on_prefill("advance", {"current_tokens": done})
+    try:
+        return engine.step(entries)
+    finally:
+        engine.on_pass = before
+
+
 def _run_batch(engine, prompts, batch, max_new_tokens, stop, sampler, results, on_token, on_prefill):
     slots = {i: engine.acquire() for i in batch}
     out: Dict[int, List[int]] = {i: [] for i in batch}
@@ -101,7 +115,7 @@ def _run_batch(engine, prompts, batch, max_new_tokens, stop, sampler, results, o
         t0 = time.time()
         if on_prefill:
             on_prefill("begin", {"total_tokens": sum(len(prompts[i]) for i in batch)})
-        logits = engine.step([StepEntry(slots[i], list(prompts[i]), [len(prompts[i]) - 1]) for i in batch])
+        logits = _prompt_step(engine, prompts, batch, slots, on_prefill)
         tokens = sampler.sample(logits, batch, [0] * len(batch)).tolist()
         _sync(engine)
         prefill_time = time.time() - t0
@@ -152,7 +166,7 @@ def _run_batch_overlapped(engine, prompts, batch, max_new_tokens, stop, sampler,
         t0 = time.time()
         if on_prefill:
             on_prefill("begin", {"total_tokens": sum(len(prompts[i]) for i in batch)})
-        logits = engine.step([StepEntry(slots[i], list(prompts[i]), [len(prompts[i]) - 1]) for i in batch])
+        logits = _prompt_step(engine, prompts, batch, slots, on_prefill)
         first = sampler.sample(logits, batch, [0] * len(batch))
         tokens = first.tolist()
         prefill_time = time.time() - t0

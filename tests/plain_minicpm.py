@@ -134,7 +134,7 @@ def compressed_keys(k, ks, st):
     return torch.stack([k[st * j: st * j + ks].mean(0) for j in range(n_ck)])
 
 
-def infllm_select(q, ck, p, sc, nkv):
+def infllm_select(q, ck, p, sc, nkv, pools=None):
     """Blocks of keys that the query at absolute position p attends to, for
     each kv head: list (per head) of sorted block indices, or None for dense.
 
@@ -151,7 +151,8 @@ def infllm_select(q, ck, p, sc, nkv):
       5. candidates b <= floor(p/bs) - window_size/bs; the min(topk, #cand)
          largest, ties to the lower index;
       6. window: blocks floor(p/bs) - window_size/bs < b <= floor(p/bs).
-    q [nh, hd] rotated query, ck [n_ck, nkv, hd]."""
+    q [nh, hd] rotated query, ck [n_ck, nkv, hd].  ``pools``: a list that receives every kv head's
+    pooled scores of the candidate blocks (a test asks how clear a choice was)."""
     ks, st, bs = sc["kernel_size"], sc["kernel_stride"], sc["block_size"]
     if p + 1 <= sc["dense_len"]:
         return None
@@ -175,6 +176,8 @@ def infllm_select(q, ck, p, sc, nkv):
                     pool[b] = max(pool[b], score[j])
         for b in range(min(sc["init_blocks"], n_cand)):
             pool[b] = float("inf")
+        if pools is not None:
+            pools.append(pool.clone())
         order = sorted(range(n_cand), key=lambda b: (-pool[b].item(), b))
         chosen = sorted(order[:min(sc["topk"], n_cand)])
         out.append(sorted(set(chosen) | set(window)))

@@ -180,3 +180,59 @@ def test_the_sampler_sees_request_and_step_of_every_row(overlapped):
     # nothing is drawn for a sequence beyond the step after its stop token (overlapped) or its stop token (plain)
     assert used - {(1, 2)} == {(0, k) for k in range(4)} | {(1, 0), (1, 1)} | {(2, k) for k in range(4)}
     assert ((1, 2) in used) == overlapped
+
+
+def test_display_plain_and_formatted():
+    """What the command line prints beside the text (cpmcu/common/display.py:95-115, 182-260): plain mode has one
+    fact a line and nothing that moves; formatted mode draws a bar in place."""
+    import io
+    from cpmcu_amd.utils.display import Display
+    out = io.StringIO()
+    d = Display(plain=True, stream=out)
+    cb = d.progress_callback()
+    cb("begin", {"total_tokens": 100})
+    cb("advance", {"current_tokens": 40})
+    cb("finish", {"total_time": 0.5})
+    d.performance(100, 0.5, 20, 2.0)
+    text = out.getvalue()
+    assert "\r" not in text and "\033" not in text
+    assert text.splitlines()[:2] == ["Prefilling: 0/100 tokens", "Prefill done: 100/100 tokens in 0.50 s"]
+    assert "  Prefill Speed: 200.0 tokens/s" in text and "  Decode Speed: 10.0 tokens/s" in text
+    out = io.StringIO()
+    d = Display(plain=False, stream=out)
+    cb = d.progress_callback()
+    cb("begin", {"total_tokens": 100})
+    for n in (10, 50, 100):
+        cb("advance", {"current_tokens": n})
+    cb("finish", {"total_time": 0.25})
+    text = out.getvalue()
+    assert text.count("\r") >= 3 and "[" + "#" * 15 + "." * 15 + "] 50/100 tokens" in text and "0.25 s" in text
+    assert "\033" not in text                                     # colours only on a terminal
+
+    class Args:
+        model_path, dtype, nothing = "/m", "bfloat16", None
+    out = io.StringIO()
+    Display(plain=False, stream=out).configuration(Args, [("Model", (("model_path", "Model Path"), ("dtype", "Data Type"),
+                                                                      ("nothing", "Unset"), ("absent", "Absent")))])
+    text = out.getvalue()
+    assert "--- Model ---" in text and "Model Path  /m" in text and "Unset" not in text and "Absent" not in text
+
+
+def test_prompt_passes_are_reported_as_progress():
+    """An engine that cuts the prompt step into forward passes reports each one: begin, advance ..., finish."""
+    class PassingEngine(FakeEngine):
+        on_pass = None
+
+        def step(self, entries, device_tokens=None):
+            out = super().step(entries)
+            if self.on_pass is not None and any(len(e.tokens) > 1 for e in entries):
+                total = sum(len(e.tokens) for e in entries)
+                for done in range(4, total + 4, 4):
+                    self.on_pass(min(done, total), total)
+            return out
+    events = []
+    eng = PassingEngine()
+    generate(eng, [[1, 2, 3, 4, 5, 6], [7, 8, 9]], 2, sampler=ArgmaxSampler(), on_prefill=lambda e, d: events.append((e, dict(d))))
+    assert [e for e, _ in events] == ["begin", "advance", "advance", "advance", "finish"]
+    assert events[0][1] == {"total_tokens": 9} and [d["current_tokens"] for e, d in events if e == "advance"] == [4, 8, 9]
+    assert eng.on_pass is None
