@@ -82,6 +82,77 @@ def prefill_flops(cfg, n):
     return 2 * n * lin + attn + 2 * V * H
 
 
+def batch_prefill_flops(cfg, lens):
+    """Prompts of several lengths in one step: the products once a token, causal attention a prompt, one head row each."""
+    H, I, V, L = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size, cfg.num_hidden_layers
+    nh, nkv, hd = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    lin = L * ((nh + 2 * nkv) * hd * H + H * nh * hd + 3 * H * I)
+    attn = sum(L * nh * hd * 2 * (n * (n + 1) // 2) * 2 for n in lens)
+    return 2 * sum(lens) * lin + attn + 2 * len(lens) * V * H
+
+
+def sparse_keys_read(sc, context):
+    """Keys a query at the end of `context` tokens attends to under InfLLM-v2: all of them up to dense_len, else
+    the chosen blocks and the window."""
+    if context <= sc["dense_len"]:
+        return context
+    return min(context, (sc["topk"] + sc["window_size"] // sc["block_size"]) * sc["block_size"])
+
+
+def sparse_decode_bytes(cfg, sc, esize, batch, context):
+    """What a decode step with block selection has to read: every weight once, and per sequence the attended
+    keys and values and the compressed keys that the selection scores."""
+    ck = cfg.num_hidden_layers * (context // sc["kernel_stride"]) * cfg.num_key_value_heads * cfg.head_dim * esize
+    return weight_bytes_per_step(cfg, esize) + batch * (sparse_keys_read(sc, context) * kv_bytes_per_token(cfg, esize) + ck)
+
+
+def sparse_prefill_flops(cfg, sc, n):
+    """A prompt of n tokens with block selection: products, attention over the keys each query attends to (causal
+    up to dense_len), the selection's scores over the compressed keys, one head row."""
+    H, I, V, L = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size, cfg.num_hidden_layers
+    nh, nkv, hd = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    lin = L * ((nh + 2 * nkv) * hd * H + H * nh * hd + 3 * H * I)
+    dense = min(n, sc["dense_len"])
+    keys = dense * (dense + 1) // 2 + sum(sparse_keys_read(sc, p + 1) for p in range(dense, n))
+    scores = sum(p // sc["kernel_stride"] for p in range(dense, n))
+    return 2 * n * lin + L * nh * hd * 2 * 2 * keys + L * nh * hd * 2 * scores + 2 * V * H
+
+
+def calibrate_read(dev):
+    """GB/s of a kernel that only reads, over 4 GiB (far beyond the caches)."""
+    import torch
+    from cpmcu_amd import ops
+    buf = torch.empty(1 << 30, dtype=torch.int32, device=dev).random_()
+    out = torch.zeros(8192, dtype=torch.int32, device=dev)
+    best = 0.0
+    for _ in range(4):
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        ops.read_bandwidth(buf, out)
+        torch.cuda.synchronize()
+        best = max(best, buf.numel() * 4 / (time.perf_counter() - t) / 1e9)
+    return best
+
+
+def timer_table(eng, run, title):
+    """The timers by kernel class (average ms a call) for `run()` with the engine's timers switched on; steps
+    then run eagerly, so the figures are of the kernels with their launches, not of the graph."""
+    from cpmcu_amd.utils.perf import PerfTimers
+    import torch
+    before = eng.perf
+    eng.perf = PerfTimers(enabled=True)
+    try:
+        run()
+        torch.cuda.synchronize()
+        rows = eng.perf.summary()
+    finally:
+        eng.perf = before
+    print(f"[bench] timers, {title}:", file=sys.stderr)
+    for label, kind, count, total, avg in sorted(rows, key=lambda r: -r[3]):
+        print(f"[bench]   {label:<28}{count:>7} calls{total:>11.3f} ms{avg * 1e3:>10.1f} us each", file=sys.stderr)
+    return {label: round(avg, 5) for label, kind, count, total, avg in rows}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -95,6 +166,9 @@ def main():
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--hip-graph", type=int, default=1)
+    ap.add_argument("--perf", action="store_true",
+                    help="after the timed runs, a few eager steps with the engine's timers on: average ms by kernel "
+                         "class (products / attention / selection / norms / head) on stderr and under 'timers'")
     ap.add_argument("--scenario", default="headline", choices=["headline", "small_batch64", "sparse32k"],
                     help="headline: the 8B shape at batch 8, context 4,096 (the default, the contract's line); "
                          "small_batch64: the 0.5B shape, 64 unequal prompts through the generation loop; sparse32k: "
@@ -196,16 +270,7 @@ def main():
         """What this GPU gives a kernel that only reads (GB/s) and the library's product of two large bf16
         matrices (FLOP/s): the ceilings that memory-bound and matrix-bound work can be held against besides
         the published peaks."""
-        buf = torch.empty(1 << 30, dtype=torch.int32, device=dev).random_()     # 4 GiB: far beyond the caches
-        out = torch.zeros(8192, dtype=torch.int32, device=dev)
-        best = 0.0
-        for _ in range(4):
-            torch.cuda.synchronize()
-            t = time.perf_counter()
-            ops.read_bandwidth(buf, out)
-            torch.cuda.synchronize()
-            best = max(best, buf.numel() * 4 / (time.perf_counter() - t) / 1e9)
-        del buf
+        best = calibrate_read(dev)
         a = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
         b = torch.randn(8192, 8192, device=dev, dtype=torch.bfloat16)
         c = torch.empty_like(a)
@@ -275,6 +340,18 @@ def main():
             pts[f"decode_b{b}_ms"] = round(d / st * 1e3, 4)
             pts[f"decode_b{b}_frac"] = round(gbs / HBM_PEAK_GBS, 4)
         rec["points"] = pts
+    if args.perf:
+        def few_steps():
+            slots = fill_context(args.batch, args.context)
+            for _ in range(4):
+                eng.step([StepEntry(s, [1], [0]) for s in slots])
+            for s in slots:
+                eng.release(s)
+            if not args.no_prefill:
+                s = eng.acquire()
+                eng.step([StepEntry(s, rand_ids(args.prefill_tokens), [args.prefill_tokens - 1])])
+                eng.release(s)
+        rec["timers"] = timer_table(eng, few_steps, f"batch {args.batch}, context {args.context}")
     print(json.dumps(rec), flush=True)
 
 
@@ -300,6 +377,13 @@ def other_scenarios(args, dev):
         prefill_s = max(o.prefill_time for o in outs)
         decode_s = max(o.decode_time for o in outs)
         n_dec = sum(len(o.tokens) - 1 for o in outs)
+        esize = 2 if args.dtype == "bfloat16" else 4
+        ms_step = decode_s / (new - 1) * 1e3
+        # a decode step reads every weight once and the live cache: all 64 sequences, half-way through their 256 tokens
+        step_b = weight_bytes_per_step(cfg, esize) + sum(n + new // 2 for n in lens) * kv_bytes_per_token(cfg, esize)
+        read_gbs = calibrate_read(dev)
+        achieved = step_b / (ms_step * 1e-3) / 1e9
+        peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
         rec = {"metric": "MiniCPM4-0.5B shape, 64 unequal prompts (128..2048), 256 new tokens each: decode tok/s through "
                          "the generation loop", "value": round(n_dec / decode_s, 1), "unit": "tokens/s", "n_gpus": 1,
                "steps": new - 1, "warmup": 0, "ms_per_step": round(decode_s / (new - 1) * 1e3, 4),
@@ -309,13 +393,22 @@ def other_scenarios(args, dev):
                           "heads": 16, "kv_heads": 2, "head_dim": 64, "intermediate": 4096, "vocab": 73448,
                           "global_batch": 64, "prompt_tokens": sum(lens), "new_tokens": new, "parallelism": "1gpu",
                           "hip_graph": bool(args.hip_graph)},
-               "prefill": {"value": round(sum(lens) / prefill_s, 1), "tokens": sum(lens), "ms": round(prefill_s * 1e3, 2)}}
+               "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                            "frac": round(achieved / HBM_PEAK_GBS, 4), "bytes_per_step": step_b,
+                            "read_kernel": round(read_gbs, 1), "frac_of_read_kernel": round(achieved / read_gbs, 4)},
+               "prefill": {"value": round(sum(lens) / prefill_s, 1), "tokens": sum(lens), "ms": round(prefill_s * 1e3, 2),
+                           "frac": round(batch_prefill_flops(cfg, lens) / prefill_s / peak, 4)}}
+        if args.perf:
+            rec["timers"] = timer_table(eng, lambda: generate(eng, prompts[:64], 4), "64 unequal prompts, 4 tokens each")
         print(json.dumps(rec), flush=True)
         return
     raw = config_8b(args.layers)
     raw["sparse_config"] = dict(SPARSE_32K)
     cfg = MiniCPMConfig.from_dict(raw)
     n_prompt, new = 32000, 256
+    esize = 2 if args.dtype == "bfloat16" else 4
+    peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
+    read_gbs = calibrate_read(dev)
     eng = Engine.from_tensors(cfg, random_tensors(cfg, 0, device=dev), EngineOptions(
         dtype=args.dtype, max_tokens=4 * 32768, max_slots=4, max_step_tokens=2048, device=dev,
         hip_graph=bool(args.hip_graph)))
@@ -355,11 +448,30 @@ def other_scenarios(args, dev):
         dec = time.perf_counter() - t
         for sl in slots:
             eng.release(sl)
+        ms_step = dec / (new - 8) * 1e3
+        step_b = sparse_decode_bytes(cfg, SPARSE_32K, esize, batch, n_prompt + new // 2)
+        achieved = step_b / (ms_step * 1e-3) / 1e9
         if batch == 1:
             rec.update({"value": round((new - 8) / dec, 2), "steps": new - 8, "warmup": 8,
-                        "ms_per_step": round(dec / (new - 8) * 1e3, 4),
-                        "prefill": {"value": round(n_prompt / pre, 1), "tokens": n_prompt, "ms": round(pre * 1e3, 1)}})
+                        "ms_per_step": round(ms_step, 4),
+                        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                     "frac": round(achieved / HBM_PEAK_GBS, 4), "bytes_per_step": step_b,
+                                     "read_kernel": round(read_gbs, 1),
+                                     "frac_of_read_kernel": round(achieved / read_gbs, 4)},
+                        "prefill": {"value": round(n_prompt / pre, 1), "tokens": n_prompt, "ms": round(pre * 1e3, 1),
+                                    "frac": round(sparse_prefill_flops(cfg, SPARSE_32K, n_prompt) / (pre / batch) / peak, 4)}})
         rec["points"][f"decode_b{batch}"] = round(batch * (new - 8) / dec, 2)
+        rec["points"][f"decode_b{batch}_ms"] = round(ms_step, 4)
+        rec["points"][f"decode_b{batch}_frac"] = round(achieved / HBM_PEAK_GBS, 4)
+    if args.perf:
+        def few_steps():
+            sl = eng.acquire()
+            for a in range(0, n_prompt, 2048):
+                eng.step([StepEntry(sl, warm[a:min(a + 2048, n_prompt)], [])])
+            for i in range(4):
+                eng.step([StepEntry(sl, [warm[n_prompt + i]], [0])])
+            eng.release(sl)
+        rec["timers"] = timer_table(eng, few_steps, "a 32,000-token prompt in chunks of 2,048 and 4 decode steps")
     print(json.dumps(rec), flush=True)
 
 

@@ -13,7 +13,10 @@
 //   value pools, page table, positions, token slots, optional block lists.
 // * It calls no hipMalloc, hipFree or allocating library routine.  Its first call on a device asks the
 //   runtime for that device's address of the array (hipGetSymbolAddress), with that device current; later
-//   calls only launch kernels on `stream`, which must belong to the current device.
+//   calls only launch kernels on `stream`, which must belong to the current device.  That first call may
+//   make the runtime load the library's code and takes a lock: a caller that captures a graph makes one call
+//   on the device OUTSIDE any capture first (the runtime may refuse such calls under capture or end the
+//   capture); the calls it then records only launch kernels.
 // * n * heads * n_splits * (head_dim + 2) floats of shares must fit into the array; a larger call is refused
 //   with a message that names the sizes, and nothing is launched.
 // * All calls on one GPU share that GPU's array.  It keeps the last call's contents; nothing in it has to

@@ -265,7 +265,16 @@ __global__ __launch_bounds__(NW * 64) void qkv_rope_kernel(
 // Rows a workgroup owns for a weight of `total_rows` rows (even, 16..32): 16, unless that leaves some CUs with
 // one workgroup more than the others and a few more rows each even that out.
 extern "C" int cpmcu_qkv_rope_rows_per_workgroup(int total_rows) {
-    const int cus = 256;
+    static int device_cus = 0;              // asked of the current device once; 256 (the MI355X) if it cannot say
+    if (device_cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+            (void)hipGetLastError();
+            n = 256;
+        }
+        device_cus = n;
+    }
+    const int cus = device_cus;
     const int strips = (total_rows + 15) / 16;
     if (strips <= cus || strips % cus == 0) return 16;
     const int rounds = strips / cus;

@@ -781,8 +781,10 @@ __global__ __launch_bounds__(256) void select_normalise_kernel(const int* __rest
     const int groups = (n_vis + 63) / 64;
     float* ms = stats_in_lds ? (float*)(gst + (long)sc.n_groups * G) : (float*)gst;
     float* inv = ms + G;
-    // all threads fetch the groups' (max, sum) at once; then a thread a head merges them in their order,
-    // so the result does not depend on which workgroup forms it
+    // all threads fetch the groups' (max, sum) at once; then a wavefront a head in turn, a lane a group of 64
+    // keys, maximum and sum by wave reductions: the same sums in the same order as select_blocks_kernel forms
+    // when it normalises the scores itself, so both forms give the same scores to the last bit, and the
+    // result does not depend on which workgroup forms it
     const float2* st = (const float2*)(sc.stats + row * sc.n_groups * G * 2);
     const float2* src = st;
     if (stats_in_lds) {
@@ -790,16 +792,21 @@ __global__ __launch_bounds__(256) void select_normalise_kernel(const int* __rest
         __syncthreads();
         src = gst;
     }
-    for (int h = tid; h < G; h += 256) {
+    const int wave = tid >> 6, lane = tid & 63;
+    for (int h = wave; h < G; h += 4) {
         float mm = -INFINITY;
-        for (int gi = 0; gi < groups; ++gi) mm = fmaxf(mm, src[gi * G + h].x);
+        for (int gi = lane; gi < groups; gi += 64) mm = fmaxf(mm, src[gi * G + h].x);
+        mm = wave_max(mm);
         float ll = 0.f;
-        for (int gi = 0; gi < groups; ++gi) {
+        for (int gi = lane; gi < groups; gi += 64) {
             const float2 v = src[gi * G + h];
             ll += v.y * exp2f(v.x - mm);
         }
-        ms[h] = mm;
-        inv[h] = ll > 0.f ? 1.0f / ll : 0.f;
+        ll = wave_sum(ll);
+        if (lane == 0) {
+            ms[h] = mm;
+            inv[h] = ll > 0.f ? 1.0f / ll : 0.f;
+        }
     }
     __syncthreads();
     const int j = blockIdx.z * 256 + tid;

@@ -76,12 +76,14 @@ class DecoderModel(Part):
 
     def forward(self, ctx: StepContext) -> torch.Tensor:
         """float32 logits [R, V] at ctx.logit_rows; the step's tokens enter the cache."""
-        stream = ResidualStream(self.embedding.forward(ctx))
+        with ctx.timed("embed"):
+            stream = ResidualStream(self.embedding.forward(ctx))
         for r in self.schedule:
             self.layers[r.layer].forward(stream, ctx, ctx.cache.view(r.cache) if ctx.cache is not None else None,
                                          r.writes_cache)
         if ctx.logit_rows is None or ctx.logit_rows.numel() == 0:
             return None
-        y = self.final_norm.forward(stream.x, stream.pending, stream.pending_scale, ctx, rows=ctx.logit_rows,
-                                    tag="final.y")
-        return self.head.forward(y, ctx)
+        with ctx.timed("head"):
+            y = self.final_norm.forward(stream.x, stream.pending, stream.pending_scale, ctx, rows=ctx.logit_rows,
+                                        tag="final.y")
+            return self.head.forward(y, ctx)

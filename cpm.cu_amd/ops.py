@@ -345,6 +345,19 @@ def prefill_tiles(q_lens: Sequence[int], tokens_per_wave: int, device) -> torch.
     return torch.tensor(tiles, dtype=torch.int32).to(device)
 
 
+_cu_count = None
+
+
+def compute_units() -> int:
+    """CUs of the current GPU (256 on the MI355X, which is also what the heuristics below were measured on and
+    what they assume when no GPU is visible)."""
+    global _cu_count
+    if _cu_count is None:
+        _cu_count = (torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
+                     if torch.cuda.is_available() else 256)
+    return _cu_count
+
+
 def attention_splits(n_tokens: int, nkv: int, group: int, max_keys: int) -> int:
     """Shares of a token's keys for steps of few tokens.  Measured on the MI355X (head size 128, 2 kv heads,
     workgroups of 4 wavefronts, graph replay over keys that come from memory, attention + merge, in us for
@@ -360,11 +373,12 @@ def attention_splits(n_tokens: int, nkv: int, group: int, max_keys: int) -> int:
     registers: one sequence at 32,000 keys, whole step, 3.89 ms with 64 shares against 3.60 with 32).  A step
     that has 128 workgroups or more by itself takes two shares from 4,096 keys on (they even out the
     workgroups' ends) and one below (no merge kernel: 64 sequences of the 0.5B shape)."""
-    if n_tokens > 256:
+    cus = compute_units()
+    if n_tokens > cus:
         return 1
     groups = n_tokens * nkv * -(-group // 16)
-    want = max(1, 256 // max(groups, 1))
-    if groups >= 128:
+    want = max(1, cus // max(groups, 1))
+    if groups >= cus // 2:
         want = 2 if max_keys >= 4096 else 1
     return max(1, min(want, max_keys // 128, 32))
 
@@ -657,7 +671,7 @@ def skinny_split(M: int, N: int, K: int) -> int:
     cost traffic."""
     wgs = -(-N // 64)
     cap = 16 if M <= 16 else (8 if M <= 32 else 4)
-    most = 1280 if M <= 16 else 256
+    most = 5 * compute_units() if M <= 16 else compute_units()
     want = 1
     while want * 2 <= cap and wgs * want * 2 <= most and K // (want * 2) >= 512:
         want *= 2

@@ -64,7 +64,7 @@ class GQAAttention(Mixer):
         # split-KV shares of steps of few tokens: their number grows with the context
         if rt.dtype == torch.bfloat16:
             most = max((n * ops.attention_splits(n, self.nkv, self.nh // self.nkv, rt.max_seq_len)
-                        for n in range(1, min(max_step_tokens, 256) + 1)), default=0)
+                        for n in range(1, min(max_step_tokens, ops.compute_units()) + 1)), default=0)
             if most > 1:
                 ws.get("attn.part_o", (most, self.nh, self.hd), torch.float32)
                 ws.get("attn.part_ml", (most, self.nh, 2), torch.float32)
@@ -124,15 +124,18 @@ class GQAAttention(Mixer):
         output projection."""
         sel_blocks, sel_count, bs, window_blocks = sel if sel is not None else (None, None, 0, 0)
         out = ctx.ws.get("attn.out", tuple(q.shape), q.dtype)
-        ops.attention(q, out, self.nh, self.nkv, self.hd, self.scale, cache.streams["k"], cache.streams["v"],
-                      cache.page_table, cache.page_size, ctx, sel_blocks, sel_count, bs, window_blocks)
+        with ctx.timed("attn_core"):
+            ops.attention(q, out, self.nh, self.nkv, self.hd, self.scale, cache.streams["k"], cache.streams["v"],
+                          cache.page_table, cache.page_size, ctx, sel_blocks, sel_count, bs, window_blocks)
         if defer_last and self.o.defers(out):
             return DeferredBranch(self.o, out, ctx, "attn.o")
-        return self.o.forward(out, ctx, "attn.o", out_dtype=torch.float32, partials=True)
+        with ctx.timed("attn_o"):
+            return self.o.forward(out, ctx, "attn.o", out_dtype=torch.float32, partials=True)
 
     def forward(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool = True, row_scale=None,
                 defer_last: bool = False):
-        q = self.project_and_store(h, ctx, cache, writes_cache, row_scale)
+        with ctx.timed("attn_qkv_rope"):
+            q = self.project_and_store(h, ctx, cache, writes_cache, row_scale)
         return self.attend_and_project(q, ctx, cache, defer_last=defer_last)
 
 
@@ -177,11 +180,13 @@ class InfLLMv2Attention(GQAAttention):
                 defer_last: bool = False):
         # decode steps: the projection kernel completes the compressed keys itself (one kernel of the chain less)
         fused = self._fused_projection(h.shape[0], h.dtype, cache, writes_cache)
-        q = self.project_and_store(h, ctx, cache, writes_cache, row_scale,
-                                   compress=(cache.streams["ck"], self.ks, self.st) if fused else None)
+        with ctx.timed("attn_qkv_rope"):
+            q = self.project_and_store(h, ctx, cache, writes_cache, row_scale,
+                                       compress=(cache.streams["ck"], self.ks, self.st) if fused else None)
         if writes_cache and not fused:
-            ops.compress_keys(cache.streams["k"], cache.streams["ck"], self.nkv, cache.page_table, cache.page_size,
-                              ctx.positions, ctx.tok_slot, self.ks, self.st)
+            with ctx.timed("attn_compress"):
+                ops.compress_keys(cache.streams["k"], cache.streams["ck"], self.nkv, cache.page_table,
+                                  cache.page_size, ctx.positions, ctx.tok_slot, self.ks, self.st)
         sel = None
         if ctx.max_pos + 1 > self.dense_len:
             n = q.shape[0]
@@ -190,9 +195,11 @@ class InfLLMv2Attention(GQAAttention):
             sel_count = ctx.ws.get("attn.sel_count", (n, self.nkv), torch.int32)
             need = ops.sparse_select_scratch(q.dtype, n, self.nh, self.nkv, self.hd, ctx.max_pos, self.ks, self.st, self.bs)
             scratch = ctx.ws.get("attn.sel_scores", (need,), torch.float32) if need else None
-            ops.sparse_select(q, cache.streams["ck"], self.nh, self.nkv, self.hd, self.scale, cache.page_table,
-                              cache.page_size, ctx.positions, ctx.tok_slot, self.ks, self.st, self.bs,
-                              self.init_blocks, self.topk, self.window_blocks, self.dense_len, ctx.max_pos,
-                              sel_blocks, sel_count, scratch=scratch)
+            # the reference times its two selection stages apart (minicpm4_attn.cuh:107-202); here they are one call
+            with ctx.timed("attn_select"):
+                ops.sparse_select(q, cache.streams["ck"], self.nh, self.nkv, self.hd, self.scale, cache.page_table,
+                                  cache.page_size, ctx.positions, ctx.tok_slot, self.ks, self.st, self.bs,
+                                  self.init_blocks, self.topk, self.window_blocks, self.dense_len, ctx.max_pos,
+                                  sel_blocks, sel_count, scratch=scratch)
             sel = (sel_blocks, sel_count, self.bs, self.window_blocks)
         return self.attend_and_project(q, ctx, cache, sel, defer_last=defer_last)

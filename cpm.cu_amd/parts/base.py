@@ -94,6 +94,17 @@ class Runtime:
     page_size: int = 64           # tokens a cache page
 
 
+class _NoTimer:
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_TIMER = _NoTimer()
+
+
 @dataclass
 class StepContext:
     """One step's batch as every part sees it: packed tokens of several sequences."""
@@ -114,6 +125,14 @@ class StepContext:
     logit_rows: Optional[torch.Tensor] = None     # int32 [R]: packed token rows whose logits are wanted
     extras: Dict[str, object] = field(default_factory=dict)   # what kernels derive from the batch once a step
     perf: Optional[object] = None                 # label-keyed timers (utils.perf.PerfTimers) when switched on
+
+    def timed(self, label: str):
+        """A context manager that times the GPU work inside it under ``prefill_<label>`` or ``decode_<label>``
+        while the timers are switched on, and does nothing otherwise.  The reference's labels make the same
+        distinction (src/model/minicpm4/minicpm4_layer.cuh:46-83, minicpm4_attn.cuh:107-202)."""
+        if self.perf is None or not self.perf.enabled:
+            return _NO_TIMER
+        return self.perf.gpu(("decode_" if self.single_token else "prefill_") + label)
 
 
 class DeferredBranch:

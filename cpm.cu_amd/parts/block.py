@@ -11,7 +11,7 @@ from __future__ import annotations
 from typing import List, Optional
 
 from ..cache.paged import CacheView
-from .base import (BLOCKS, Block, FeedForward, Mixer, Norm, Part, ResidualStream, StepContext, branch_tensor,
+from .base import (BLOCKS, Block, DeferredBranch, FeedForward, Mixer, Norm, Part, ResidualStream, StepContext, branch_tensor,
                    forward_declares)
 
 
@@ -39,11 +39,14 @@ class PreNormBlock(Block):
         row factor and that factor's ingredients."""
         if not norm.takes_deferred_branch:
             branch = branch_tensor(branch)
-        if deferred:
-            hs = norm.forward_unscaled(x, branch, branch_scale, ctx, tag="block.h")
-            if hs is not None:
-                return hs
-        return norm.forward(x, branch, branch_scale, ctx, tag="block.h"), None
+        # a norm that takes a branch's last product over runs it in the same kernel: the label says so
+        label = "norm+" + branch.tag.split(".")[-1] if isinstance(branch, DeferredBranch) else "norm"
+        with ctx.timed(label):
+            if deferred:
+                hs = norm.forward_unscaled(x, branch, branch_scale, ctx, tag="block.h")
+                if hs is not None:
+                    return hs
+            return norm.forward(x, branch, branch_scale, ctx, tag="block.h"), None
 
     def _mix(self, stream, ctx, cache, writes_cache):
         n = stream.x.shape[0]
@@ -64,16 +67,10 @@ class PreNormBlock(Block):
         return self.feed_forward.forward(h, ctx, **kw)
 
     def forward(self, stream: ResidualStream, ctx: StepContext, cache: Optional[CacheView], writes_cache: bool = True):
-        if ctx.perf is not None and ctx.perf.enabled:
-            # the reference's timer labels distinguish prefill from decode and attention from feed-forward
-            # (src/model/minicpm4/minicpm4_layer.cuh:46-83)
-            phase = "decode" if ctx.single_token else "prefill"
-            with ctx.perf.gpu(f"{phase}_attn"):
-                a = self._mix(stream, ctx, cache, writes_cache)
-            with ctx.perf.gpu(f"{phase}_ffn"):
-                stream.pending = self._feed(stream, a, ctx)
-            stream.pending_scale = self.residual_scale
-            return
-        a = self._mix(stream, ctx, cache, writes_cache)
-        stream.pending = self._feed(stream, a, ctx)
+        # the reference's timer labels distinguish prefill from decode and attention from feed-forward
+        # (src/model/minicpm4/minicpm4_layer.cuh:46-83); the parts inside time their own kernels by class
+        with ctx.timed("attn"):
+            a = self._mix(stream, ctx, cache, writes_cache)
+        with ctx.timed("ffn"):
+            stream.pending = self._feed(stream, a, ctx)
         stream.pending_scale = self.residual_scale

@@ -32,7 +32,9 @@ class GatedFFN(FeedForward):
     can_defer_last = True
 
     def forward(self, h: torch.Tensor, ctx: StepContext, row_scale=None, defer_last: bool = False):
-        act = self.gate_up.forward_gated(h, ctx, "ffn.gate_up", row_scale=row_scale)
+        with ctx.timed("ffn_gate_up"):
+            act = self.gate_up.forward_gated(h, ctx, "ffn.gate_up", row_scale=row_scale)
         if defer_last and self.down.defers(act):
             return DeferredBranch(self.down, act, ctx, "ffn.down")
-        return self.down.forward(act, ctx, "ffn.down", out_dtype=torch.float32, partials=True)
+        with ctx.timed("ffn_down"):
+            return self.down.forward(act, ctx, "ffn.down", out_dtype=torch.float32, partials=True)

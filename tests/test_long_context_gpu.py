@@ -193,14 +193,14 @@ class _Ctx:
 
 
 @pytest.mark.parametrize("n_tokens,start", [(1100, 0), (16500, 0), (2048, 14000), (700, 3000)])
-@pytest.mark.parametrize("nh,nkv,hd", [(8, 2, 32), (32, 2, 128)])
+@pytest.mark.parametrize("nh,nkv,hd", [(8, 2, 32), (32, 2, 128), (4, 1, 128)])
 def test_prompt_attention_of_long_prompts_through_the_dispatcher(n_tokens, start, nh, nkv, hd):
     """Whole prompts on either side of the sizes where the dispatcher changes the kernel's shape (1,024 and
     16,384 tokens), and chunks that continue a long sequence: tokens at the edges of tiles, pages and the
     prompt against the float64 reference."""
     from cpmcu_amd import ops
-    if n_tokens > 4096 and hd == 128:
-        pytest.skip("the small head size covers this length")
+    if n_tokens > 4096 and hd == 128 and nh > 4:
+        pytest.skip("this length at the head size of 128 runs with 4 heads (the next parameters)")
     L = start + n_tokens
     K, V, kpool, vpool, table = long_paged(L, nkv, hd, seed=n_tokens + hd)
     positions = list(range(start, L))
