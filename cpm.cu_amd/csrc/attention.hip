@@ -10,7 +10,9 @@
 //
 // Formula (reference: src/model/attn.cuh:200-227, src/flash_attn/flash_api.hpp:294-394):
 // s_j = (q.k_j) * scale for keys j <= position of the query, softmax over j in
-// float, out = sum_j p_j v_j; query head h reads kv head h / (nh/nkv).
+// float, out = sum_j p_j v_j; query head h reads kv head h / (nh/nkv).  With head_slopes (one number a query
+// head) the score of key j for the query at position p is lowered by slope * (p - j): the seam for position
+// encodings that bias scores instead of rotating vectors (the reference has none).
 #include "common.h"
 #include "no_alloc.h"
 
@@ -20,7 +22,8 @@ template <typename T>
 __global__ __launch_bounds__(64) void attention_paged_kernel(
     const T* __restrict__ q, T* __restrict__ out, const T* __restrict__ kpool, const T* __restrict__ vpool,
     PagedView pv, const int* __restrict__ positions, const int* __restrict__ tok_slot, int nh, int nkv, int hd,
-    float scale, const int* __restrict__ sel_blocks, const int* __restrict__ sel_count, int max_sel, int block_size) {
+    float scale, const int* __restrict__ sel_blocks, const int* __restrict__ sel_count, int max_sel, int block_size,
+    const float* __restrict__ head_slopes) {
     __shared__ float qs[256];
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int g = h / (nh / nkv);
@@ -31,6 +34,8 @@ __global__ __launch_bounds__(64) void attention_paged_kernel(
     const int nd = (hd + 63) / 64;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, l = 0.f;
+    // a position encoding that biases the scores by distance: s_j -= slope[head] * (position - j)
+    const float slope = head_slopes ? head_slopes[h] : 0.f;
 
     int n_seg = 1;
     const int* sel = nullptr;
@@ -57,7 +62,7 @@ __global__ __launch_bounds__(64) void attention_paged_kernel(
                 const T* kr = kpool + key_index(row, g, nkv, hd);
                 float dot = 0.f;
                 for (int d = 0; d < hd; ++d) dot += qs[d] * to_f32(kr[key_d_offset(d)]);
-                s = dot * scale;
+                s = dot * scale - slope * (float)(pos - j);
             }
             const float m_new = fmaxf(m, wave_max(s));
             const float p = valid ? expf(s - m_new) : 0.f;
@@ -90,7 +95,8 @@ extern "C" const char* cpmcu_attention_plain(const void* q, void* out, int dtype
                                              float scale, const void* kpool, const void* vpool,
                                              const int* page_table, int table_width, int page_size,
                                              const int* positions, const int* tok_slot, const int* sel_blocks,
-                                             const int* sel_count, int max_sel, int block_size, hipStream_t stream) {
+                                             const int* sel_count, int max_sel, int block_size,
+                                             const float* head_slopes, hipStream_t stream) {
     CPMCU_REQUIRE(n > 0 && nh > 0 && nkv > 0 && hd > 0, "attention: empty shape n=%d heads=%d kv_heads=%d head_dim=%d",
                   n, nh, nkv, hd);
     CPMCU_REQUIRE(nh % nkv == 0, "attention: %d heads are not a multiple of %d kv heads", nh, nkv);
@@ -102,12 +108,13 @@ extern "C" const char* cpmcu_attention_plain(const void* q, void* out, int dtype
     if (dtype == CPMCU_F32)
         attention_paged_kernel<float><<<grid, 64, 0, stream>>>((const float*)q, (float*)out, (const float*)kpool,
                                                                (const float*)vpool, pv, positions, tok_slot, nh, nkv,
-                                                               hd, scale, sel_blocks, sel_count, max_sel, block_size);
+                                                               hd, scale, sel_blocks, sel_count, max_sel, block_size,
+                                                               head_slopes);
     else if (dtype == CPMCU_BF16)
         attention_paged_kernel<bf16_t><<<grid, 64, 0, stream>>>((const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kpool,
                                                                 (const bf16_t*)vpool, pv, positions, tok_slot, nh,
                                                                 nkv, hd, scale, sel_blocks, sel_count, max_sel,
-                                                                block_size);
+                                                                block_size, head_slopes);
     else
         CPMCU_FAIL("attention: unknown dtype %d", dtype);
     CPMCU_LAUNCH_CHECK("attention_plain");

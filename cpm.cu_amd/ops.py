@@ -230,8 +230,9 @@ def attention_plain(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hd: i
                     kpool: torch.Tensor, vpool: torch.Tensor, page_table: torch.Tensor, page_size: int,
                     positions: torch.Tensor, tok_slot: torch.Tensor,
                     sel_blocks: Optional[torch.Tensor] = None, sel_count: Optional[torch.Tensor] = None,
-                    block_size: int = 0):
-    """Causal GQA attention of n query tokens over their sequences' cached keys (plain kernel)."""
+                    block_size: int = 0, head_slopes: Optional[torch.Tensor] = None):
+    """Causal GQA attention of n query tokens over their sequences' cached keys (plain kernel).  head_slopes
+    (float32 [nh]): the score of key j for the query at position p is lowered by head_slopes[h] * (p - j)."""
     _need(q, "attention q", shape=(None, nh * hd))
     n = q.shape[0]
     _need(out, "attention out", q.dtype, (n, nh * hd))
@@ -245,10 +246,12 @@ def attention_plain(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hd: i
         _need(sel_count, "attention block counts", torch.int32, (n, nkv))
         _need(sel_blocks, "attention block list", torch.int32, (n, nkv, None))
         max_sel = sel_blocks.shape[2]
+    if head_slopes is not None:
+        _need(head_slopes, "attention head slopes", torch.float32, (nh,))
     _check(_fn("attention", "cpmcu_attention_plain")(
         _p(q), _p(out), c_int(_code(q)), c_int(n), c_int(nh), c_int(nkv), c_int(hd), c_float(scale), _p(kpool),
         _p(vpool), _p(page_table), c_int(page_table.shape[1]), c_int(page_size), _p(positions), _p(tok_slot),
-        _p(sel_blocks), _p(sel_count), c_int(max_sel), c_int(block_size), _stream()))
+        _p(sel_blocks), _p(sel_count), c_int(max_sel), c_int(block_size), _p(head_slopes), _stream()))
 
 
 MFMA_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128)
@@ -708,8 +711,14 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, alpha: float = 1
 
 
 def attention(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, ctx,
-              sel_blocks=None, sel_count=None, block_size=0, window_blocks=0):
-    """Attention of the step's queries over the cache, with the kernel that suits the step; writes ``out``."""
+              sel_blocks=None, sel_count=None, block_size=0, window_blocks=0, head_slopes=None):
+    """Attention of the step's queries over the cache, with the kernel that suits the step; writes ``out``.
+    head_slopes (float32 [nh], a position encoding's bias of the scores by distance) is taken by the plain
+    kernel only, in both element types."""
+    if head_slopes is not None:
+        attention_plain(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, ctx.positions, ctx.tok_slot,
+                        sel_blocks, sel_count, block_size, head_slopes)
+        return
     if sel_count is None and not ctx.single_token and attention_mfma_ok(q, hd, page_size):
         r, nw = attention_prefill_shape(q.shape[0], nh, nkv, hd)
         tpw = attention_prefill_tokens_per_wave(nh, nkv, r)

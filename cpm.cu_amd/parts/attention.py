@@ -57,7 +57,7 @@ class GQAAttention(Mixer):
 
     def reserve_workspace(self, ws, rt: Runtime, max_step_tokens: int, max_slots: int):
         # the q/k/v weight in the fused decode kernel's order, if any step of this engine can run that kernel
-        plain_rotation = self.position is None or self.position.rotary_params() is not None
+        plain_rotation = self._kernel_rotates()
         if (self._qkv_fused is None and plain_rotation and rt.dtype == torch.bfloat16 and self.qkv.tiled is not None
                 and self.hd % 16 == 0 and self.hidden_size % 8 == 0 and rt.page_size % 32 == 0):
             self._qkv_fused = ops.qkv_rope_weight(self.qkv.weight, self.nh, self.nkv, self.hd)
@@ -73,10 +73,16 @@ class GQAAttention(Mixer):
         w = self.nkv * self.hd
         return CacheNeeds(streams=(("k", StreamSpec(w)), ("v", StreamSpec(w))))
 
+    def _kernel_rotates(self) -> bool:
+        """Whether the projection kernels do all that the position encoding asks of q and k: a rotate-half
+        rotation, or nothing (no encoding, or one that only biases the scores)."""
+        return (self.position is None or self.position.rotary_params() is not None
+                or not self.position.rewrites_vectors())
+
     # -- steps of forward, so that a subclass can put its own between them --
     def _fused_projection(self, n: int, dtype, cache: Optional[CacheView], writes_cache: bool) -> bool:
         """Decode steps: projection, rotation and cache write in one kernel (one kernel of the chain less)."""
-        plain_rotation = self.position is None or self.position.rotary_params() is not None
+        plain_rotation = self._kernel_rotates()
         return (writes_cache and cache is not None and plain_rotation and n <= ops.QKV_ROPE_MAX_ROWS
                 and dtype == torch.bfloat16 and self.qkv.tiled is not None and self.hd % 16 == 0
                 and self.hidden_size % 8 == 0 and cache.page_size % 32 == 0)
@@ -91,7 +97,7 @@ class GQAAttention(Mixer):
         then also writes the compressed keys that the step's tokens complete."""
         n = h.shape[0]
         nh, nkv, hd = self.nh, self.nkv, self.hd
-        plain_rotation = self.position is None or self.position.rotary_params() is not None
+        plain_rotation = self._kernel_rotates()
         if self._fused_projection(n, h.dtype, cache, writes_cache):
             if self._qkv_fused is None:           # a part used outside an engine (reserve_workspace makes it)
                 self._qkv_fused = ops.qkv_rope_weight(self.qkv.weight, nh, nkv, hd)
@@ -107,7 +113,7 @@ class GQAAttention(Mixer):
         qkv = self.qkv.forward(h, ctx, "attn.qkv", rows=None if writes_cache else nh * hd, partials=plain_rotation)
         rot = self.position.rotary_params() if self.position is not None else None
         inv_freq, mag = (rot if rot is not None else (None, 1.0))
-        if self.position is not None and rot is None:
+        if self.position is not None and rot is None and self.position.rewrites_vectors():
             q3 = qkv[:, :nh * hd].unflatten(1, (nh, hd))
             k3 = qkv[:, nh * hd:(nh + nkv) * hd].unflatten(1, (nkv, hd)) if writes_cache else None
             self.position.apply(q3, k3, ctx)
@@ -124,9 +130,11 @@ class GQAAttention(Mixer):
         output projection."""
         sel_blocks, sel_count, bs, window_blocks = sel if sel is not None else (None, None, 0, 0)
         out = ctx.ws.get("attn.out", tuple(q.shape), q.dtype)
+        slopes = self.position.score_bias() if self.position is not None else None
         with ctx.timed("attn_core"):
             ops.attention(q, out, self.nh, self.nkv, self.hd, self.scale, cache.streams["k"], cache.streams["v"],
-                          cache.page_table, cache.page_size, ctx, sel_blocks, sel_count, bs, window_blocks)
+                          cache.page_table, cache.page_size, ctx, sel_blocks, sel_count, bs, window_blocks,
+                          head_slopes=slopes)
         if defer_last and self.o.defers(out):
             return DeferredBranch(self.o, out, ctx, "attn.o")
         with ctx.timed("attn_o"):

@@ -10,7 +10,8 @@ Kinds of parts and what each must provide:
 * ``Norm``:      forward(x, branch, branch_scale, ctx, rows=None) -> normed [n or R, H]
                  (adds ``branch_scale * branch`` into the float residual ``x`` first)
 * ``PositionEncoding``: rotary_params() -> (inv_freq, magnitude) or None, and
-                 apply(q, k, ctx) for encodings that are not a plain rotation
+                 apply(q, k, ctx) for encodings that are not a plain rotation, and/or
+                 score_bias() -> per-head slopes for encodings that bias the scores by distance
 * ``Mixer``:     cache_needs() and forward(h, ctx, cache, writes_cache) -> branch [n, H] or [P, n, H]
 * ``FeedForward``: forward(h, ctx) -> branch [n, H] or [P, n, H]
 * ``Block``:     forward(stream, ctx, cache, writes_cache): the arrangement of the above
@@ -248,8 +249,18 @@ class PositionEncoding(Part):
 
     def apply(self, q: torch.Tensor, k: Optional[torch.Tensor], ctx: StepContext):
         """Encode positions into q [n, heads, hd] and k [n, kv_heads, hd] in place (used when
-        rotary_params() is None)."""
+        rotary_params() is None and a subclass defines it)."""
         raise NotImplementedError
+
+    def score_bias(self) -> Optional[torch.Tensor]:
+        """float32 [heads] on the device, or None: an encoding that lowers the score of key j for the query at
+        position p by slope[head] * (p - j) instead of (or beside) changing q and k.  The attention kernels
+        take it as it is; nothing about positions is then stored in the cache."""
+        return None
+
+    def rewrites_vectors(self) -> bool:
+        """Whether ``apply`` is this encoding's own (an encoding that only biases scores leaves it out)."""
+        return type(self).apply is not PositionEncoding.apply
 
 
 class Mixer(Part):

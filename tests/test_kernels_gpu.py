@@ -445,6 +445,44 @@ def test_prompt_attention_from_position_zero_and_continued(nh, nkv, hd):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,hd", [(6, 2, 48), (5, 1, 16)])
+def test_attention_with_a_distance_bias(nh, nkv, hd, dtype):
+    """head_slopes: the score of key j for the query at p is lowered by slope[head] * (p - j).  Checked against
+    a library attention with that bias as its mask; a slope that large for one head that only the nearest keys
+    count shows a wrong sign or a wrong head at once."""
+    from cpmcu_amd import ops
+    page = 64
+    lens = [200, 33]
+    ks, vs, kpool, vpool, table = paged_setup(lens, nkv, hd, page, dtype, seed=hd + 1)
+    positions = list(range(150, 200)) + [32, 0]
+    seq_of = [0] * 50 + [1, 1]
+    n = len(positions)
+    q = rnd(n, nh, hd, seed=6, dtype=dtype)
+    slopes = torch.tensor([0.0, 0.01, 0.3, 12.0, 0.05, 1.0][:nh], dtype=torch.float32)
+    G = nh // nkv
+    ref = torch.empty(n, nh, hd, dtype=torch.float64)
+    for t, (p, s) in enumerate(zip(positions, seq_of)):
+        k, v = ks[s][:p + 1], vs[s][:p + 1]                      # [keys, nkv, hd]
+        dist = (p - torch.arange(p + 1, dtype=torch.float64))
+        mask = (-slopes.double()[:, None] * dist[None, :])[:, None, :]            # [head, 1, key]
+        ref[t] = F.scaled_dot_product_attention(q[t].double().cpu()[:, None, :], k.repeat_interleave(G, 1).transpose(0, 1),
+                                                v.repeat_interleave(G, 1).transpose(0, 1), attn_mask=mask)[:, 0]
+    out = torch.empty(n, nh * hd, dtype=dtype, device=DEV)
+    ops.attention_plain(q.view(n, -1), out, nh, nkv, hd, hd ** -0.5, kpool, vpool, table, page,
+                        torch.tensor(positions, dtype=torch.int32, device=DEV),
+                        torch.tensor(seq_of, dtype=torch.int32, device=DEV), head_slopes=slopes.to(DEV))
+    tol = 2e-6 if dtype == torch.float32 else 2 ** -7
+    assert float((out.double().cpu().view(n, nh, hd) - ref).abs().max()) <= tol
+    # the head with slope 12 sees (almost) only the query's own position: its output is that position's value
+    own = torch.stack([vs[s][p, 3 // G] for p, s in zip(positions, seq_of)])
+    assert float((out.double().cpu().view(n, nh, hd)[:, 3] - own).abs().max()) < 0.02
+    with pytest.raises(ops.KernelError, match="head slopes"):
+        ops.attention_plain(q.view(n, -1), out, nh, nkv, hd, hd ** -0.5, kpool, vpool, table, page,
+                            torch.tensor(positions, dtype=torch.int32, device=DEV),
+                            torch.tensor(seq_of, dtype=torch.int32, device=DEV), head_slopes=slopes[:2].to(DEV))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_attention_finds_one_far_key_among_hundreds(dtype):
     """One key far back is made to stand out: the output must be its value (a kernel that skips or misplaces
     a page, or mixes up the transposed values, fails this)."""

@@ -1,9 +1,11 @@
-"""Parts defined here, outside the package: a feed-forward that routes every token to one of several experts
-and a position encoding that rotates interleaved pairs.  They are registered, chosen layer by layer by a toy
-configuration, built from a model folder and stepped; the package's files stay as they are (GPU).
+"""Parts defined here, outside the package: a feed-forward that routes every token to one of several experts,
+a position encoding that rotates interleaved pairs, and one that rotates nothing and lowers the scores by
+distance instead.  They are registered, chosen layer by layer by a toy configuration, built from a model
+folder and stepped; the package's files stay as they are (GPU).
 
-Neither is a model of anyone's: the experts are the package's own gated feed-forwards behind a softmax router
-with one winner, the position encoding is the rotation of the pairs (2c, 2c+1) instead of (c, c + hd/2)."""
+None is a model of anyone's: the experts are the package's own gated feed-forwards behind a softmax router
+with one winner, the first position encoding is the rotation of the pairs (2c, 2c+1) instead of (c, c + hd/2),
+the second subtracts slope[head] * distance from every score."""
 from dataclasses import dataclass
 from typing import Any, Dict
 
@@ -35,6 +37,8 @@ def _define():
 
         def bind(self, tensors, rt):
             self.rt = rt
+
+        graph_capturable = False      # which experts run is read on the host, step by step
 
         def forward(self, h, ctx):
             logits = self.router.forward(h, ctx, "toy.router", out_dtype=torch.float32)
@@ -77,6 +81,19 @@ def _define():
                 x[..., 0::2] = (a * cs - b * sn).to(x.dtype)
                 x[..., 1::2] = (a * sn + b * cs).to(x.dtype)
 
+    class DistanceBias(PositionEncoding):
+        """No rotation: the score of key j for the query at p is lowered by slope[head] * (p - j), slopes
+        first, first / ratio, first / ratio^2 ... over the heads.  Only ``score_bias`` is defined."""
+
+        def __init__(self, num_heads: int, first: float, ratio: float):
+            self.slopes = [first / ratio ** h for h in range(num_heads)]
+
+        def bind(self, tensors, rt):
+            self.device_slopes = torch.tensor(self.slopes, dtype=torch.float32, device=rt.device)
+
+        def score_bias(self):
+            return self.device_slopes
+
     @dataclass(frozen=True)
     class ToyConfig(ModelConfig):
         vocab_size: int = 0
@@ -86,7 +103,7 @@ def _define():
         head_dim: int = 0
         intermediate_size: int = 0
         n_experts: int = 0
-        layer_kinds: tuple = ()                  # per layer: "routed" or "dense"
+        layer_kinds: tuple = ()                  # per layer: "routed", "dense" or "biased"
         rope_theta: float = 10000.0
         rms_norm_eps: float = 1e-5
         max_position_embeddings: int = 128
@@ -117,14 +134,19 @@ def _define():
 
     FEED_FORWARDS.register("toy_top1_experts", Top1Experts)
     POSITION_ENCODINGS.register("toy_interleaved_rotary", InterleavedRotary)
+    POSITION_ENCODINGS.register("toy_distance_bias", DistanceBias)
 
     def build(cfg: ToyConfig):
         layers = []
         for i, kind in enumerate(cfg.layer_kinds):
             p = f"layers.{i}."
             routed = kind == "routed"
-            position = POSITION_ENCODINGS.build("toy_interleaved_rotary" if routed else "rope", head_dim=cfg.head_dim,
-                                                theta=cfg.rope_theta)
+            if kind == "biased":
+                position = POSITION_ENCODINGS.build("toy_distance_bias", num_heads=cfg.num_attention_heads, first=0.5,
+                                                    ratio=2.0)
+            else:
+                position = POSITION_ENCODINGS.build("toy_interleaved_rotary" if routed else "rope",
+                                                    head_dim=cfg.head_dim, theta=cfg.rope_theta)
             ff = (FEED_FORWARDS.build("toy_top1_experts", prefix=p + "moe.", hidden_size=cfg.hidden_size,
                                       intermediate_size=cfg.intermediate_size, n_experts=cfg.n_experts) if routed
                   else FEED_FORWARDS.build("gated_silu", prefix=p + "mlp.", hidden_size=cfg.hidden_size,
@@ -174,11 +196,19 @@ def plain_toy(raw, w, toks):
     for i, kind in enumerate(raw["layer_kinds"]):
         p = f"layers.{i}."
         a = F.rms_norm(x, (x.shape[-1],), W[p + "norm1.weight"], eps)
-        q = rotate((a @ W[p + "attn.q_proj.weight"].T).view(n, nh, hd), kind == "routed")
-        k = rotate((a @ W[p + "attn.k_proj.weight"].T).view(n, nkv, hd), kind == "routed")
+        q = (a @ W[p + "attn.q_proj.weight"].T).view(n, nh, hd)
+        k = (a @ W[p + "attn.k_proj.weight"].T).view(n, nkv, hd)
         v = (a @ W[p + "attn.v_proj.weight"].T).view(n, nkv, hd)
-        o = F.scaled_dot_product_attention(q.transpose(0, 1), k.repeat_interleave(nh // nkv, 1).transpose(0, 1),
-                                           v.repeat_interleave(nh // nkv, 1).transpose(0, 1), is_causal=True)
+        kk, vv = k.repeat_interleave(nh // nkv, 1).transpose(0, 1), v.repeat_interleave(nh // nkv, 1).transpose(0, 1)
+        if kind == "biased":
+            dist = (pos[:, None] - pos[None, :])                                      # [query, key]
+            slopes = torch.tensor([0.5 / 2.0 ** h for h in range(nh)], dtype=torch.float64)
+            mask = torch.where(dist >= 0, -slopes[:, None, None] * dist, float("-inf"))   # [head, query, key]
+            o = F.scaled_dot_product_attention(q.transpose(0, 1), kk, vv, attn_mask=mask)
+        else:
+            o = F.scaled_dot_product_attention(rotate(q, kind == "routed").transpose(0, 1),
+                                               rotate(k, kind == "routed").repeat_interleave(nh // nkv, 1).transpose(0, 1),
+                                               vv, is_causal=True)
         x = x + o.transpose(0, 1).reshape(n, nh * hd) @ W[p + "attn.o_proj.weight"].T
         f = F.rms_norm(x, (x.shape[-1],), W[p + "norm2.weight"], eps)
         if kind == "routed":
@@ -205,7 +235,7 @@ def test_routed_feed_forward_and_another_position_encoding_are_chosen_per_layer(
     try:
         raw = {"architectures": [ARCH], "vocab_size": 70, "hidden_size": 48, "num_attention_heads": 4,
                "num_key_value_heads": 2, "head_dim": 16, "intermediate_size": 40, "n_experts": 3,
-               "layer_kinds": ["routed", "dense", "routed"], "rope_theta": 500.0, "rms_norm_eps": 1e-5,
+               "layer_kinds": ["routed", "dense", "biased", "routed"], "rope_theta": 500.0, "rms_norm_eps": 1e-5,
                "max_position_embeddings": 64}
         write_model_dir(ToyConfig.from_dict(raw), str(tmp_path), seed=7, std=0.15, norm_std=0.1)
         w = load_file(str(tmp_path / "model.safetensors"))
@@ -214,7 +244,13 @@ def test_routed_feed_forward_and_another_position_encoding_are_chosen_per_layer(
         from safetensors.torch import save_file
         w = {k: (v * 5 if "router" in k else v).contiguous() for k, v in w.items()}
         save_file(w, str(tmp_path / "model.safetensors"))
-        eng = Engine.from_dir(str(tmp_path), EngineOptions(dtype=dtype, max_tokens=256, max_slots=2))
+        # graphs are asked for; the routed feed-forward says that it cannot be captured, so steps run eagerly
+        eng = Engine.from_dir(str(tmp_path), EngineOptions(dtype=dtype, max_tokens=256, max_slots=2, hip_graph=True))
+        assert not eng.uses_graph
+        # the biased layer's mixer goes through the fused projection kernel in bfloat16 (nothing to rotate) and
+        # hands the slopes to the attention
+        assert eng.model.layers[2].mixer._kernel_rotates() and eng.model.layers[2].mixer.position.score_bias() is not None
+        assert not eng.model.layers[0].mixer._kernel_rotates()
         # A token whose router nearly ties may go to another expert in reduced precision, and it feeds the later
         # tokens' keys: the bfloat16 comparison stops before the first such token, and the tokens are drawn from
         # the first seed that leaves it a long stretch.
@@ -244,3 +280,4 @@ def test_routed_feed_forward_and_another_position_encoding_are_chosen_per_layer(
         unregister_architecture(ARCH)
         FEED_FORWARDS.unregister("toy_top1_experts")
         POSITION_ENCODINGS.unregister("toy_interleaved_rotary")
+        POSITION_ENCODINGS.unregister("toy_distance_bias")
