@@ -280,3 +280,24 @@ def test_an_architecture_brings_its_own_front_end_flags(tmp_path):
         unregister_architecture("FlagToyForTests")
     with pytest.raises(SystemExit):
         create_cli_parser().parse_args(["--toy-depth", "3"])
+
+
+def test_the_package_description_names_every_subpackage_and_the_kernel_sources():
+    """pyproject.toml installs the folder `cpm.cu_amd` as `cpmcu_amd`: every folder with an __init__.py is
+    listed, the HIP sources are package data, and the scripts point at functions that exist."""
+    import importlib
+    import os
+    import tomli
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    with open(os.path.join(root, "pyproject.toml"), "rb") as f:
+        meta = tomli.load(f)
+    tool = meta["tool"]["setuptools"]
+    src = os.path.join(root, tool["package-dir"]["cpmcu_amd"])
+    found = {"cpmcu_amd"} | {"cpmcu_amd." + d for d in os.listdir(src)
+                             if os.path.isfile(os.path.join(src, d, "__init__.py"))}
+    assert set(tool["packages"]) == found
+    assert any(f.endswith(".hip") for f in os.listdir(os.path.join(src, "csrc")))
+    assert tool["package-data"]["cpmcu_amd.csrc"] == ["*.hip", "*.h"]
+    for target in meta["project"]["scripts"].values():
+        module, func = target.split(":")
+        assert callable(getattr(importlib.import_module(module), func))
