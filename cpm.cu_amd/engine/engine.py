@@ -184,7 +184,8 @@ class Engine:
         self._rehearsing = True
         try:
             s = self.acquire()
-            self.step([StepEntry(s, [0] * n_prompt, [n_prompt - 1])])
+            # token ids spread over the vocabulary (the product library sets itself up on ordinary rows)
+            self.step([StepEntry(s, [(7919 * i) % self.vocab_size for i in range(n_prompt)], [n_prompt - 1])])
             self.release(s)
             # kernels change with the number of rows at powers of two at most: those sizes and their successors
             sizes = {1}

@@ -86,6 +86,25 @@ def test_unequal_batches_one_after_another(model_dirs, references, name, dtype):
     assert not eng.cache.live
 
 
+@pytest.mark.parametrize("page", [32, 128])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_other_page_sizes(model_dirs, references, name, dtype, page):
+    """Pages of 32 and of 128 tokens (64 everywhere else): the same logits whole, token by token with graphs, and
+    in batches whose slots are used again."""
+    cfg, w, reqs, refs = references[name]
+    eng = engine_for(model_dirs, name, dtype, page_size=page, hip_graph=True, max_tokens=1536)
+    assert eng.cache.page_size == page
+    check(schedules.whole(eng, reqs), refs, dtype, f"whole, pages of {page}")
+    check(schedules.tail(eng, reqs, 32), refs, dtype, f"tail-32, pages of {page}")
+    got = schedules.batched(eng, reqs, WORK[name]["prompt"], BATCHES[:2])
+    check(got, refs, dtype, f"batched, pages of {page}")
+    got = schedules.batched(eng, reqs, WORK[name]["prompt"], BATCHES[2:])
+    check(got, refs, dtype, f"batched, slots used again, pages of {page}")
+    eng.cache.check()
+    assert not eng.cache.live
+
+
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_engine_without_the_second_copy_of_the_weights(model_dirs, references, name):
     """tiled_weights=False: the bfloat16 engine keeps the checkpoint's layout only, so decode steps go through the
