@@ -315,26 +315,43 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, l
     }
 }
 
-// bf16, I a multiple of 8: 8 columns a thread with 16-byte accesses
-__global__ void silu_mul_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, long n, int I) {
+// bf16, I a multiple of 8: 8 columns a thread with 16-byte accesses, U such pieces of a row in flight a thread
+// (the pieces of a thread lie a whole block apart, so every load of a wavefront is one contiguous KiB).  The
+// result is rounded to bfloat16, so the exponential and the reciprocal are the bare hardware instructions
+// (2^-22 relative; the 32-bit engine's kernel above keeps expf and a true division).
+template <int U>
+__global__ __launch_bounds__(256) void silu_mul_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out,
+                                                              long n, int I) {
     const int I8 = I / 8;
     const long total = n * I8;
-    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    const long base = (long)blockIdx.x * (256 * U) + threadIdx.x;
+    uint4 g4[U], u4[U];
+    long at[U];
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+        const long i = min(base + k * 256, total - 1);            // a piece beyond the end repeats the last one
         const long r = i / I8;
         const int c = (int)(i - r * I8) * 8;
-        const uint4 g4 = *(const uint4*)(gu + r * 2 * I + c);
-        const uint4 u4 = *(const uint4*)(gu + r * 2 * I + I + c);
-        const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, uw[4] = {u4.x, u4.y, u4.z, u4.w};
+        at[k] = r * I + c;
+        g4[k] = *(const uint4*)(gu + r * 2 * I + c);
+        u4[k] = *(const uint4*)(gu + r * 2 * I + I + c);
+    }
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+        if (base + k * 256 >= total) break;
+        const uint32_t gw[4] = {g4[k].x, g4[k].y, g4[k].z, g4[k].w}, uw[4] = {u4[k].x, u4[k].y, u4[k].z, u4[k].w};
         uint32_t ow[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const float g0 = __uint_as_float(gw[j] << 16), g1 = __uint_as_float(gw[j] & 0xffff0000u);
             const float u0 = __uint_as_float(uw[j] << 16), u1 = __uint_as_float(uw[j] & 0xffff0000u);
-            const bf16_t a = f32_to_bf16(g0 / (1.0f + expf(-g0)) * u0);
-            const bf16_t b = f32_to_bf16(g1 / (1.0f + expf(-g1)) * u1);
+            const float s0 = g0 * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g0));
+            const float s1 = g1 * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g1));
+            const bf16_t a = f32_to_bf16(s0 * u0);
+            const bf16_t b = f32_to_bf16(s1 * u1);
             ow[j] = (uint32_t)a.v | ((uint32_t)b.v << 16);
         }
-        *(uint4*)(out + r * I + c) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+        *(uint4*)(out + at[k]) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
     }
 }
 
@@ -342,8 +359,16 @@ extern "C" const char* cpmcu_silu_mul(const void* gu, void* out, int dtype, int 
     CPMCU_REQUIRE(n > 0 && I > 0, "silu_mul: empty shape n=%d I=%d", n, I);
     if (dtype == CPMCU_BF16 && I % 8 == 0 && (uintptr_t)gu % 16 == 0 && (uintptr_t)out % 16 == 0) {
         const long total8 = (long)n * (I / 8);
-        const int grid8 = (int)((total8 + 255) / 256 < 65535 * 8 ? (total8 + 255) / 256 : 65535 * 8);
-        silu_mul_bf16x8_kernel<<<grid8, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, n, I);
+        // many rows: 4 pieces a thread in flight; few: one, for more workgroups
+        if (total8 >= 4L * 256 * 2048) {
+            const long wgs = (total8 + 4 * 256 - 1) / (4 * 256);
+            CPMCU_REQUIRE(wgs <= 0x7fffffffL, "silu_mul: %d rows of %d columns exceed the launch grid", n, I);
+            silu_mul_bf16x8_kernel<4><<<(unsigned)wgs, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, n, I);
+        } else {
+            const long wgs = (total8 + 255) / 256;
+            CPMCU_REQUIRE(wgs <= 0x7fffffffL, "silu_mul: %d rows of %d columns exceed the launch grid", n, I);
+            silu_mul_bf16x8_kernel<1><<<(unsigned)wgs, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, n, I);
+        }
         CPMCU_LAUNCH_CHECK("silu_mul");
         return nullptr;
     }
@@ -466,17 +491,18 @@ __global__ __launch_bounds__(256) void rope_store_rows_kernel(
         const long kv_row = rows_s[lane >> 3];
         const int heads = nh + (write_kv ? nkv : 0);
         const bf16_t* row = qkv + t * width + 8 * piece;
-        // three heads' loads in flight at a time (a head beyond the last asks for the last once more)
-        for (int head0 = wave; head0 < heads; head0 += 12) {
-            ebf16x8_t a[3], b[3];
+        // UH heads' loads in flight at a time (a head beyond the last asks for the last once more)
+        constexpr int UH = 5;
+        for (int head0 = wave; head0 < heads; head0 += 4 * UH) {
+            ebf16x8_t a[UH], b[UH];
 #pragma unroll
-            for (int u = 0; u < 3; ++u) {
+            for (int u = 0; u < UH; ++u) {
                 const int head = min(head0 + 4 * u, heads - 1);
                 a[u] = *(const ebf16x8_t*)(row + (long)head * hd);
                 b[u] = *(const ebf16x8_t*)(row + (long)head * hd + half);
             }
 #pragma unroll
-            for (int u = 0; u < 3; ++u) {
+            for (int u = 0; u < UH; ++u) {
                 const int head = head0 + 4 * u;
                 if (head >= heads) break;
                 ebf16x8_t lo, hi;

@@ -298,6 +298,22 @@ def test_silu_mul(dtype, I):
     assert float((out.double() - ref).abs().max()) <= tol * float(ref.abs().max() + 1)
 
 
+def test_silu_mul_of_many_rows():
+    """Prompt chunks take the form with several pieces a thread in flight; the last workgroup's pieces run past
+    the end."""
+    from cpmcu_amd import ops
+    n, I = 1100, 16392
+    gu = rnd(n, 2 * I, dtype=torch.bfloat16, scale=3.0)
+    out = torch.full((n, I), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.silu_mul(gu, out)
+    ref = F.silu(gu[:, :I].float()) * gu[:, I:].float()
+    assert not bool(out.isnan().any())
+    assert float((out.float() - ref).abs().max()) <= 2 ** -8 * float(ref.abs().max() + 1)
+    # rows that differ everywhere: a wrong row or column offset cannot hide
+    assert torch.equal(out[-1], (F.silu(gu[-1, :I].float()) * gu[-1, I:].float()).to(torch.bfloat16)) or \
+        float((out[-1].float() - ref[-1]).abs().max()) <= 2 ** -8 * float(ref[-1].abs().max() + 1)
+
+
 # ---------------------------------------------------------------------------- attention over the paged cache
 def key_tiles(full):
     """[page tokens, kv heads, d] -> the cache's layout of keys: per chunk of 32 tokens and kv head two tiles of
