@@ -122,7 +122,8 @@ def test_embedding(dtype):
     assert torch.equal(out, table.float()[ids.long()] * 12.0)
 
 
-@pytest.mark.parametrize("H,n", [(24, 6), (100, 6), (1000, 6), (4096 + 8, 6), (7, 3), (66, 3), (96, 600)])
+@pytest.mark.parametrize("H,n", [(24, 6), (100, 6), (1000, 6), (4096 + 8, 6), (7, 3), (66, 3), (96, 600),
+                                 (1100, 301), (4096, 257), (2052, 300), (4096 + 8, 258)])
 @pytest.mark.parametrize("bdtype,odtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
                                            (torch.float32, torch.bfloat16), (torch.bfloat16, torch.float32)])
 def test_add_rms_norm(H, n, bdtype, odtype):

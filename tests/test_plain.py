@@ -146,7 +146,11 @@ def test_longrope_factor_stretches_the_positions_of_its_pair():
 
 def test_longrope_magnitude_is_a_number_known_in_closed_form():
     """Tiny B stretches 128 positions to 512: ln 4 / ln 128 = 2/7 exactly, so the magnitude is sqrt(9/7).
-    A natural logarithm of the wrong quantity (the factor lists, max/1, original/max) does not give this."""
+    A natural logarithm of the wrong quantity (the factor lists, max/1, original/max) does not give this.
+    Parity unpinned: the reference engine loads the frequencies only and leaves the magnitude out
+    (cpmcu/llm.py:189-192), and takes both from an installed package's model code, which this repository neither
+    imports nor reads; no file of the reference holds the number.  What is pinned here is the definition that
+    config.json's keys describe, in closed form; `rope_attention_scaling: false` gives the reference's engine."""
     assert P.rope_inv_freq(tiny.tiny_b())[1] == pytest.approx(1.1338934190276817, abs=1e-15)
     raw = tiny.tiny_b()
     raw["max_position_embeddings"] = 128 * 128          # stretched by the original length itself: sqrt(2)
