@@ -166,6 +166,9 @@ def main():
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--hip-graph", type=int, default=1)
+    ap.add_argument("--no-rehearse", action="store_true",
+                    help="build the engine without its rehearsal passes (a profile then holds the benchmark's own "
+                         "kernels only; the workspace grows during the warm-up steps instead)")
     ap.add_argument("--perf", action="store_true",
                     help="after the timed runs, a few eager steps with the engine's timers on: average ms by kernel "
                          "class (products / attention / selection / norms / head) on stderr and under 'timers'")
@@ -197,7 +200,7 @@ def main():
     per_seq = -(-(args.context + args.steps + args.warmup + 64) // 64) * 64
     eng = Engine.from_tensors(cfg, tensors, EngineOptions(
         dtype=args.dtype, max_tokens=max(max_b * per_seq, args.prefill_tokens + 64), max_slots=max_b,
-        max_step_tokens=max(args.prefill_tokens, 2048), device=dev, hip_graph=bool(args.hip_graph)))
+        max_step_tokens=max(args.prefill_tokens, 2048), device=dev, hip_graph=bool(args.hip_graph), rehearse=not args.no_rehearse))
     del tensors
     torch.cuda.synchronize()
     print(f"[bench] model ready in {time.time() - t0:.1f} s: {cfg.num_hidden_layers} layers, "
@@ -370,7 +373,7 @@ def other_scenarios(args, dev):
         new = 256
         eng = Engine.from_tensors(cfg, random_tensors(cfg, 0, device=dev), EngineOptions(
             dtype=args.dtype, max_tokens=sum(-(-(n + new) // 64) * 64 for n in lens), max_slots=64,
-            max_step_tokens=8192, device=dev, hip_graph=bool(args.hip_graph)))
+            max_step_tokens=8192, device=dev, hip_graph=bool(args.hip_graph), rehearse=not args.no_rehearse))
         prompts = [[int(t) for t in torch.randint(0, cfg.vocab_size, (n,), generator=g)] for n in lens]
         generate(eng, prompts[:4], 8)                                   # warm-up: kernels loaded, graphs of small batches
         outs = generate(eng, prompts, new)
@@ -411,7 +414,7 @@ def other_scenarios(args, dev):
     read_gbs = calibrate_read(dev)
     eng = Engine.from_tensors(cfg, random_tensors(cfg, 0, device=dev), EngineOptions(
         dtype=args.dtype, max_tokens=4 * 32768, max_slots=4, max_step_tokens=2048, device=dev,
-        hip_graph=bool(args.hip_graph)))
+        hip_graph=bool(args.hip_graph), rehearse=not args.no_rehearse))
     rec = {"metric": "MiniCPM4-8B shape with InfLLM-v2 at 32k context: decode tok/s at batch 1 after a 32,000-token prefill",
            "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
