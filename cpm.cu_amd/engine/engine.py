@@ -151,25 +151,32 @@ class Engine:
         free_now = torch.cuda.mem_get_info(self.device)[0] + (torch.cuda.memory_reserved(self.device)
                                                               - torch.cuda.memory_allocated(self.device))
         if options.max_tokens is None:
-            tokens = SequenceCache.tokens_for(needs, min(limit - held, free_now - (256 << 20)), max_slots, self.max_seq_len, page, self.dtype,
+            budget = min(limit - held, free_now - (256 << 20))
+            tokens = SequenceCache.tokens_for(needs, budget, max_slots, self.max_seq_len, page, self.dtype,
                                               self.max_step_tokens)
             if tokens == 0:
-                raise EngineMemoryError(self._memory_message(limit, total, plan(max_slots * page), max_slots * page))
+                raise EngineMemoryError(self._memory_message(limit, total, plan(max_slots * page), max_slots * page,
+                                                             free_now))
             self.max_tokens = tokens
         else:
             self.max_tokens = int(options.max_tokens)
-            if limit is not None and held + plan(self.max_tokens) > limit:
-                raise EngineMemoryError(self._memory_message(limit, total, plan(self.max_tokens), self.max_tokens))
+            over_limit = limit is not None and held + plan(self.max_tokens) > limit
+            if over_limit or plan(self.max_tokens) > free_now:
+                raise EngineMemoryError(self._memory_message(limit if over_limit else None, total,
+                                                             plan(self.max_tokens), self.max_tokens, free_now))
         self.cache = SequenceCache(needs, self.max_tokens, max_slots, self.max_seq_len, page, self.device, self.dtype,
                                    self.max_step_tokens)
         self.workspace.sealed = True
 
-    def _memory_message(self, limit: int, total: int, cache_bytes: int, tokens: int) -> str:
+    def _memory_message(self, limit: Optional[int], total: int, cache_bytes: int, tokens: int, free_now: int) -> str:
         gib = lambda b: f"{b / 2**30:.2f} GiB"
-        return (f"memory limit exceeded: weights {gib(self.weight_bytes)} + workspace {gib(self.workspace.bytes())} + "
-                f"cache {gib(cache_bytes)} (for {tokens} tokens) = "
-                f"{gib(self.weight_bytes + self.workspace.bytes() + cache_bytes)}, the limit is {gib(limit)} "
-                f"({self.options.memory_limit:.0%} of the device's {gib(total)})")
+        figure = (f"weights {gib(self.weight_bytes)} + workspace {gib(self.workspace.bytes())} + cache {gib(cache_bytes)} "
+                  f"(for {tokens} tokens) = {gib(self.weight_bytes + self.workspace.bytes() + cache_bytes)}")
+        if limit is None:
+            return (f"device memory exceeded: {figure}; weights and workspace are in place and the device has "
+                    f"{gib(free_now)} left for the cache")
+        return (f"memory limit exceeded: {figure}, the limit is {gib(limit)} "
+                f"({self.options.memory_limit:.0%} of the device's {gib(total)}; {gib(free_now)} of it are free for the cache)")
 
     def _rehearse(self, needs, max_slots: int):
         """One prompt pass of max_step_tokens tokens and decode passes of the largest and of small batches, on a

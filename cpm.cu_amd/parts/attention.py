@@ -177,6 +177,9 @@ class InfLLMv2Attention(GQAAttention):
                    for n in {1, min(few, max_step_tokens), min(few + 1, max_step_tokens), max_step_tokens})
         if need:
             ws.get("attn.sel_scores", (need,), torch.float32)
+        # the block lists of the largest step (a rehearsal pass at short positions never selects)
+        ws.get("attn.sel_blocks", (max_step_tokens, self.nkv, self.topk + self.window_blocks), torch.int32)
+        ws.get("attn.sel_count", (max_step_tokens, self.nkv), torch.int32)
 
     def cache_needs(self) -> CacheNeeds:
         w = self.nkv * self.hd

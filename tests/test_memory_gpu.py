@@ -64,6 +64,9 @@ def test_a_limit_that_weights_workspace_and_cache_exceed_is_refused_when_the_eng
     with pytest.raises(EngineMemoryError, match="memory limit exceeded"):
         Engine.from_dir(model_dirs["B"], EngineOptions(dtype="bfloat16", max_tokens=None, max_slots=4,
                                                        memory_limit=(mem["weight_bytes"] + 1000) / total_memory()))
+    # no limit given, but a cache that the device cannot hold: said at build too, not by the allocator later
+    with pytest.raises(EngineMemoryError, match=r"device memory exceeded: weights .* \+ workspace .* \+ cache .*left for"):
+        Engine.from_dir(model_dirs["B"], EngineOptions(dtype="bfloat16", max_tokens=2_000_000_000, max_slots=4))
     with pytest.raises(ValueError, match="max_tokens, or a memory_limit"):
         Engine.from_dir(model_dirs["B"], EngineOptions(dtype="bfloat16", max_tokens=None))
 
