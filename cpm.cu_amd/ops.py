@@ -495,6 +495,16 @@ class TiledWeight:
         self.data = wp.view(Np // 16, 16, Kp // 128, 4, 4, 8).permute(0, 2, 3, 4, 1, 5).contiguous()
         self.N, self.K = N, K
 
+    def first_rows(self, n: int) -> "TiledWeight":
+        """The same memory seen as the weight's first n rows (whole strips of 16, or all of it)."""
+        if n == self.N:
+            return self
+        if n <= 0 or n > self.N or n % 16:
+            raise KernelError(f"a tiled weight of {self.N} rows gives its first rows in whole strips of 16, not {n}")
+        view = object.__new__(TiledWeight)
+        view.data, view.N, view.K = self.data[:n // 16], n, self.K
+        return view
+
 
 
 
@@ -696,6 +706,9 @@ def library_gemm_ok(x: torch.Tensor, out_dtype: torch.dtype) -> bool:
 def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, alpha: float = 1.0, w_tiled=None):
     """out = alpha * x . w^T with the kernel that suits the element type and the number of rows."""
     M = x.shape[0]
+    if w is None and (w_tiled is None or M > SKINNY_MAX_ROWS and out.dtype == torch.bfloat16 and alpha == 1.0):
+        raise KernelError(f"linear: {M} rows need the weight in the checkpoint's layout, which this engine let go "
+                          f"(it was built for forward passes of at most {SKINNY_MAX_ROWS} tokens)")
     if x.dtype == torch.bfloat16 and x.shape[1] % 8 == 0:
         if M <= SKINNY_MAX_ROWS:
             gemm_skinny(x, w_tiled if w_tiled is not None else w, out, alpha)

@@ -57,6 +57,10 @@ class LMHead(Part):
         # the table in the decode product's layout (made here and not at bind: a tied table is bound by its owner)
         if self.tiled is None and rt.dtype == torch.bfloat16 and rt.tiled_weights:
             self.tiled = ops.TiledWeight(self.tied_to.table if self.tied_to is not None else self.weight)
+        # logits are float32: every product of the head goes through the re-laid copy, whatever the number of rows,
+        # so a head of its own lets the checkpoint's layout go (a tied head's table stays: the embedding reads it)
+        if self.tiled is not None and self.tied_to is None and self.hidden_size % 8 == 0:
+            self.weight = None
 
     def forward(self, y: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         w = self.tied_to.table if self.tied_to is not None else self.weight

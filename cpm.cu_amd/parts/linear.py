@@ -34,14 +34,24 @@ class Linear(Part):
         # a second copy laid out for the decode product (bf16 engine; costs the weight's size again)
         self.tiled = ops.TiledWeight(self.weight) if (rt.dtype == torch.bfloat16 and rt.tiled_weights) else None
 
+    def reserve_workspace(self, ws, rt: Runtime, max_step_tokens: int, max_slots: int):
+        # An engine whose forward passes never carry more rows than the decode product takes reads the re-laid
+        # copy only: the checkpoint's layout (what the library's many-row product and the 32-bit kernels read)
+        # is let go, which halves what the weights hold.
+        if self.tiled is not None and max_step_tokens <= ops.SKINNY_MAX_ROWS and self.in_features % 8 == 0:
+            self.weight = None
+
     def forward(self, x: torch.Tensor, ctx: StepContext, tag: str, out_dtype: Optional[torch.dtype] = None,
                 alpha: float = 1.0, rows: Optional[int] = None, partials: bool = False) -> torch.Tensor:
         """x [n, in] -> [n, out] (the first ``rows`` output features only, if given).  With ``partials`` the
         result may come as float32 partial sums [S, n, out] over slices of the input axis, for a consumer
         that adds them up (the norm and the position-encoding kernels do)."""
-        w = self.weight if rows is None else self.weight[:rows]
-        wt = self.tiled if rows is None else None
-        n, N = x.shape[0], w.shape[0]
+        if self.weight is not None:
+            w = self.weight if rows is None else self.weight[:rows]
+            wt = self.tiled if rows is None else None
+        else:                                     # the re-laid copy alone: its first strips serve the first rows
+            w, wt = None, (self.tiled if rows is None else self.tiled.first_rows(rows))
+        n, N = x.shape[0], (self.out_features if rows is None else rows)
         if partials and ops.skinny_ok(x):
             S = ops.skinny_split(n, N, self.in_features)
             if S > 1:

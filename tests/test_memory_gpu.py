@@ -95,3 +95,29 @@ def test_llm_sizes_its_cache_from_the_memory_limit_and_generates(model_dirs, nam
     llm.engine.cache.check()
     with pytest.raises(ValueError, match="exceeds maximum supported length"):
         llm.prefill(list(range(limit + 1)))
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_an_engine_of_short_passes_lets_the_checkpoint_layout_go(model_dirs, name):
+    """With forward passes of at most 32 tokens no product reads the weights in the checkpoint's layout: the linear
+    layers keep their re-laid copy only (and the fused q/k/v copy), the memory figure shows it, and prompts, cut
+    into passes of 32, and decode steps give the logits of the plain implementation."""
+    import plain_minicpm as plain
+    import schedules
+    from cpmcu_amd import Engine, EngineOptions
+    from cpmcu_amd.parts.linear import Linear
+    cfg, w = tiny.read_model(model_dirs[name])
+    full = Engine.from_dir(model_dirs[name], EngineOptions(dtype="bfloat16", max_tokens=1024, max_slots=3))
+    short = Engine.from_dir(model_dirs[name], EngineOptions(dtype="bfloat16", max_tokens=1024, max_slots=3,
+                                                            max_step_tokens=32, hip_graph=True))
+    linears = [p for p in short.model.all_parts() if isinstance(p, Linear)]
+    assert linears and all(p.weight is None and p.tiled is not None for p in linears)
+    assert all(p.weight is not None for p in full.model.all_parts() if isinstance(p, Linear))
+    assert short.memory_report()["weight_bytes"] < 0.8 * full.memory_report()["weight_bytes"]
+    reqs = {"x": tiny.random_tokens(150, cfg["vocab_size"], 31), "y": tiny.random_tokens(45, cfg["vocab_size"], 32)}
+    refs = {r: plain.forward(cfg, w, t).float() for r, t in reqs.items()}
+    for what, got in (("whole", schedules.whole(short, reqs)), ("tail", schedules.tail(short, reqs, 20)),
+                      ("batched", schedules.batched(short, reqs, {"x": 100, "y": 7}, [("x", "y")]))):
+        for r, ref in refs.items():
+            assert float((got[r] - ref).abs().max()) < 0.01 * float(ref.abs().max()), (what, r)
+    short.cache.check()
