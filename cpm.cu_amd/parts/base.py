@@ -76,7 +76,7 @@ class Workspace:
                 self.generation += 1
             buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=self.device)
             self._buf[name] = buf
-            if self.sealed:
+            if self.sealed and name not in self.grown:
                 self.grown.append(name)
         return buf[:nbytes].view(dtype).view(*shape)
 
