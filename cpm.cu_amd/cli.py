@@ -115,11 +115,30 @@ def make_prompts(args, tokenizer, vocab_size: int) -> List[List[int]]:
     return [tokenizer.encode(prompt)]
 
 
+def resolve_model_flags(args, arch) -> dict:
+    """The flags of the architecture that config.json names, as the command line gave them: the options the
+    architecture declares, then what the --model-type name sets where no option said otherwise ('minicpm4' turns
+    block-sparse attention on, cpmcu/common/utils.py:123).  A model type or an option that belongs to another
+    architecture is refused by name."""
+    from .registry import declared_flags
+    flags = {f.name: getattr(args, f.name, None) for f in arch.flags}
+    if args.model_type != "auto":
+        if args.model_type not in arch.model_types:
+            raise ValueError(f"--model-type {args.model_type}: architecture '{arch.name}' knows "
+                             f"{sorted(arch.model_types) or 'no model types'} (and 'auto')")
+        for k, v in arch.model_types[args.model_type].items():
+            if flags.get(k) is None:
+                flags[k] = v
+    foreign = [f.name for f in declared_flags() if f.name not in flags and getattr(args, f.name, None) is not None]
+    if foreign:
+        raise ValueError(f"architecture '{arch.name}' has no flags {foreign}")
+    return flags
+
+
 def run_generation(args):
     from . import get_architecture
     from .config.base import architecture_name, read_config_json
     from .llm import LLM
-    from .registry import declared_flags
     from .utils.display import Display
 
     display = Display(plain=args.plain_output)
@@ -140,19 +159,8 @@ def run_generation(args):
     if not os.path.isdir(model_path):
         raise FileNotFoundError(f"model folder not found: {model_path} (there is no download: give a local folder)")
 
-    # the architecture that config.json names declares its flags and what a --model-type name sets
     arch = get_architecture(architecture_name(read_config_json(model_path)))
-    flags = {f.name: getattr(args, f.name, None) for f in arch.flags}
-    if args.model_type != "auto":
-        if args.model_type not in arch.model_types:
-            raise ValueError(f"--model-type {args.model_type}: architecture '{arch.name}' knows "
-                             f"{sorted(arch.model_types) or 'no model types'} (and 'auto')")
-        for k, v in arch.model_types[args.model_type].items():
-            if flags.get(k) is None:
-                flags[k] = v
-    foreign = [f.name for f in declared_flags() if f.name not in flags and getattr(args, f.name, None) is not None]
-    if foreign:
-        raise ValueError(f"architecture '{arch.name}' has no flags {foreign}")
+    flags = resolve_model_flags(args, arch)
     sections = list(SUMMARY_SECTIONS)
     if arch.flags:
         sections.append((arch.name, tuple((f.name, f.name.replace("_", " ").title()) for f in arch.flags)))

@@ -301,3 +301,33 @@ def test_the_package_description_names_every_subpackage_and_the_kernel_sources()
     for target in meta["project"]["scripts"].values():
         module, func = target.split(":")
         assert callable(getattr(importlib.import_module(module), func))
+
+
+def test_the_command_lines_model_type_and_flags_resolve_through_the_architecture(model_dirs):
+    """--model-type names set what their architecture says unless an option says otherwise; names and options of
+    another architecture are refused (cpmcu/common/utils.py:123: 'minicpm4' means block-sparse attention)."""
+    from cpmcu_amd.args import parse_cli_args
+    from cpmcu_amd.cli import resolve_model_flags
+    from cpmcu_amd.llm import LLM
+    arch = get_architecture("MiniCPMForCausalLM")
+    flags = resolve_model_flags(parse_cli_args(["--model-type", "minicpm4", "--sparse-topk-k", "2"]), arch)
+    assert flags["apply_sparse"] is True and flags["sparse_topk_k"] == 2 and flags["sink_window_size"] is None
+    assert LLM(model_dirs["B"], **flags).config.sparse_config.topk == 2
+    with pytest.raises(ValueError, match="no sparse_config"):
+        LLM(model_dirs["A"], **flags)                            # 'minicpm4' on a model that describes no sparse attention
+    flags = resolve_model_flags(parse_cli_args(["--model-type", "minicpm"]), arch)
+    assert flags["apply_sparse"] is False
+    llm = LLM(model_dirs["B"], **flags)
+    assert llm.model_options == {"sparse": False}
+    assert type(arch.build_model(llm.config, llm.model_options).layers[0].mixer).__name__ == "GQAAttention"
+    # an explicit option wins over the model type's setting
+    flags = resolve_model_flags(parse_cli_args(["--model-type", "minicpm", "--apply-sparse", "true"]), arch)
+    assert flags["apply_sparse"] is True
+    # an architecture without model types refuses a name, and options that are not its own
+    from cpmcu_amd.registry import Architecture
+    bare = Architecture("BareForTests", MiniCPMConfig, build=lambda cfg: None)
+    with pytest.raises(ValueError, match="knows no model types"):
+        resolve_model_flags(parse_cli_args(["--model-type", "minicpm4"]), bare)
+    with pytest.raises(ValueError, match="has no flags \\['sparse_topk_k'\\]"):
+        resolve_model_flags(parse_cli_args(["--sparse-topk-k", "2"]), bare)
+    assert resolve_model_flags(parse_cli_args([]), bare) == {}
